@@ -1,0 +1,353 @@
+// Flash-attention forward: O = softmax(scale * Q K^T [+ causal mask]) V, [Z,H,S,D] contiguous.
+//
+// Matrix-core kernel (fp16 / bf16, D = 64 or 128): a workgroup of 4 waves owns 128 query rows (32 per wave) and
+// walks the keys in blocks of 64. K and V blocks are copied global -> LDS with global_load_lds_dwordx4, double
+// buffered. Per key block and wave:
+//   S^T = K Q^T  with v_mfma_f32_32x32x16 (K fragment first): a lane then holds 32 scores of ONE query row
+//                (row = lane%32), so row max / row sum are in-lane reductions plus one exchange with lane^32;
+//   online softmax in fp32 with exp2 and scale*log2(e) folded in (running max m, running sum l);
+//   O^T += V^T P^T: the probabilities go straight from the score registers to the MFMA operand (the k-slot to
+//                key assignment of an MFMA is free, so it is chosen to match the score register layout) and the
+//                V fragment comes from LDS through the transposing read ds_read_b64_tr_b16.
+// Causal: key blocks past the diagonal are skipped, the diagonal blocks are masked element-wise, and workgroups
+// are numbered so the longest (last) query blocks start first.
+//
+// fp32 inputs take a plain one-wave-per-query-row kernel (no fp32 matrix-core path is needed by any caller).
+#include "hexmi_common.h"
+
+namespace hexmi {
+namespace {
+
+#define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+
+constexpr int kBlockM = 128;   // query rows per workgroup
+constexpr int kBlockN = 64;    // keys per step
+
+template <typename T> struct MfmaT;
+template <> struct MfmaT<f16> {
+  typedef f16x8 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ Frag pack(const float* p) {
+    return Frag{(f16)p[0], (f16)p[1], (f16)p[2], (f16)p[3], (f16)p[4], (f16)p[5], (f16)p[6], (f16)p[7]};
+  }
+};
+template <> struct MfmaT<bf16> {
+  typedef bf16x8 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ Frag pack(const float* p) {
+    return Frag{(bf16)p[0], (bf16)p[1], (bf16)p[2], (bf16)p[3], (bf16)p[4], (bf16)p[5], (bf16)p[6], (bf16)p[7]};
+  }
+};
+
+// LDS tile [64 keys][D], 16-byte chunks, XOR swizzled per row. K is read with ds_read_b128 by 32 rows at one
+// chunk position; V with transposing 8-byte reads that touch 8 rows x 64 bytes.
+template <int D> __device__ __forceinline__ int swz_ktile(int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); }
+template <int D> __device__ __forceinline__ int swz_vtile(int row) {
+  return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
+}
+
+template <typename T, int D, bool IS_V>
+__device__ __forceinline__ void copy_kv_tile(const T* __restrict__ g, int key0, int key_max, T* lds, int wave,
+                                             int lane) {
+  constexpr int CPR = D / 8;                       // chunks per row
+  constexpr int INSTS = kBlockN * CPR / 64;        // wave-wide copies per tile
+#pragma unroll
+  for (int j = 0; j < INSTS / 4; ++j) {
+    const int inst = j * 4 + wave;
+    const int lin = inst * 64 + lane;
+    const int row = lin / CPR;
+    const int c = (lin % CPR) ^ (IS_V ? swz_vtile<D>(row) : swz_ktile<D>(row));
+    int key = key0 + row;
+    key = key < key_max ? key : key_max;
+    __builtin_amdgcn_global_load_lds(HEXMI_GLB(g + (int64_t)key * D + c * 8), HEXMI_LDS(lds + inst * 64 * 8), 16, 0, 0);
+  }
+}
+
+template <typename OutT>
+__device__ __forceinline__ void store4o(OutT* p, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void store4o<float>(float* p, float a, float b, float c, float d) {
+  *reinterpret_cast<f32x4*>(p) = f32x4{a, b, c, d};
+}
+template <> __device__ __forceinline__ void store4o<f16>(f16* p, float a, float b, float c, float d) {
+  *reinterpret_cast<f16x4*>(p) = f16x4{(f16)a, (f16)b, (f16)c, (f16)d};
+}
+template <> __device__ __forceinline__ void store4o<bf16>(bf16* p, float a, float b, float c, float d) {
+  *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)a, (bf16)b, (bf16)c, (bf16)d};
+}
+
+template <typename T, typename OutT, int D, bool CAUSAL>
+__global__ __launch_bounds__(256)
+void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+                      OutT* __restrict__ O, int ZH, int S, float scale_log2e) {
+  typedef typename MfmaT<T>::Frag Frag;
+  constexpr int DS = D / 16;                        // 16-wide steps over the head dimension
+  constexpr int DT = D / 32;                        // 32-wide output tiles over the head dimension
+  constexpr int CPR = D / 8;
+  __shared__ __attribute__((aligned(16))) T k_lds0[kBlockN * D];
+  __shared__ __attribute__((aligned(16))) T k_lds1[kBlockN * D];
+  __shared__ __attribute__((aligned(16))) T v_lds0[kBlockN * D];
+  __shared__ __attribute__((aligned(16))) T v_lds1[kBlockN * D];
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int nqb = (S + kBlockM - 1) / kBlockM;
+  const int zh = blockIdx.x % ZH;
+  const int qb = nqb - 1 - blockIdx.x / ZH;          // longest rows first
+  const int64_t base = (int64_t)zh * S * D;
+  const T* q_g = Q + base;
+  const T* k_g = K + base;
+  const T* v_g = V + base;
+
+  const int q0 = qb * kBlockM + wave * 32;           // first query row of this wave
+  const int qrow = q0 + lane % 32;                    // the query row this lane's scores belong to
+  const int half = lane / 32;
+
+  // Q fragments stay in registers: lane = (row lane%32, d = ds*16 + half*8 .. +8)
+  Frag qf[DS];
+  {
+    const int qr = qrow < S ? qrow : S - 1;
+#pragma unroll
+    for (int ds = 0; ds < DS; ++ds)
+      qf[ds] = *reinterpret_cast<const Frag*>(q_g + (int64_t)qr * D + ds * 16 + half * 8);
+  }
+
+  f32x16 o_acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.0f;
+  float m_i = -INFINITY;                              // running max (already multiplied by scale*log2e)
+  float l_i = 0.0f;                                   // this lane's share of the running sum
+
+  const int key_end = CAUSAL ? ((qb + 1) * kBlockM < S ? (qb + 1) * kBlockM : S) : S;
+  const int n_steps = (key_end + kBlockN - 1) / kBlockN;
+
+  auto load_kv = [&](int step, T* k_dst, T* v_dst) {
+    copy_kv_tile<T, D, false>(k_g, step * kBlockN, S - 1, k_dst, wave, lane);
+    copy_kv_tile<T, D, true>(v_g, step * kBlockN, S - 1, v_dst, wave, lane);
+  };
+
+  auto process = [&](int step, const T* k_src, const T* v_src) {
+    const int n0 = step * kBlockN;
+    // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4]
+    f32x16 s[2];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[jt][r] = 0.0f;
+      const int krow = jt * 32 + lane % 32;
+#pragma unroll
+      for (int ds = 0; ds < DS; ++ds) {
+        const int c = (ds * 2 + half) ^ swz_ktile<D>(krow);
+        Frag kf = *reinterpret_cast<const Frag*>(k_src + (krow * CPR + c) * 8);
+        s[jt] = MfmaT<T>::run(kf, qf[ds], s[jt]);
+      }
+    }
+    // ---- mask (diagonal and ragged blocks only)
+    const bool need_mask = (CAUSAL && n0 + kBlockN - 1 > q0) || (n0 + kBlockN > S);
+    if (need_mask) {
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = n0 + jt * 32 + 8 * (r / 4) + 4 * half + r % 4;
+          if ((CAUSAL && key > qrow) || key >= S) s[jt][r] = -INFINITY;
+        }
+    }
+    // ---- online softmax
+    float mx = -INFINITY;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[jt][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m_i, mx * scale_log2e);
+    const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+    float p[2][16];
+    float sum = 0.0f;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        p[jt][r] = __builtin_amdgcn_exp2f(fmaf(s[jt][r], scale_log2e, -m_new));
+        sum += p[jt][r];
+      }
+    l_i = l_i * alpha + sum;
+    m_i = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+    // ---- O^T += V^T P^T. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
+    //      which is score register hf*8 + e of this lane.
+    const int g = lane / 16, i16 = lane % 16;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        Frag pf = MfmaT<T>::pack(&p[jt][hf * 8]);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          union { i16x4 h[2]; Frag f; } vf;
+#pragma unroll
+          for (int pp = 0; pp < 2; ++pp) {
+            const int row = jt * 32 + hf * 16 + 8 * pp + 4 * (g >> 1) + (i16 >> 2);
+            const int col = dt * 32 + (g & 1) * 16 + (i16 & 3) * 4;
+            const int c = (col / 8) ^ swz_vtile<D>(row);
+            const T* addr = v_src + (row * CPR + c) * 8 + (col % 8);
+            vf.h[pp] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
+          }
+          o_acc[dt] = MfmaT<T>::run(vf.f, pf, o_acc[dt]);
+        }
+      }
+  };
+
+  load_kv(0, k_lds0, v_lds0);
+  int step = 0;
+  for (; step + 1 < n_steps; step += 2) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    load_kv(step + 1, k_lds1, v_lds1);
+    process(step, k_lds0, v_lds0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (step + 2 < n_steps) load_kv(step + 2, k_lds0, v_lds0);
+    process(step + 1, k_lds1, v_lds1);
+  }
+  if (step < n_steps) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    process(step, k_lds0, v_lds0);
+  }
+
+  // ---- epilogue: o_acc[dt][r] is O[qrow][dt*32 + 8*(r/4) + 4*half + r%4] * l
+  const float l_tot = l_i + __shfl_xor(l_i, 32, kWave);
+  const float inv_l = 1.0f / l_tot;
+  if (qrow < S) {
+    OutT* o_row = O + base + (int64_t)qrow * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d = dt * 32 + 8 * q4 + 4 * half;
+        store4o<OutT>(o_row + d, o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l,
+                      o_acc[dt][q4 * 4 + 2] * inv_l, o_acc[dt][q4 * 4 + 3] * inv_l);
+      }
+  }
+}
+
+// fp32 (or any dtype / head size <= 256): one wave per query row; lanes take keys lane, lane+64, ...; each lane
+// keeps its own (m, l, o[D]) and the 64 partial states are merged at the end.
+template <typename T, typename OutT, int DMAX>
+__global__ __launch_bounds__(256)
+void flash_fwd_rowwise(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+                       OutT* __restrict__ O, int64_t rows_total, int S, int D, float scale_log2e, int causal) {
+  __shared__ float q_s[4][DMAX];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;      // over ZH*S
+  if (row >= rows_total) return;
+  const int64_t zh = row / S;
+  const int qi = (int)(row % S);
+  const T* q = Q + row * D;
+  const T* k = K + zh * S * D;
+  const T* v = V + zh * S * D;
+  for (int d = lane; d < D; d += kWave) q_s[wave][d] = to_f32<T>(q[d]);
+  __builtin_amdgcn_wave_barrier();
+  float o[DMAX];
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) o[d] = 0.0f;
+  float m = -INFINITY, l = 0.0f;
+  const int kend = causal ? qi + 1 : S;
+  for (int j = lane; j < kend; j += kWave) {
+    const T* kj = k + (int64_t)j * D;
+    float sdot = 0.0f;
+    for (int d = 0; d < D; ++d) sdot = fmaf(q_s[wave][d], to_f32<T>(kj[d]), sdot);
+    const float sv = sdot * scale_log2e;
+    const float m_new = fmaxf(m, sv);
+    const float alpha = exp2f(m - m_new);
+    const float p = exp2f(sv - m_new);
+    l = l * alpha + p;
+    const T* vj = v + (int64_t)j * D;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d)
+      if (d < D) o[d] = o[d] * alpha + p * to_f32<T>(vj[d]);
+    m = m_new;
+  }
+  const float m_all = wave_max(m);
+  const float w = (m == -INFINITY) ? 0.0f : exp2f(m - m_all);
+  const float l_all = wave_sum(l * w);
+  const float inv = 1.0f / l_all;
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) {
+    if (d < D) {
+      const float od = wave_sum(o[d] * w);
+      if (lane == 0) O[row * D + d] = from_f32<OutT>(od * inv);
+    }
+  }
+}
+
+template <typename T, typename OutT, int D>
+int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
+                bool causal, hipStream_t st) {
+  const int64_t nqb = (S + kBlockM - 1) / kBlockM;
+  const int64_t blocks = nqb * ZH;
+  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  if (causal)
+    hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, true>), dim3((unsigned)blocks), dim3(256), 0, st,
+                       static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                       static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e);
+  else
+    hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, false>), dim3((unsigned)blocks), dim3(256), 0, st,
+                       static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                       static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e);
+  return launch_status();
+}
+
+template <typename T, typename OutT>
+int launch_rowwise(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, int64_t D,
+                   float scale_log2e, bool causal, hipStream_t st) {
+  const int64_t rows = ZH * S;
+  const int64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffff || D > 128) return HEXMI_ENOTSUP;
+  hipLaunchKernelGGL((flash_fwd_rowwise<T, OutT, 128>), dim3((unsigned)blocks), dim3(256), 0, st,
+                     static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                     static_cast<OutT*>(O), rows, (int)S, (int)D, scale_log2e, causal ? 1 : 0);
+  return launch_status();
+}
+
+template <typename T, typename OutT>
+int dispatch_half(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, int64_t D,
+                  float scale_log2e, bool causal, hipStream_t st) {
+  const bool ok = aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16);
+  if (ok && D == 128) return launch_mfma<T, OutT, 128>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
+  if (ok && D == 64) return launch_mfma<T, OutT, 64>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
+  return launch_rowwise<T, OutT>(Q, K, V, O, ZH, S, D, scale_log2e, causal, st);
+}
+
+}  // namespace
+}  // namespace hexmi
+
+using namespace hexmi;
+
+extern "C" int hexmi_flash_attn_fwd(const void* Q, const void* K, const void* V, void* O, int64_t Z, int64_t H,
+                                    int64_t S, int64_t D, float sm_scale, int causal, int in_dtype, int out_dtype,
+                                    hexmi_stream_t stream) {
+  if (Z < 0 || H < 0 || S < 0 || D < 0) return HEXMI_EINVAL;
+  if (Z == 0 || H == 0 || S == 0 || D == 0) return HEXMI_OK;
+  if (!Q || !K || !V || !O) return HEXMI_EINVAL;
+  if (S > 0x7fffffff / 2 || Z * H > 0x7fffffff) return HEXMI_ENOTSUP;
+  const float c = sm_scale * 1.44269504088896340736f;
+  hipStream_t st = as_stream(stream);
+  const bool cz = causal != 0;
+  const int64_t ZH = Z * H;
+  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F16) return dispatch_half<f16, f16>(Q, K, V, O, ZH, S, D, c, cz, st);
+  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F32) return dispatch_half<f16, float>(Q, K, V, O, ZH, S, D, c, cz, st);
+  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_BF16) return dispatch_half<bf16, bf16>(Q, K, V, O, ZH, S, D, c, cz, st);
+  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_F32) return dispatch_half<bf16, float>(Q, K, V, O, ZH, S, D, c, cz, st);
+  if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) return launch_rowwise<float, float>(Q, K, V, O, ZH, S, D, c, cz, st);
+  return HEXMI_ENOTSUP;
+}

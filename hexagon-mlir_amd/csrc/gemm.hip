@@ -1,0 +1,324 @@
+// Dense GEMM C[M,N] = A[M,K] * op(B) on gfx950 matrix cores (fp16 / bf16 in, fp32 accumulate).
+//
+// Workgroup = 256 threads = 4 waves in a 2x2 arrangement; each wave owns a (WM*32) x (WN*32) block of C as
+// WM x WN accumulators of v_mfma_f32_32x32x16. The K loop walks 64-wide slabs. A slab of A (and of B) is copied
+// global -> LDS by global_load_lds_dwordx4 (no register staging), double buffered: the copy of slab k+1 is in
+// flight while slab k is multiplied. The two buffers of each operand are separate LDS objects so that the
+// compiler's wait-count tracking keeps reads of one buffer independent of copies into the other.
+//
+// LDS layouts (16-byte chunks, XOR swizzled through the *source* address each lane fetches, since the LDS side
+// of a global_load_lds is fixed at base + lane*16):
+//   K-contiguous operand (A, and B given as [N,K]): [row][8 chunks]; chunk c of row r sits at c ^ ((r>>1)&7).
+//     A fragment is one ds_read_b128 per lane (row = lane%32, 8 consecutive k).
+//   N-contiguous operand (B given as [K,N]): [k][BN/8 chunks]; chunk c of row k sits at c ^ ((k&3)<<2).
+//     A fragment is two ds_read_b64_tr_b16: the transposing LDS read hands each lane 4 consecutive k of one column.
+//
+// The MFMA is issued with the B fragment as its first operand, so a lane's 4 consecutive accumulator registers
+// are 4 consecutive columns of one C row and go out as one 8-byte (fp16/bf16) or 16-byte (fp32) store.
+#include "hexmi_common.h"
+
+namespace hexmi {
+namespace {
+
+#define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+
+constexpr int BK = 64;                 // K extent of a slab (elements)
+constexpr int kChunk = 8;              // elements per 16-byte chunk
+
+template <typename T> struct Mfma;
+template <> struct Mfma<f16> {
+  typedef f16x8 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma<bf16> {
+  typedef bf16x8 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ int swz_k(int row) { return (row >> 1) & 7; }      // K-contiguous tiles
+__device__ __forceinline__ int swz_n(int k) { return (k & 3) << 2; }          // N-contiguous tiles
+
+// Copy a [ROWS x 64] K-contiguous slab (rows clamped to row_max) into LDS. ROWS/32 instructions per wave.
+template <typename T, int ROWS>
+__device__ __forceinline__ void copy_kmajor(const T* __restrict__ g, int64_t ld, int row0, int row_max, int k0,
+                                            T* lds, int wave, int lane) {
+#pragma unroll
+  for (int j = 0; j < ROWS / 32; ++j) {
+    const int inst = j * 4 + wave;                  // 8 rows per instruction
+    const int row = inst * 8 + lane / 8;
+    const int c = (lane % 8) ^ swz_k(row);
+    int grow = row0 + row;
+    grow = grow < row_max ? grow : row_max;
+    __builtin_amdgcn_global_load_lds(HEXMI_GLB(g + (int64_t)grow * ld + k0 + c * kChunk),
+                                     HEXMI_LDS(lds + inst * 8 * BK), 16, 0, 0);
+  }
+}
+
+// Copy a [64 x COLS] N-contiguous slab (column chunks clamped to col_max) into LDS. COLS/32 instructions per wave.
+template <typename T, int COLS>
+__device__ __forceinline__ void copy_nmajor(const T* __restrict__ g, int64_t ld, int k0, int col0, int col_max,
+                                            T* lds, int wave, int lane) {
+  constexpr int CPR = COLS / kChunk;                // chunks per row
+#pragma unroll
+  for (int j = 0; j < COLS / 32; ++j) {
+    const int inst = j * 4 + wave;
+    const int lin = inst * 64 + lane;
+    const int k = lin / CPR;
+    const int c = (lin % CPR) ^ swz_n(k);
+    int gcol = col0 + c * kChunk;
+    gcol = gcol < col_max ? gcol : col_max;
+    __builtin_amdgcn_global_load_lds(HEXMI_GLB(g + (int64_t)(k0 + k) * ld + gcol), HEXMI_LDS(lds + inst * 64 * kChunk),
+                                     16, 0, 0);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::Frag read_kmajor(const T* lds, int row, int chunk) {
+  typedef typename Mfma<T>::Frag Frag;
+  return *reinterpret_cast<const Frag*>(lds + row * BK + ((chunk ^ swz_k(row)) * kChunk));
+}
+
+template <typename T, int COLS>
+__device__ __forceinline__ typename Mfma<T>::Frag read_nmajor(const T* lds, int col_tile, int ks, int lane) {
+  typedef typename Mfma<T>::Frag Frag;
+  constexpr int CPR = COLS / kChunk;
+  const int g = lane / 16, i = lane % 16;
+  const int n = col_tile + (g & 1) * 16 + (i & 3) * 4;    // 4 consecutive columns fetched by this lane
+  const int kb = ks * 16 + (g >> 1) * 8 + (i >> 2);
+  union { i16x4 h[2]; Frag f; } u;
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int k = kb + p * 4;
+    const int c = (n / kChunk) ^ swz_n(k);
+    const T* addr = lds + (k * CPR + c) * kChunk + (n % kChunk);
+    u.h[p] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
+  }
+  return u.f;
+}
+
+template <typename OutT>
+__device__ __forceinline__ void store4(OutT* p, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
+  f32x4 v = {a, b, c, d};
+  *reinterpret_cast<f32x4*>(p) = v;
+}
+template <> __device__ __forceinline__ void store4<f16>(f16* p, float a, float b, float c, float d) {
+  f16x4 v = {(f16)a, (f16)b, (f16)c, (f16)d};
+  *reinterpret_cast<f16x4*>(p) = v;
+}
+template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float a, float b, float c, float d) {
+  bf16x4 v = {(bf16)a, (bf16)b, (bf16)c, (bf16)d};
+  *reinterpret_cast<bf16x4*>(p) = v;
+}
+
+// Map the linear workgroup id to a C tile: consecutive ids go to different XCDs (each with its own L2), so
+// first give every XCD a contiguous run of logical ids, then walk tiles in bands of GROUP_M tile-rows so the
+// tiles resident on one XCD share A and B panels.
+__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  int logical = pid;
+  if (total % 8 == 0) logical = (pid % 8) * (total / 8) + pid / 8;
+  constexpr int GROUP_M = 4;
+  const int group_size = GROUP_M * tiles_n;
+  const int group = logical / group_size;
+  const int first_m = group * GROUP_M;
+  const int gm = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int in_group = logical % group_size;
+  tm = first_m + in_group % gm;
+  tn = in_group / gm;
+}
+
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B>
+__global__ __launch_bounds__(256)
+void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restrict__ C, int M, int N, int K,
+                 int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n) {
+  typedef typename Mfma<T>::Frag Frag;
+  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  __shared__ __attribute__((aligned(16))) T a_lds0[BM * BK];
+  __shared__ __attribute__((aligned(16))) T a_lds1[BM * BK];
+  __shared__ __attribute__((aligned(16))) T b_lds0[BN * BK];
+  __shared__ __attribute__((aligned(16))) T b_lds1[BN * BK];
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int wm = wave / 2, wn = wave % 2;
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  auto load_slab = [&](int kt, T* a_dst, T* b_dst) {
+    copy_kmajor<T, BM>(A, lda, m0, M - 1, kt * BK, a_dst, wave, lane);
+    if constexpr (TRANS_B) copy_kmajor<T, BN>(B, ldb, n0, N - 1, kt * BK, b_dst, wave, lane);
+    else copy_nmajor<T, BN>(B, ldb, kt * BK, n0, N - kChunk, b_dst, wave, lane);
+  };
+
+  auto multiply_slab = [&](const T* a_src, const T* b_src) {
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      Frag af[WM], bf[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) af[i] = read_kmajor<T>(a_src, (wm * WM + i) * 32 + lane % 32, ks * 2 + lane / 32);
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+        if constexpr (TRANS_B) bf[j] = read_kmajor<T>(b_src, (wn * WN + j) * 32 + lane % 32, ks * 2 + lane / 32);
+        else bf[j] = read_nmajor<T, BN>(b_src, (wn * WN + j) * 32, ks, lane);
+      }
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) acc[i][j] = Mfma<T>::run(bf[j], af[i], acc[i][j]);
+    }
+  };
+
+  const int KT = K / BK;
+  load_slab(0, a_lds0, b_lds0);
+  int kt = 0;
+  for (; kt + 1 < KT; kt += 2) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();                                  // slab kt landed everywhere; buffer 1 no longer read
+    load_slab(kt + 1, a_lds1, b_lds1);
+    multiply_slab(a_lds0, b_lds0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (kt + 2 < KT) load_slab(kt + 2, a_lds0, b_lds0);
+    multiply_slab(a_lds1, b_lds1);
+  }
+  if (kt < KT) {                                      // odd slab count: the last slab sits in buffer 0
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    multiply_slab(a_lds0, b_lds0);
+  }
+
+  // acc[i][j][r]: row = lane%32 of the 32x32 tile, column = 8*(r/4) + 4*(lane/32) + r%4.
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int row = m0 + (wm * WM + i) * 32 + lane % 32;
+    if (row >= M) continue;
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int col = n0 + (wn * WN + j) * 32 + 8 * q + 4 * (lane / 32);
+        if (col < N)
+          store4<OutT>(C + (int64_t)row * ldc + col, acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1],
+                       acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+      }
+    }
+  }
+}
+
+// Any shape, any alignment: 64x64 tile, scalar guarded loads through LDS, MFMA 32x32x16 with zero padding.
+template <typename T, typename OutT, bool TRANS_B>
+__global__ __launch_bounds__(256)
+void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT* __restrict__ C, int M, int N, int K,
+                         int64_t lda, int64_t ldb, int64_t ldc) {
+  typedef typename Mfma<T>::Frag Frag;
+  constexpr int TB = 64, TK = 16, PAD = 8;
+  __shared__ __attribute__((aligned(16))) T a_s[TB][TK + PAD];   // [m][k]
+  __shared__ __attribute__((aligned(16))) T b_s[TB][TK + PAD];   // [n][k]
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int m0 = blockIdx.y * TB, n0 = blockIdx.x * TB;
+  const int wm = wave / 2, wn = wave % 2;
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  for (int k0 = 0; k0 < K; k0 += TK) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < TB * TK; e += 256) {
+      const int r = e / TK, k = e % TK;
+      const int gm = m0 + r, gk = k0 + k;
+      a_s[r][k] = (gm < M && gk < K) ? A[(int64_t)gm * lda + gk] : (T)0.0f;
+      const int gn = n0 + r;
+      T bv = (T)0.0f;
+      if (gn < N && gk < K) bv = TRANS_B ? B[(int64_t)gn * ldb + gk] : B[(int64_t)gk * ldb + gn];
+      b_s[r][k] = bv;
+    }
+    __syncthreads();
+    Frag af = *reinterpret_cast<const Frag*>(&a_s[wm * 32 + lane % 32][(lane / 32) * 8]);
+    Frag bf = *reinterpret_cast<const Frag*>(&b_s[wn * 32 + lane % 32][(lane / 32) * 8]);
+    acc = Mfma<T>::run(bf, af, acc);
+  }
+  const int row = m0 + wm * 32 + lane % 32;
+  if (row >= M) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int col = n0 + wn * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+    if (col < N) C[(int64_t)row * ldc + col] = from_f32<OutT>(acc[r]);
+  }
+}
+
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B>
+int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                 int64_t ldc, hipStream_t s) {
+  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+  hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A, B, C,
+                     (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+  return launch_status();
+}
+
+template <typename T, typename OutT, bool TRANS_B>
+int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N, int64_t K, int64_t lda,
+                  int64_t ldb, int64_t ldc, hipStream_t s) {
+  const T* A = static_cast<const T*>(Av);
+  const T* B = static_cast<const T*>(Bv);
+  OutT* C = static_cast<OutT*>(Cv);
+  const bool fast = K % BK == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && N % 8 == 0 && M >= 1 &&
+                    aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(C, 16) && N >= 8;
+  if (fast) {
+    const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    if (big_tiles >= 128) return launch_tiled<T, OutT, 4, 4, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s);
+    return launch_tiled<T, OutT, 2, 2, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s);
+  }
+  dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+  if (grid.y > 65535) return HEXMI_ENOTSUP;
+  hipLaunchKernelGGL((gemm_kernel_generic<T, OutT, TRANS_B>), grid, dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K,
+                     lda, ldb, ldc);
+  return launch_status();
+}
+
+template <typename T, typename OutT>
+int dispatch_trans(bool trans_b, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                   int64_t ldb, int64_t ldc, hipStream_t s) {
+  return trans_b ? dispatch_gemm<T, OutT, true>(A, B, C, M, N, K, lda, ldb, ldc, s)
+                 : dispatch_gemm<T, OutT, false>(A, B, C, M, N, K, lda, ldb, ldc, s);
+}
+
+}  // namespace
+}  // namespace hexmi
+
+using namespace hexmi;
+
+extern "C" int hexmi_gemm(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb,
+                          void* C, int64_t ldc, int in_dtype, int out_dtype, int trans_b, hexmi_stream_t stream) {
+  if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
+  if (M == 0 || N == 0) return HEXMI_OK;
+  if (!A || !B || !C) return HEXMI_EINVAL;
+  if (lda < K || ldc < N || ldb < (trans_b ? K : N)) return HEXMI_EINVAL;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return HEXMI_ENOTSUP;
+  if (K == 0) return HEXMI_ENOTSUP;
+  hipStream_t s = as_stream(stream);
+  const bool tb = trans_b != 0;
+  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F16) return dispatch_trans<f16, f16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
+  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F32) return dispatch_trans<f16, float>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
+  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_BF16) return dispatch_trans<bf16, bf16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
+  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_F32) return dispatch_trans<bf16, float>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
+  return HEXMI_ENOTSUP;
+}
+
+extern "C" int hexmi_matmul_f16f16_f32(int64_t n_row, int64_t n_col, int64_t n_inner, float* out, const void* act,
+                                       const void* w, hexmi_stream_t stream) {
+  return hexmi_gemm(n_row, n_col, n_inner, act, n_inner, w, n_col, out, n_col, HEXMI_F16, HEXMI_F32, 0, stream);
+}

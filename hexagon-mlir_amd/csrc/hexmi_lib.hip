@@ -1,0 +1,21 @@
+// Library-level entry points: version, status text, device query.
+#include "hexmi_common.h"
+
+extern "C" const char* hexmi_version(void) { return "hexmi 0.1 gfx950"; }
+
+extern "C" const char* hexmi_strerror(int status) {
+  switch (status) {
+    case HEXMI_OK: return "ok";
+    case HEXMI_EINVAL: return "invalid argument (null pointer, negative size, bad leading dimension or alignment)";
+    case HEXMI_ENOTSUP: return "unsupported dtype or shape";
+    case HEXMI_ELAUNCH: return "HIP launch failed";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int hexmi_num_cus(void) {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  return cus;
+}

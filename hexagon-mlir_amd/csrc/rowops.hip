@@ -1,0 +1,298 @@
+// Row reductions: softmax, RMSNorm, LayerNorm. Single pass over HBM: a row is
+// loaded once with 16-byte accesses, kept in registers in fp32-convertible
+// form, reduced with wavefront butterflies (and one LDS exchange when a row
+// spans several waves), and stored once.
+//
+//   rows up to 16 KiB : one 64-lane wave per row, no LDS, no barrier
+//   rows up to 128 KiB: one 1024-thread workgroup per row, LDS reduction
+//   anything else (or misaligned): generic strided kernel, row re-read from L2
+#include "hexmi_common.h"
+
+namespace hexmi {
+namespace {
+
+template <typename T> struct Vec16 {               // one 16-byte global access
+  static constexpr int N = 16 / sizeof(T);
+  T v[N];
+};
+
+template <typename T>
+__device__ __forceinline__ Vec16<T> load16(const T* p) {
+  Vec16<T> r;
+  *reinterpret_cast<u32x4*>(r.v) = *reinterpret_cast<const u32x4*>(p);
+  return r;
+}
+template <typename T>
+__device__ __forceinline__ void store16(T* p, const Vec16<T>& r) {
+  *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(r.v);
+}
+// Streaming variants: the row is touched exactly once, so keep it out of the
+// way of resident data (weights, bias) in L2.
+template <typename T>
+__device__ __forceinline__ Vec16<T> load16_stream(const T* p) {
+  Vec16<T> r;
+  *reinterpret_cast<u32x4*>(r.v) = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return r;
+}
+template <typename T>
+__device__ __forceinline__ void store16_stream(T* p, const Vec16<T>& r) {
+  __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(r.v), reinterpret_cast<u32x4*>(p));
+}
+
+// Reduce across the waves of a workgroup through LDS. `red` holds one float
+// per wave; every thread returns the combined value.
+template <bool IS_MAX, int WAVES>
+__device__ __forceinline__ float block_reduce(float v, float* red) {
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  if constexpr (WAVES == 1) return v;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  __syncthreads();                                  // previous use of `red` finished
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float r = red[0];
+#pragma unroll
+  for (int w = 1; w < WAVES; ++w) r = IS_MAX ? fmaxf(r, red[w]) : r + red[w];
+  return r;
+}
+
+enum RowOp { kSoftmax = 0, kRmsNorm = 1, kLayerNorm = 2 };
+
+// THREADS threads cooperate on one row (THREADS == 64: a wave per row, several
+// rows per workgroup). Each thread owns CHUNKS 16-byte chunks, chunk c of
+// thread t covering elements [(c*THREADS + t)*N, +N).
+template <typename T, int OP, int CHUNKS, int THREADS, int ROWS_PER_BLOCK>
+__global__ __launch_bounds__(THREADS * ROWS_PER_BLOCK)
+void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict__ w,
+                const T* __restrict__ b, float* __restrict__ mean_out, float* __restrict__ rstd_out,
+                int64_t rows, int cols, int64_t ld_x, int64_t ld_y, float eps) {
+  constexpr int N = Vec16<T>::N;
+  constexpr int WAVES = THREADS / kWave;
+  __shared__ float red[WAVES > 1 ? WAVES : 1];
+  const int t = threadIdx.x % THREADS;
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / THREADS;
+  if (row >= rows) return;                          // whole waves leave together (THREADS % 64 == 0)
+
+  const T* xr = x + row * ld_x;
+  T* yr = y + row * ld_y;
+  float v[CHUNKS][N];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int col = (c * THREADS + t) * N;
+    if (col < cols) {
+      Vec16<T> raw = load16_stream(xr + col);
+#pragma unroll
+      for (int i = 0; i < N; ++i) v[c][i] = to_f32<T>(raw.v[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; ++i) v[c][i] = (OP == kSoftmax) ? -INFINITY : 0.0f;
+    }
+  }
+
+  if constexpr (OP == kSoftmax) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < N; ++i) m = fmaxf(m, v[c][i]);
+    m = block_reduce<true, WAVES>(m, red);
+    float s = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < N; ++i) { v[c][i] = __expf(v[c][i] - m); s += v[c][i]; }
+    s = block_reduce<false, WAVES>(s, red);
+    const float inv = 1.0f / s;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const int col = (c * THREADS + t) * N;
+      if (col < cols) {
+        Vec16<T> o;
+#pragma unroll
+        for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i] * inv);
+        store16_stream(yr + col, o);
+      }
+    }
+  } else {
+    const float inv_n = 1.0f / (float)cols;
+    float mean = 0.0f;
+    if constexpr (OP == kLayerNorm) {
+      float s = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+        for (int i = 0; i < N; ++i) s += v[c][i];
+      mean = block_reduce<false, WAVES>(s, red) * inv_n;
+    }
+    float q = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const int col = (c * THREADS + t) * N;
+      if (col < cols) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) { v[c][i] -= mean; q += v[c][i] * v[c][i]; }
+      }
+    }
+    q = block_reduce<false, WAVES>(q, red);
+    const float rstd = 1.0f / sqrtf(q * inv_n + eps);
+    if constexpr (OP == kLayerNorm) {
+      if (t == 0) {
+        if (mean_out) mean_out[row] = mean;
+        if (rstd_out) rstd_out[row] = rstd;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const int col = (c * THREADS + t) * N;
+      if (col < cols) {
+        Vec16<T> o;
+        if (w) {
+          Vec16<T> wv = load16(w + col);
+#pragma unroll
+          for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd * to_f32<T>(wv.v[i]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd;
+        }
+        if (OP == kLayerNorm && b) {
+          Vec16<T> bv = load16(b + col);
+#pragma unroll
+          for (int i = 0; i < N; ++i) v[c][i] += to_f32<T>(bv.v[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i]);
+        store16_stream(yr + col, o);
+      }
+    }
+  }
+}
+
+// Any shape / alignment: 256 threads per row, scalar accesses, the row is read
+// again for each sweep (it stays in L2 for any row this path is chosen for).
+template <typename T, int OP>
+__global__ __launch_bounds__(256)
+void row_kernel_generic(const T* __restrict__ x, T* __restrict__ y, const T* __restrict__ w,
+                        const T* __restrict__ b, float* __restrict__ mean_out, float* __restrict__ rstd_out,
+                        int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps) {
+  constexpr int WAVES = 4;
+  __shared__ float red[WAVES];
+  const int64_t row = blockIdx.x;
+  const T* xr = x + row * ld_x;
+  T* yr = y + row * ld_y;
+  const int t = threadIdx.x;
+  if constexpr (OP == kSoftmax) {
+    float m = -INFINITY;
+    for (int64_t i = t; i < cols; i += 256) m = fmaxf(m, to_f32<T>(xr[i]));
+    m = block_reduce<true, WAVES>(m, red);
+    float s = 0.0f;
+    for (int64_t i = t; i < cols; i += 256) s += __expf(to_f32<T>(xr[i]) - m);
+    s = block_reduce<false, WAVES>(s, red);
+    const float inv = 1.0f / s;
+    for (int64_t i = t; i < cols; i += 256) yr[i] = from_f32<T>(__expf(to_f32<T>(xr[i]) - m) * inv);
+  } else {
+    const float inv_n = 1.0f / (float)cols;
+    float mean = 0.0f;
+    if constexpr (OP == kLayerNorm) {
+      float s = 0.0f;
+      for (int64_t i = t; i < cols; i += 256) s += to_f32<T>(xr[i]);
+      mean = block_reduce<false, WAVES>(s, red) * inv_n;
+    }
+    float q = 0.0f;
+    for (int64_t i = t; i < cols; i += 256) { float d = to_f32<T>(xr[i]) - mean; q += d * d; }
+    q = block_reduce<false, WAVES>(q, red);
+    const float rstd = 1.0f / sqrtf(q * inv_n + eps);
+    if constexpr (OP == kLayerNorm) {
+      if (t == 0) {
+        if (mean_out) mean_out[row] = mean;
+        if (rstd_out) rstd_out[row] = rstd;
+      }
+    }
+    for (int64_t i = t; i < cols; i += 256) {
+      float o = (to_f32<T>(xr[i]) - mean) * rstd;
+      if (w) o *= to_f32<T>(w[i]);
+      if (OP == kLayerNorm && b) o += to_f32<T>(b[i]);
+      yr[i] = from_f32<T>(o);
+    }
+  }
+}
+
+template <typename T, int OP, int CHUNKS, int THREADS, int RPB>
+int launch_tile(const T* x, T* y, const T* w, const T* b, float* mean, float* rstd, int64_t rows,
+                int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s) {
+  const int64_t blocks = (rows + RPB - 1) / RPB;
+  hipLaunchKernelGGL((row_kernel<T, OP, CHUNKS, THREADS, RPB>), dim3((unsigned)blocks), dim3(THREADS * RPB), 0, s,
+                     x, y, w, b, mean, rstd, rows, (int)cols, ld_x, ld_y, eps);
+  return launch_status();
+}
+
+template <typename T, int OP>
+int dispatch_rows(const void* xv, void* yv, const void* wv, const void* bv, float* mean, float* rstd,
+                  int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s) {
+  const T* x = static_cast<const T*>(xv);
+  T* y = static_cast<T*>(yv);
+  const T* w = static_cast<const T*>(wv);
+  const T* b = static_cast<const T*>(bv);
+  constexpr int N = 16 / sizeof(T);
+  const bool vec_ok = cols % N == 0 && ld_x % N == 0 && ld_y % N == 0 && aligned_to(x, 16) && aligned_to(y, 16) &&
+                      (!w || aligned_to(w, 16)) && (!b || aligned_to(b, 16));
+  const int64_t chunks = (cols + N - 1) / N;        // 16-byte chunks per row
+#define HEXMI_TILE(C, TH, RPB) return launch_tile<T, OP, C, TH, RPB>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s)
+  if (vec_ok && rows <= 0x7fffffff) {
+    if (chunks <= 64 * 1) HEXMI_TILE(1, 64, 4);
+    if (chunks <= 64 * 2) HEXMI_TILE(2, 64, 4);
+    if (chunks <= 64 * 4) HEXMI_TILE(4, 64, 4);
+    if (chunks <= 64 * 8) HEXMI_TILE(8, 64, 4);
+    if (chunks <= 256 * 4) HEXMI_TILE(4, 256, 1);
+    if (chunks <= 256 * 8) HEXMI_TILE(8, 256, 1);
+    if (chunks <= 1024 * 4) HEXMI_TILE(4, 1024, 1);
+    if (chunks <= 1024 * 8) HEXMI_TILE(8, 1024, 1);
+  }
+#undef HEXMI_TILE
+  if (rows > 0x7fffffff) return HEXMI_ENOTSUP;
+  hipLaunchKernelGGL((row_kernel_generic<T, OP>), dim3((unsigned)rows), dim3(256), 0, s, x, y, w, b, mean, rstd, rows,
+                     cols, ld_x, ld_y, eps);
+  return launch_status();
+}
+
+template <int OP>
+int dispatch_dtype(int dtype, const void* x, void* y, const void* w, const void* b, float* mean, float* rstd,
+                   int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s) {
+  switch (dtype) {
+    case HEXMI_F32: return dispatch_rows<float, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s);
+    case HEXMI_F16: return dispatch_rows<f16, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s);
+    case HEXMI_BF16: return dispatch_rows<bf16, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s);
+    default: return HEXMI_ENOTSUP;
+  }
+}
+
+}  // namespace
+}  // namespace hexmi
+
+using namespace hexmi;
+
+extern "C" int hexmi_softmax(const void* x, void* y, int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y,
+                             int dtype, hexmi_stream_t stream) {
+  if (rows < 0 || cols < 0 || ld_x < cols || ld_y < cols) return HEXMI_EINVAL;
+  if (rows == 0 || cols == 0) return HEXMI_OK;
+  if (!x || !y) return HEXMI_EINVAL;
+  return dispatch_dtype<kSoftmax>(dtype, x, y, nullptr, nullptr, nullptr, nullptr, rows, cols, ld_x, ld_y, 0.0f,
+                                  as_stream(stream));
+}
+
+extern "C" int hexmi_rms_norm(const void* x, const void* weight, void* y, int64_t rows, int64_t cols, float eps,
+                              int dtype, hexmi_stream_t stream) {
+  if (rows < 0 || cols < 0) return HEXMI_EINVAL;
+  if (rows == 0 || cols == 0) return HEXMI_OK;
+  if (!x || !y) return HEXMI_EINVAL;
+  return dispatch_dtype<kRmsNorm>(dtype, x, y, weight, nullptr, nullptr, nullptr, rows, cols, cols, cols, eps,
+                                  as_stream(stream));
+}
+
+extern "C" int hexmi_layer_norm(const void* x, const void* weight, const void* bias, void* y, float* mean,
+                                float* rstd, int64_t rows, int64_t cols, float eps, int dtype,
+                                hexmi_stream_t stream) {
+  if (rows < 0 || cols < 0) return HEXMI_EINVAL;
+  if (rows == 0 || cols == 0) return HEXMI_OK;
+  if (!x || !y) return HEXMI_EINVAL;
+  return dispatch_dtype<kLayerNorm>(dtype, x, y, weight, bias, mean, rstd, rows, cols, cols, cols, eps,
+                                    as_stream(stream));
+}

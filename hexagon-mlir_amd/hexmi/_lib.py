@@ -1,0 +1,66 @@
+"""ctypes loader for libhexmi.so (the C ABI declared in include/hexmi.h).
+
+There is no fallback: if the library has not been built the import of any
+operator raises, and every non-zero status from the library raises
+HexmiError.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhexmi.so")
+
+OK, EINVAL, ENOTSUP, ELAUNCH = 0, -1, -2, -3
+F32, F16, BF16, I8 = 0, 1, 2, 3
+
+
+class HexmiError(RuntimeError):
+    def __init__(self, status, what):
+        self.status = status
+        super().__init__("%s failed with status %d: %s" % (what, status, strerror(status)))
+
+
+_c = ctypes
+_i64, _int, _f32, _ptr = _c.c_int64, _c.c_int, _c.c_float, _c.c_void_p
+
+# name -> (restype, argtypes); must list every symbol of include/hexmi.h
+SIGNATURES = {
+    "hexmi_version": (_c.c_char_p, []),
+    "hexmi_strerror": (_c.c_char_p, [_int]),
+    "hexmi_num_cus": (_int, []),
+    "hexmi_softmax": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _int, _ptr]),
+    "hexmi_rms_norm": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _f32, _int, _ptr]),
+    "hexmi_layer_norm": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _f32, _int, _ptr]),
+    "hexmi_matmul_f16f16_f32": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "hexmi_gemm": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _int, _int, _ptr]),
+    "hexmi_gemm_w8a16": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "hexmi_dequant_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "hexmi_flash_attn_fwd": (_int, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _ptr]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it was never built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libhexmi.so is missing at %s: build it with `python hexagon-mlir_amd/build.py` "
+                "(there is no CPU or eager fallback)" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)          # AttributeError if the symbol is not exported
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def strerror(status):
+    return lib().hexmi_strerror(int(status)).decode()
+
+
+def check(status, what):
+    if status != OK:
+        raise HexmiError(status, what)

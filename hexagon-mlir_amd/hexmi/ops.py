@@ -1,0 +1,260 @@
+"""Tensor-in / tensor-out operators over libhexmi.so.
+
+Every operator is registered as a PyTorch custom op (`torch.ops.hexmi.*`,
+CUDA/HIP dispatch key only) whose implementation hands device pointers and the
+current HIP stream to the C ABI. The public functions below add what the
+reference's launcher does around a kernel: host tensors are accepted, staged
+to the GPU, and results are written back into the caller's `out` tensor in
+place (qcom_hexagon_backend/backend/triton_hexagon_launcher.py:716-728 copies
+device results back into the tensors the user passed).
+
+There is no CPU implementation: without a GPU or without libhexmi.so these
+functions raise.
+"""
+import math
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.int8: _lib.I8}
+
+
+def _dt(t):
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError("hexmi: unsupported dtype %s" % t.dtype) from None
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+# --------------------------------------------------------------------------
+# custom-op registration (schema: inputs..., Tensor(a!) out) -> ()
+# --------------------------------------------------------------------------
+_LIBDEF = torch.library.Library("hexmi", "DEF")
+_LIBDEF.define("softmax(Tensor x, Tensor(a!) out) -> ()")
+_LIBDEF.define("rms_norm(Tensor x, Tensor? weight, float eps, Tensor(a!) out) -> ()")
+_LIBDEF.define("layer_norm(Tensor x, Tensor? weight, Tensor? bias, float eps, Tensor(a!) out, "
+               "Tensor(b!)? mean, Tensor(c!)? rstd) -> ()")
+_LIBDEF.define("matmul(Tensor a, Tensor b, bool trans_b, Tensor(a!) out) -> ()")
+_LIBDEF.define("w8a16_matmul(Tensor a, Tensor w, Tensor scales, Tensor(a!) out) -> ()")
+_LIBDEF.define("dequant_w8(Tensor w, Tensor scales, Tensor(a!) out) -> ()")
+_LIBDEF.define("flash_attention(Tensor q, Tensor k, Tensor v, float sm_scale, bool causal, Tensor(a!) out) -> ()")
+
+
+def _softmax_impl(x, out):
+    rows, cols = x.shape
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().hexmi_softmax(_p(x), _p(out), rows, cols, x.stride(0), out.stride(0), _dt(x),
+                                            _stream()), "hexmi_softmax")
+
+
+def _rms_norm_impl(x, weight, eps, out):
+    rows, cols = x.shape
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().hexmi_rms_norm(_p(x), _p(weight), _p(out), rows, cols, eps, _dt(x), _stream()),
+                   "hexmi_rms_norm")
+
+
+def _layer_norm_impl(x, weight, bias, eps, out, mean, rstd):
+    rows, cols = x.shape
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().hexmi_layer_norm(_p(x), _p(weight), _p(bias), _p(out), _p(mean), _p(rstd), rows, cols,
+                                               eps, _dt(x), _stream()), "hexmi_layer_norm")
+
+
+def _matmul_impl(a, b, trans_b, out):
+    M, K = a.shape
+    N = b.shape[0] if trans_b else b.shape[1]
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().hexmi_gemm(M, N, K, _p(a), a.stride(0), _p(b), b.stride(0), _p(out), out.stride(0),
+                                         _dt(a), _dt(out), 1 if trans_b else 0, _stream()), "hexmi_gemm")
+
+
+def _w8a16_impl(a, w, scales, out):
+    M, K = a.shape
+    N = w.shape[0]
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().hexmi_gemm_w8a16(M, N, K, _p(a), _p(w), _p(scales), _p(out), _stream()),
+                   "hexmi_gemm_w8a16")
+
+
+def _dequant_impl(w, scales, out):
+    N, K = w.shape
+    with torch.cuda.device(w.device):
+        _lib.check(_lib.lib().hexmi_dequant_w8(N, K, _p(w), _p(scales), _p(out), _stream()), "hexmi_dequant_w8")
+
+
+def _flash_impl(q, k, v, sm_scale, causal, out):
+    Z, H, S, D = q.shape
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().hexmi_flash_attn_fwd(_p(q), _p(k), _p(v), _p(out), Z, H, S, D, sm_scale,
+                                                   1 if causal else 0, _dt(q), _dt(out), _stream()),
+                   "hexmi_flash_attn_fwd")
+
+
+for _name, _fn in (("softmax", _softmax_impl), ("rms_norm", _rms_norm_impl), ("layer_norm", _layer_norm_impl),
+                   ("matmul", _matmul_impl), ("w8a16_matmul", _w8a16_impl), ("dequant_w8", _dequant_impl),
+                   ("flash_attention", _flash_impl)):
+    _LIBDEF.impl(_name, _fn, "CUDA")
+
+
+# --------------------------------------------------------------------------
+# staging helpers
+# --------------------------------------------------------------------------
+def _device():
+    if not torch.cuda.is_available():
+        raise RuntimeError("hexmi needs a GPU (gfx950); there is no CPU path")
+    _lib.lib()
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _stage(t, dev):
+    """Contiguous device copy (or the tensor itself when it already is one)."""
+    if t is None:
+        return None
+    if t.device.type != "cuda":
+        t = t.to(dev, non_blocking=False)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _finish(result, out):
+    """Write `result` (device) into the caller's `out` if they are different tensors."""
+    if out is None:
+        return result
+    if out.data_ptr() != result.data_ptr() or out.device != result.device:
+        out.copy_(result)
+    return out
+
+
+def _out_like(out, shape, dtype, dev):
+    """Device tensor to compute into: `out` itself when usable, else a fresh one."""
+    if out is not None:
+        if tuple(out.shape) != tuple(shape):
+            raise ValueError("hexmi: out has shape %s, expected %s" % (tuple(out.shape), tuple(shape)))
+        if out.dtype != dtype:
+            raise TypeError("hexmi: out has dtype %s, expected %s" % (out.dtype, dtype))
+        if out.device.type == "cuda" and out.is_contiguous():
+            return out
+    return torch.empty(shape, dtype=dtype, device=dev)
+
+
+# --------------------------------------------------------------------------
+# public operators
+# --------------------------------------------------------------------------
+def softmax(x, out=None, dim=-1):
+    """Softmax over the last dimension (`F.softmax(x, dim=1)` of
+    test/python/triton/test_softmax.py:93 for 2-D input)."""
+    if dim not in (-1, x.dim() - 1):
+        raise ValueError("hexmi.softmax reduces over the last dimension only")
+    if x.dim() < 1:
+        raise ValueError("hexmi.softmax needs at least 1 dimension")
+    dev = _device() if x.device.type != "cuda" else x.device
+    xd = _stage(x, dev)
+    od = _out_like(out, x.shape, x.dtype, dev)
+    cols = x.shape[-1]
+    torch.ops.hexmi.softmax(xd.view(-1, cols), od.view(-1, cols))
+    return _finish(od, out)
+
+
+def rms_norm(x, weight=None, eps=1e-5, out=None):
+    """`F.rms_norm(x, (C,), weight, eps)` (test/python/triton/test_rms_norm.py:85-87)."""
+    dev = _device() if x.device.type != "cuda" else x.device
+    cols = x.shape[-1]
+    if weight is not None and (weight.shape != (cols,) or weight.dtype != x.dtype):
+        raise ValueError("hexmi.rms_norm: weight must be [%d] of %s" % (cols, x.dtype))
+    xd, wd = _stage(x, dev), _stage(weight, dev)
+    od = _out_like(out, x.shape, x.dtype, dev)
+    torch.ops.hexmi.rms_norm(xd.view(-1, cols), wd, float(eps), od.view(-1, cols))
+    return _finish(od, out)
+
+
+def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=None):
+    """`F.layer_norm(x, (C,), weight, bias, eps)` (test/python/triton/test_layer_norm.py:111-113);
+    `mean` / `rstd` (fp32, one per row) are filled when given, as the reference kernel does."""
+    dev = _device() if x.device.type != "cuda" else x.device
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    for name, t in (("weight", weight), ("bias", bias)):
+        if t is not None and (t.shape != (cols,) or t.dtype != x.dtype):
+            raise ValueError("hexmi.layer_norm: %s must be [%d] of %s" % (name, cols, x.dtype))
+    xd, wd, bd = _stage(x, dev), _stage(weight, dev), _stage(bias, dev)
+    od = _out_like(out, x.shape, x.dtype, dev)
+    md = None if mean is None else _out_like(mean if mean.dtype == torch.float32 else None, (rows,), torch.float32, dev)
+    rd = None if rstd is None else _out_like(rstd if rstd.dtype == torch.float32 else None, (rows,), torch.float32, dev)
+    torch.ops.hexmi.layer_norm(xd.view(-1, cols), wd, bd, float(eps), od.view(-1, cols), md, rd)
+    if mean is not None:
+        _finish(md, mean)
+    if rstd is not None:
+        _finish(rd, rstd)
+    return _finish(od, out)
+
+
+def matmul(a, b, out=None, out_dtype=None, trans_b=False):
+    """C = A @ B (or A @ B.T when trans_b), fp16/bf16 inputs, fp32 accumulation.
+    out_dtype: the input dtype (default) or torch.float32
+    (test/python/triton/test_matmul.py:35-91; docs/tutorials/triton/matmul_hexkl.md:61-111)."""
+    if a.dim() != 2 or b.dim() != 2:
+        raise ValueError("hexmi.matmul takes 2-D tensors")
+    if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("hexmi.matmul: A and B must both be float16 or both bfloat16")
+    M, K = a.shape
+    N = b.shape[0] if trans_b else b.shape[1]
+    if (b.shape[1] if trans_b else b.shape[0]) != K:
+        raise ValueError("hexmi.matmul: inner dimensions differ: %s x %s" % (tuple(a.shape), tuple(b.shape)))
+    if out_dtype is None:
+        out_dtype = out.dtype if out is not None else a.dtype
+    dev = _device() if a.device.type != "cuda" else a.device
+    ad, bd = _stage(a, dev), _stage(b, dev)
+    od = _out_like(out, (M, N), out_dtype, dev)
+    torch.ops.hexmi.matmul(ad, bd, bool(trans_b), od)
+    return _finish(od, out)
+
+
+def w8a16_matmul(a, w_int8, scales, out=None):
+    """C[m,n] = sum_k A[m,k] * (W[n,k] * scales[n]); A fp16 [M,K], W int8 [N,K], scales fp16 [N]."""
+    if a.dtype != torch.float16 or w_int8.dtype != torch.int8 or scales.dtype != torch.float16:
+        raise TypeError("hexmi.w8a16_matmul: expected fp16 activations, int8 weights, fp16 scales")
+    if a.dim() != 2 or w_int8.dim() != 2 or a.shape[1] != w_int8.shape[1] or scales.shape != (w_int8.shape[0],):
+        raise ValueError("hexmi.w8a16_matmul: shapes A[M,K], W[N,K], scales[N] required")
+    dev = _device() if a.device.type != "cuda" else a.device
+    ad, wd, sd = _stage(a, dev), _stage(w_int8, dev), _stage(scales, dev)
+    od = _out_like(out, (a.shape[0], w_int8.shape[0]), torch.float16, dev)
+    torch.ops.hexmi.w8a16_matmul(ad, wd, sd, od)
+    return _finish(od, out)
+
+
+def dequant_w8(w_int8, scales, out=None):
+    """fp32 [N,K] = float(W[n,k]) * float(scales[n]) (the dequantisation the fused kernel applies)."""
+    if w_int8.dtype != torch.int8 or scales.dtype != torch.float16:
+        raise TypeError("hexmi.dequant_w8: expected int8 weights, fp16 scales")
+    dev = _device() if w_int8.device.type != "cuda" else w_int8.device
+    wd, sd = _stage(w_int8, dev), _stage(scales, dev)
+    od = _out_like(out, w_int8.shape, torch.float32, dev)
+    torch.ops.hexmi.dequant_w8(wd, sd, od)
+    return _finish(od, out)
+
+
+def flash_attention(q, k, v, sm_scale=None, causal=False, out=None, out_dtype=None):
+    """softmax(sm_scale * Q K^T [+causal]) V for [Z,H,S,D] tensors
+    (`F.scaled_dot_product_attention(q, k, v, scale=...)`, test/python/triton/test_flash_attention.py:212)."""
+    if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("hexmi.flash_attention: q, k, v must share one [Z,H,S,D] shape")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("hexmi.flash_attention: q, k, v dtypes differ")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(q.shape[-1])
+    if out_dtype is None:
+        out_dtype = out.dtype if out is not None else q.dtype
+    dev = _device() if q.device.type != "cuda" else q.device
+    qd, kd, vd = _stage(q, dev), _stage(k, dev), _stage(v, dev)
+    od = _out_like(out, q.shape, out_dtype, dev)
+    torch.ops.hexmi.flash_attention(qd, kd, vd, float(sm_scale), bool(causal), od)
+    return _finish(od, out)

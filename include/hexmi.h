@@ -1,0 +1,145 @@
+/*
+ * hexmi.h - C ABI of libhexmi.so: hand-written gfx950 (MI355X) kernels for the
+ * operator set that hexagon-mlir lowers its tutorial kernels to.
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is
+ *     allocated, freed or retained by the library;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     calls enqueue work and return without synchronising;
+ *   - the return value is HEXMI_OK or a negative hexmi_status; nothing throws;
+ *   - calls are re-entrant; two calls may run concurrently on different streams.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the hexagon-mlir source tree).
+ */
+#ifndef HEXMI_H
+#define HEXMI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *hexmi_stream_t; /* hipStream_t */
+
+typedef enum hexmi_status {
+  HEXMI_OK = 0,
+  HEXMI_EINVAL = -1,  /* null pointer, non-positive size, bad leading dim, misaligned */
+  HEXMI_ENOTSUP = -2, /* dtype / shape combination with no kernel */
+  HEXMI_ELAUNCH = -3  /* hipLaunchKernel or another HIP call failed */
+} hexmi_status;
+
+/* Element types. Values match the reference's raw-tensor dtype ids where one
+ * exists (test/utils/dsp/include/tensor.h:26-38 is the id table the device
+ * harness and backend/utils.py:36-54 share). */
+typedef enum hexmi_dtype {
+  HEXMI_F32 = 0,
+  HEXMI_F16 = 1,
+  HEXMI_BF16 = 2,
+  HEXMI_I8 = 3
+} hexmi_dtype;
+
+/* Library / device ------------------------------------------------------- */
+
+/* "hexmi <major>.<minor> gfx950" */
+const char *hexmi_version(void);
+/* Text for a status code. */
+const char *hexmi_strerror(int status);
+/* Number of compute units of the current device (0 if no device). The
+ * reference counterpart is the fixed thread count the launcher passes
+ * (backend/hexagon_options.py:24 num_threads). */
+int hexmi_num_cus(void);
+
+/* Row reductions --------------------------------------------------------- */
+
+/* y[r, :] = softmax(x[r, :]) for r in [0, rows). exp is evaluated in fp32 for
+ * every dtype; max-subtracted; masked columns behave as -inf.
+ * Stands in for the compiled `softmax_kernel(x_ptr, output_ptr, NUM_ROWS,
+ * NUM_COLS, BLOCK_SIZE)` of test/python/triton/test_softmax.py:44-72 and
+ * nn.Softmax(dim=1) of test/python/torch-mlir/test_softmax_torch.py:24-31.
+ * ld_x / ld_y: elements between consecutive rows (>= cols).
+ * dtype: HEXMI_F32, HEXMI_F16 or HEXMI_BF16 (input and output alike). */
+int hexmi_softmax(const void *x, void *y, int64_t rows, int64_t cols,
+                  int64_t ld_x, int64_t ld_y, int dtype, hexmi_stream_t stream);
+
+/* y = x * rsqrt(mean(x^2) + eps) * weight, fp32 accumulation.
+ * Stands in for `rms_norm_fwd_kernel(x_ptr, y_ptr, weights_ptr, BLOCK_SIZE,
+ * EPSILON, NUM_COLS, NUM_ROWS)` of test/python/triton/test_rms_norm.py:37-63.
+ * x, y: [rows, cols] contiguous; weight: [cols]; all of `dtype`. */
+int hexmi_rms_norm(const void *x, const void *weight, void *y, int64_t rows,
+                   int64_t cols, float eps, int dtype, hexmi_stream_t stream);
+
+/* y = (x - mean) * rstd * weight + bias with biased variance, fp32
+ * accumulation; mean / rstd (fp32 [rows]) are written when non-NULL.
+ * Stands in for `layer_norm_fwd_kernel(x_ptr, y_ptr, weights_ptr, biases_ptr,
+ * mean_ptr, rstd_ptr, BLOCK_SIZE, EPSILON, NUM_COLS, NUM_ROWS)` of
+ * test/python/triton/test_layer_norm.py:42-82 and nn.LayerNorm of
+ * test/python/torch-mlir/test_layernorm_torch.py:24-31.
+ * weight / bias may be NULL (treated as 1 / 0). */
+int hexmi_layer_norm(const void *x, const void *weight, const void *bias,
+                     void *y, float *mean, float *rstd, int64_t rows,
+                     int64_t cols, float eps, int dtype, hexmi_stream_t stream);
+
+/* Dense GEMM ------------------------------------------------------------- */
+
+/* out[n_row, n_col] (fp32) = act[n_row, n_inner] (fp16) * w[n_inner, n_col]
+ * (fp16), all row-major contiguous. Same name order and meaning as the
+ * runtime routine the compiler calls for hexkl.matmul:
+ * `int hexkl_matmul_f16f16_f32(n_row, n_col, n_inner, outM, inAct, inW)`,
+ * qcom_hexagon_backend/bin/runtime/include/HexKLAPI.h:17-20 (body
+ * bin/runtime/src/HexKLAPI.cpp:15-141), plus the stream. */
+int hexmi_matmul_f16f16_f32(int64_t n_row, int64_t n_col, int64_t n_inner,
+                            float *out, const void *act, const void *w,
+                            hexmi_stream_t stream);
+
+/* C[M,N] = A[M,K] * op(B); fp32 accumulation on MFMA.
+ *   trans_b == 0: B is [K,N] row-major with leading dim ldb (the `matmul`
+ *     kernel of test/python/triton/test_matmul.py:35-70: strides (K,1),(N,1),(N,1));
+ *   trans_b != 0: B is [N,K] row-major (`x @ W.T`,
+ *     test/python/torch-mlir/test_hexkl_macro_matmul.py:24-28).
+ * in_dtype: HEXMI_F16 or HEXMI_BF16 (A and B). out_dtype: in_dtype or HEXMI_F32
+ * (the fp16 x fp16 -> fp32 form of docs/tutorials/triton/matmul_hexkl.md:61-97). */
+int hexmi_gemm(int64_t M, int64_t N, int64_t K, const void *A, int64_t lda,
+               const void *B, int64_t ldb, void *C, int64_t ldc, int in_dtype,
+               int out_dtype, int trans_b, hexmi_stream_t stream);
+
+/* Weight-only int8 GEMM (W8A16): C[m,n] = sum_k A[m,k] * (float(W[n,k]) *
+ * float(scales[n])), fp32 accumulation, C fp16.
+ * A fp16 [M,K]; W int8 [N,K] row-major (symmetric, zero-point 0); scales fp16
+ * [N], one per output channel. The reference has no such kernel; this is the
+ * fusion of quant.dcast lowering
+ * (qcom_hexagon_backend/lib/Conversion/LinalgToLLVM/LinalgToLLVMPass.cpp:224-230)
+ * with the transposed-weight matmul of test_hexkl_macro_matmul.py:24-28. */
+int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void *A,
+                     const int8_t *W, const void *scales, void *C,
+                     hexmi_stream_t stream);
+
+/* out[n,k] (fp32) = float(W[n,k]) * float(scales[n]): the dequantisation the
+ * fused kernel applies, exposed so indexing and scale selection can be
+ * checked bit-exactly. */
+int hexmi_dequant_w8(int64_t N, int64_t K, const int8_t *W, const void *scales,
+                     float *out, hexmi_stream_t stream);
+
+/* Attention -------------------------------------------------------------- */
+
+/* O = softmax(sm_scale * Q K^T [+ causal mask]) V per (z, h), online softmax
+ * with fp32 running max / sum, exp2 with sm_scale*log2(e) folded in.
+ * Q, K, V, O: [Z, H, S, D] contiguous (strides H*S*D, S*D, D, 1).
+ * Stands in for `attention_fwd_kernel(pid1, Q, K, V, sm_scale, Out, H, N_CTX,
+ * BLOCK_M, BLOCK_DMODEL, BLOCK_N, STAGE, stride_0..3)` of
+ * test/python/triton/test_flash_attention.py:37-168 (STAGE=1 is causal == 0)
+ * and tm_tensor.attention (include/hexagon/Dialect/TmTensor/IR/TmTensorOps.td:28-56).
+ * in_dtype: HEXMI_F16 / HEXMI_BF16 (MFMA path) or HEXMI_F32.
+ * out_dtype: in_dtype, or HEXMI_F32 with fp16 inputs (the fp16 QKV -> fp32 O
+ * form of test/python/mlir/hexkl_attention/input.mlir:1-169). */
+int hexmi_flash_attn_fwd(const void *Q, const void *K, const void *V, void *O,
+                         int64_t Z, int64_t H, int64_t S, int64_t D,
+                         float sm_scale, int causal, int in_dtype,
+                         int out_dtype, hexmi_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HEXMI_H */

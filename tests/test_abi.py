@@ -1,0 +1,81 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/hexmi.h declares; the Python
+loader binds exactly that set; argument checks that need no device return the documented status."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hexmi.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hexmi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_expected_entry_points():
+    names = _declared()
+    for must in ("hexmi_softmax", "hexmi_rms_norm", "hexmi_layer_norm", "hexmi_matmul_f16f16_f32", "hexmi_gemm",
+                 "hexmi_gemm_w8a16", "hexmi_dequant_w8", "hexmi_flash_attn_fwd"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    import hexmi
+    assert os.path.exists(hexmi.LIB_PATH), "build libhexmi.so first: python hexagon-mlir_amd/build.py"
+    handle = ctypes.CDLL(hexmi.LIB_PATH)
+    for name in _declared():
+        assert hasattr(handle, name), "libhexmi.so does not export %s" % name
+
+
+def test_loader_binds_exactly_the_header():
+    from hexmi import _lib
+    assert sorted(_lib.SIGNATURES) == _declared()
+    lib = _lib.lib()
+    assert lib.hexmi_version().decode().startswith("hexmi ")
+    assert "invalid" in _lib.strerror(_lib.EINVAL)
+
+
+def test_argument_errors_need_no_device():
+    from hexmi import _lib
+    lib = _lib.lib()
+    # negative sizes and short leading dimensions are rejected before any HIP call
+    assert lib.hexmi_softmax(None, None, -1, 8, 8, 8, _lib.F32, None) == _lib.EINVAL
+    assert lib.hexmi_softmax(None, None, 4, 8, 4, 8, _lib.F32, None) == _lib.EINVAL
+    assert lib.hexmi_softmax(None, None, 4, 8, 8, 8, _lib.F32, None) == _lib.EINVAL      # null pointers
+    assert lib.hexmi_softmax(None, None, 0, 8, 8, 8, _lib.F32, None) == _lib.OK          # empty: nothing to do
+    assert lib.hexmi_rms_norm(None, None, None, 3, 5, 1e-5, _lib.F16, None) == _lib.EINVAL
+    assert lib.hexmi_layer_norm(None, None, None, None, None, None, 0, 0, 1e-5, _lib.F16, None) == _lib.OK
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from hexmi import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libhexmi.so")
+    with pytest.raises(RuntimeError, match="no CPU or eager fallback"):
+        _lib.lib()
+
+
+def test_ops_refuse_to_run_without_gpu():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    import hexmi
+    with pytest.raises(RuntimeError, match="needs a GPU"):
+        hexmi.softmax(torch.zeros(2, 2))
+
+
+def test_kernel_front_checks_grid_and_options():
+    import torch
+    import hexmi
+    k = hexmi.kernels.softmax_kernel
+    with pytest.raises(ValueError, match="at least 1 thread"):
+        k[(0,)]
+    x = torch.zeros(2, 2)
+    with pytest.raises(TypeError):
+        k[(1,)](x, x, NUM_ROWS=2, NUM_COLS=2, BLOCK_SIZE=2, notAnOption=True)
+    with pytest.raises(RuntimeError, match="outside"):
+        k(x, x)
