@@ -1,0 +1,336 @@
+#!/usr/bin/env python3
+"""Roofline bench of the hexmi kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-suite] [--no-cpu]
+
+Prints ONE JSON line. The headline `value` is the primary workload's throughput (default `norms`: one step =
+RMSNorm + LayerNorm over the fp16 [8192, 4096] batch, GB/s of algorithmic bytes) with inputs resident in HBM
+and the buffers rotated over > 512 MB so the 256 MB Infinity Cache cannot serve them. `suite` carries the same
+measurement for every other configuration (GEMM / attention in TFLOP/s, W8A16 and softmax in GB/s), each with
+its own roofline fraction. `cpu_baseline` times the reference's CPU path (the PyTorch CPU op its tests use as
+oracle) on the host cores for the primary workload; suite entries carry their own `cpu` leg.
+
+Kernel launch durations are measured with HIP events on the stream the kernels are launched on (torch's
+current stream, which hexmi passes to the C ABI).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "hexagon-mlir_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 / bf16 matrix, published
+ROTATE_BYTES = 640 << 20       # rotate HBM-bound workloads over more than 2x the 256 MB Infinity Cache
+
+
+class Workload:
+    """One measured configuration: device buffers (several rotated sets), the launch, its algorithmic work."""
+
+    name = ""
+    bound = "hbm"
+    dtype = ""
+    work = 0                   # algorithmic bytes (hbm) or FLOP (mfma) per step
+    desc = ""
+    kernel = ""                # name of the dominant kernel as rocprofv3 reports it
+
+    def setup(self, torch, hexmi):
+        raise NotImplementedError
+
+    def step(self, i):
+        raise NotImplementedError
+
+    def cpu(self, torch):
+        """Returns (seconds per step-equivalent, sample description) for the reference's CPU path."""
+        raise NotImplementedError
+
+
+def _sets(torch, tensors, bytes_per_set, rotate=True):
+    n = max(1, -(-ROTATE_BYTES // bytes_per_set)) if rotate else 1
+    out = []
+    for _ in range(n):
+        out.append({k: (v.cuda() if hasattr(v, "cuda") else v) for k, v in tensors.items()})
+    return out
+
+
+class Softmax(Workload):
+    name, bound, dtype, kernel = "softmax_f32_4096x1024", "hbm", "f32", "row_kernel"
+    desc = "row softmax fp32 [4096,1024] N(0,1) seed 0"
+
+    def setup(self, torch, hexmi):
+        from hexmi.workloads import softmax_inputs, softmax_bytes
+        self.hexmi, self.host = hexmi, softmax_inputs()
+        self.work = softmax_bytes(4096, 1024, 4)
+        self.sets = _sets(torch, self.host, self.work)
+        for s in self.sets:
+            s["out"] = torch.empty_like(s["x"])
+
+    def step(self, i):
+        s = self.sets[i % len(self.sets)]
+        self.hexmi.softmax(s["x"], out=s["out"])
+
+    def cpu(self, torch):
+        from oracle import torch_cpu
+        return _time_cpu(lambda: torch_cpu.softmax(self.host["x"]), 5), "full [4096,1024], torch.softmax on CPU"
+
+
+class Norms(Workload):
+    name, bound, dtype, kernel = "norms_f16_8192x4096", "hbm", "f16", "row_kernel"
+    desc = "RMSNorm + LayerNorm fp16 [8192,4096] N(0,1), w~N(1,0.1), b~N(0,0.1), eps 1e-5, fp32 accumulation"
+    which = ("rms", "ln")
+
+    def setup(self, torch, hexmi):
+        from hexmi.workloads import norm_inputs, rms_norm_bytes, layer_norm_bytes
+        self.hexmi, self.host = hexmi, norm_inputs()
+        self.work_rms, self.work_ln = rms_norm_bytes(8192, 4096), layer_norm_bytes(8192, 4096)
+        self.work = (self.work_rms if "rms" in self.which else 0) + (self.work_ln if "ln" in self.which else 0)
+        t = {k: v for k, v in self.host.items() if k != "eps"}
+        self.sets = _sets(torch, t, self.work_rms)
+        for s in self.sets:
+            s["out"] = torch.empty_like(s["x"])
+
+    def step(self, i):
+        s = self.sets[i % len(self.sets)]
+        if "rms" in self.which:
+            self.hexmi.rms_norm(s["x"], s["weight"], 1e-5, out=s["out"])
+        if "ln" in self.which:
+            self.hexmi.layer_norm(s["x"], s["weight"], s["bias"], 1e-5, out=s["out"])
+
+    def cpu(self, torch):
+        from oracle import torch_cpu
+        h = self.host
+
+        def run():
+            if "rms" in self.which:
+                torch_cpu.rms_norm(h["x"], h["weight"], 1e-5)
+            if "ln" in self.which:
+                torch_cpu.layer_norm(h["x"], h["weight"], h["bias"], 1e-5)
+        return _time_cpu(run, 3), "full [8192,4096], F.rms_norm / F.layer_norm on CPU"
+
+
+class RmsNorm(Norms):
+    name, which = "rms_norm_f16_8192x4096", ("rms",)
+    desc = "RMSNorm fp16 [8192,4096]"
+
+
+class LayerNorm(Norms):
+    name, which = "layer_norm_f16_8192x4096", ("ln",)
+    desc = "LayerNorm fp16 [8192,4096]"
+
+
+class Gemm(Workload):
+    bound, kernel = "mfma", "gemm_kernel"
+
+    def __init__(self, size, dtype_name):
+        self.size, self.dtype = size, dtype_name
+        self.name = "gemm_%s_%d" % (dtype_name, size)
+        self.desc = "C=A.B %s [%d,%d]x[%d,%d] U(-1,1), fp32 accumulate, %s out" % (dtype_name, size, size, size, size,
+                                                                                   dtype_name)
+
+    def setup(self, torch, hexmi):
+        from hexmi.workloads import gemm_inputs, gemm_flops
+        dt = torch.float16 if self.dtype == "f16" else torch.bfloat16
+        self.hexmi, self.host = hexmi, gemm_inputs(self.size, self.size, self.size, dt)
+        self.work = gemm_flops(self.size, self.size, self.size)
+        self.sets = _sets(torch, self.host, 0, rotate=False)
+        self.sets[0]["out"] = torch.empty(self.size, self.size, dtype=dt, device="cuda")
+
+    def step(self, i):
+        s = self.sets[0]
+        self.hexmi.matmul(s["a"], s["b"], out=s["out"])
+
+    def cpu(self, torch):
+        from oracle import torch_cpu
+        n = self.size
+        rows = n if n <= 4096 else n // 8
+        a = self.host["a"][:rows]
+        t = _time_cpu(lambda: torch_cpu.matmul(a, self.host["b"]), 1 if n > 4096 else 2)
+        return t * (n / rows), "rows 0..%d of A (of %d) x full B, fp32 torch.matmul on CPU, time scaled to the full GEMM" % (rows, n)
+
+
+class W8A16(Workload):
+    bound, dtype, kernel = "hbm", "f16", "w8a16_kernel"
+
+    def __init__(self, M):
+        self.M = M
+        self.name = "w8a16_m%d" % M
+        self.desc = "W8A16 A fp16 [%d,4096] N(0,1), W int8 [11008,4096], per-channel fp16 scales, fp32 accumulate" % M
+
+    def setup(self, torch, hexmi):
+        from hexmi.workloads import w8a16_inputs, w8a16_bytes
+        self.hexmi, self.host = hexmi, w8a16_inputs(self.M)
+        self.work = w8a16_bytes(self.M, 11008, 4096)
+        self.sets = _sets(torch, self.host, self.work)
+        for s in self.sets:
+            s["out"] = torch.empty(self.M, 11008, dtype=torch.float16, device="cuda")
+
+    def step(self, i):
+        s = self.sets[i % len(self.sets)]
+        self.hexmi.w8a16_matmul(s["a"], s["w"], s["scales"], out=s["out"])
+
+    def cpu(self, torch):
+        from oracle import torch_cpu
+        h = self.host
+        return (_time_cpu(lambda: torch_cpu.w8a16_matmul(h["a"], h["w"], h["scales"]), 2),
+                "full size, dequantise + fp32 matmul on CPU")
+
+
+class Attention(Workload):
+    bound, dtype, kernel = "mfma", "f16", "flash_fwd_kernel"
+
+    def __init__(self, Z, H, S, D):
+        self.shape = (Z, H, S, D)
+        self.name = "attn_causal_f16_%dx%dx%dx%d" % self.shape
+        self.desc = "causal flash-attention fwd fp16 [%d,%d,%d,%d] N(0,1), scale 1/sqrt(%d), fp32 stats" % (Z, H, S, D, D)
+
+    def setup(self, torch, hexmi):
+        from hexmi.workloads import attention_inputs, attention_flops
+        self.hexmi, self.host = hexmi, attention_inputs(*self.shape)
+        self.work = attention_flops(*self.shape, causal=True)
+        t = {k: v for k, v in self.host.items() if k != "sm_scale"}
+        self.sets = _sets(torch, t, 0, rotate=False)
+        self.sets[0]["out"] = torch.empty_like(self.sets[0]["q"])
+
+    def step(self, i):
+        s = self.sets[0]
+        self.hexmi.flash_attention(s["q"], s["k"], s["v"], self.host["sm_scale"], True, out=s["out"])
+
+    def cpu(self, torch):
+        from oracle import torch_cpu
+        Z, H, S, D = self.shape
+        heads = 8 if S <= 4096 else 2
+        h = self.host
+        q, k, v = (h[n].reshape(Z * H, S, D)[:heads][None] for n in ("q", "k", "v"))
+        t = _time_cpu(lambda: torch_cpu.attention(q, k, v, h["sm_scale"], True), 1)
+        return t * (Z * H / heads), "%d of %d heads, fp32 F.scaled_dot_product_attention(is_causal=True) on CPU, time scaled" % (heads, Z * H)
+
+
+def _time_cpu(fn, iters):
+    fn()                                                # warm-up
+    ts = []
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def make_workloads():
+    return {w.name: w for w in (
+        Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
+        W8A16(1), W8A16(16), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128))}
+
+
+ALIASES = {"norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "gemm": "gemm_f16_4096",
+           "gemm_bf16": "gemm_bf16_8192", "attn": "attn_causal_f16_4x32x4096x128",
+           "attn_long": "attn_causal_f16_1x32x16384x128", "rms_norm": "rms_norm_f16_8192x4096",
+           "layer_norm": "layer_norm_f16_8192x4096"}
+
+
+def measure(torch, wl, steps, warmup):
+    """Returns ms per step from HIP events around `steps` launches on the current stream."""
+    for i in range(warmup):
+        wl.step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        wl.step(warmup + i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return e0.elapsed_time(e1) / steps, wall_ms
+
+
+def report(wl, ms):
+    if wl.bound == "hbm":
+        achieved, peak, unit = wl.work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved, peak, unit = wl.work / (ms * 1e-3) / 1e12, MFMA_PEAK_TFLOPS, "TFLOP/s"
+    return {"bound": wl.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": None, "kernel": wl.kernel, "work_per_step": wl.work}
+
+
+def steps_for(wl, steps):
+    if wl.name.startswith("gemm_bf16_8192") or "16384" in wl.name:
+        return max(5, steps // 5)
+    return steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="norms")
+    ap.add_argument("--no-suite", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    import hexmi
+    hexmi.lib()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+
+    wls = make_workloads()
+    primary = wls[ALIASES.get(args.workload, args.workload)]
+    primary.setup(torch, hexmi)
+    ms, wall_ms = measure(torch, primary, args.steps, args.warmup)
+    roof = report(primary, ms)
+    unit = roof["unit"]
+    line = {
+        "metric": "GEMM/attn TFLOP/s + softmax/norm GB/s, % of MI355X roofline, 1 GPU",
+        "value": roof["achieved"], "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 5), "wall_ms_per_step": round(wall_ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": primary.dtype, "data": "synthetic",
+        "config": {"workload": primary.name, "description": primary.desc,
+                   "buffers": "%d rotated sets" % len(primary.sets)},
+        "roofline": roof,
+    }
+    if not args.no_cpu:
+        sec, sample = primary.cpu(torch)
+        cpu_val = primary.work / sec / (1e9 if primary.bound == "hbm" else 1e12)
+        line["cpu_baseline"] = {"value": round(cpu_val, 3), "unit": unit, "cores": cores, "kind": "port",
+                                "sample": sample, "ms": round(sec * 1e3, 3)}
+    primary.sets = None
+    torch.cuda.empty_cache()
+
+    if not args.no_suite:
+        suite = []
+        for name, wl in wls.items():
+            if wl is primary or name in ("norms_f16_8192x4096",):
+                continue
+            print("# measuring %s" % name, file=sys.stderr, flush=True)
+            wl.setup(torch, hexmi)
+            k = steps_for(wl, args.steps)
+            wms, _ = measure(torch, wl, k, args.warmup)
+            entry = {"workload": name, "ms": round(wms, 5), "steps": k}
+            entry.update(report(wl, wms))
+            if not args.no_cpu:
+                sec, sample = wl.cpu(torch)
+                entry["cpu"] = {"ms": round(sec * 1e3, 3), "cores": cores, "sample": sample,
+                                "value": round(wl.work / sec / (1e9 if wl.bound == "hbm" else 1e12), 4)}
+            suite.append(entry)
+            wl.sets = None
+            wl.host = None
+            torch.cuda.empty_cache()
+        line["suite"] = suite
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -160,7 +160,8 @@ def softmax(x, out=None, dim=-1):
     xd = _stage(x, dev)
     od = _out_like(out, x.shape, x.dtype, dev)
     cols = x.shape[-1]
-    torch.ops.hexmi.softmax(xd.view(-1, cols), od.view(-1, cols))
+    rows = x.numel() // max(cols, 1)
+    torch.ops.hexmi.softmax(xd.view(rows, cols), od.view(rows, cols))
     return _finish(od, out)
 
 
@@ -168,11 +169,12 @@ def rms_norm(x, weight=None, eps=1e-5, out=None):
     """`F.rms_norm(x, (C,), weight, eps)` (test/python/triton/test_rms_norm.py:85-87)."""
     dev = _device() if x.device.type != "cuda" else x.device
     cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
     if weight is not None and (weight.shape != (cols,) or weight.dtype != x.dtype):
         raise ValueError("hexmi.rms_norm: weight must be [%d] of %s" % (cols, x.dtype))
     xd, wd = _stage(x, dev), _stage(weight, dev)
     od = _out_like(out, x.shape, x.dtype, dev)
-    torch.ops.hexmi.rms_norm(xd.view(-1, cols), wd, float(eps), od.view(-1, cols))
+    torch.ops.hexmi.rms_norm(xd.view(rows, cols), wd, float(eps), od.view(rows, cols))
     return _finish(od, out)
 
 
@@ -189,7 +191,7 @@ def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=No
     od = _out_like(out, x.shape, x.dtype, dev)
     md = None if mean is None else _out_like(mean if mean.dtype == torch.float32 else None, (rows,), torch.float32, dev)
     rd = None if rstd is None else _out_like(rstd if rstd.dtype == torch.float32 else None, (rows,), torch.float32, dev)
-    torch.ops.hexmi.layer_norm(xd.view(-1, cols), wd, bd, float(eps), od.view(-1, cols), md, rd)
+    torch.ops.hexmi.layer_norm(xd.view(rows, cols), wd, bd, float(eps), od.view(rows, cols), md, rd)
     if mean is not None:
         _finish(md, mean)
     if rstd is not None:

@@ -3,7 +3,8 @@
 Tolerances. The kernel accumulates in fp32 on the matrix cores; the oracle accumulates in double.
   fp32 output: |got - want| <= 1e-5 * sum_k |a_ik b_kj| (rel-err 1e-5 of the magnitude actually summed; the
     plain rel-err of max|C| is reported by the config-size test and must be <= 1e-5 as well);
-  fp16 / bf16 output: within one unit in the last place of the oracle's rounded value. (A flat 2e-2 max-abs is
+  fp16 / bf16 output: within one unit in the last place of the oracle's rounded value, or within 1e-5 of the
+    summed magnitude where the value is a cancellation residue. (A flat 2e-2 max-abs is
     also asserted after scaling by 1/sqrt(K), the scale attention-sized outputs have; at |c| ~ 100 one fp16 ulp
     is 0.06, so the raw bound cannot hold for any implementation.)
 """
@@ -59,7 +60,8 @@ def test_gemm_parity(hexmi, oracle, shape, dtype, trans_b):
     assert ((got32 - want32).abs() <= 1e-5 * mag + 1e-30).all()
     got = hexmi.matmul(a.cuda(), b.cuda(), trans_b=trans_b).cpu()
     want = _oracle_mm(oracle, a, b, dtype, trans_b)
-    assert got.dtype == dtype and close16(got, want, max_ulp=1)
+    # values that are cancellation residues (|c| << sum |a b|) carry the fp32 rounding of the larger partial sums
+    assert got.dtype == dtype and close16(got, want, max_ulp=1, atol=1e-5 * float(mag.max()))
     assert ((got.float() - want.float()).abs().max() / math.sqrt(K)) <= 2e-2
 
 
@@ -108,7 +110,7 @@ def test_reference_matmul_call_site(hexmi, oracle):
     hexmi.kernels.matmul[(1,)](A, B, C, 1024, 512, 64, enableMultiThreading=True, enableVTCMTiling=True,
                                enableConvertToHexagonmem=True, enableHexagonmemCopyToDMA=True)
     want = from_np(oracle.matmul(A.numpy(), B.numpy()), torch.float16)
-    assert torch.allclose(C, want, atol=2e-1) and close16(C, want, 1)
+    assert torch.allclose(C, want, atol=2e-1) and close16(C, want, 1, atol=1e-4)
     # matmul_hexkl.md:100-111: fp32 C, rtol 1e-2
     C32 = torch.zeros((1024, 512), dtype=torch.float32)
     hexmi.kernels.matmul_hexkl[(1,)](A, B, C32, 1024, 512, 64, enableHexKL=True)
@@ -121,12 +123,12 @@ def test_macro_matmul_shapes(hexmi, oracle):
     x = torch.randn(512, 1024).half()
     w = torch.randn(1024, 1024).half()
     got = hexmi.matmul(x.cuda(), w.cuda()).cpu()
-    assert close16(got, from_np(oracle.matmul(x.numpy(), w.numpy()), torch.float16), 1)
+    assert close16(got, from_np(oracle.matmul(x.numpy(), w.numpy()), torch.float16), 1, atol=1e-4)
     x2 = torch.randn(1024, 512).half()
     w2 = torch.randn(256, 512).half()
     got2 = hexmi.matmul(x2.cuda(), w2.cuda(), trans_b=True).cpu()
     want2 = from_np(oracle.matmul(x2.numpy(), w2.numpy(), trans_b=True), torch.float16)
-    assert close16(got2, want2, 1) and torch.allclose(got2.float(), want2.float(), rtol=1e-2, atol=1e-2)
+    assert close16(got2, want2, 1, atol=1e-4) and torch.allclose(got2.float(), want2.float(), rtol=1e-2, atol=1e-2)
 
 
 @pytest.mark.parametrize("dtype,size", [(torch.float16, 4096), (torch.bfloat16, 8192)])
@@ -149,7 +151,7 @@ def test_gemm_config_sizes(hexmi, oracle, dtype, size):
     assert rel_err(got32, want32) <= 1e-5
     od = "bf16" if dtype == torch.bfloat16 else np.float16
     want = from_np(oracle.matmul(an, bn, out_dtype=od, dtype=tag), dtype)
-    assert close16(c[rows.cuda()].cpu(), want, 1)
+    assert close16(c[rows.cuda()].cpu(), want, 1, atol=1e-4)
     perm = torch.randperm(size, generator=_gen(7)).cuda()
     c_perm = hexmi.matmul(ad[perm].contiguous(), bd)
     assert torch.equal(c_perm, c[perm])

@@ -82,8 +82,8 @@ def test_softmax_host_tensors_in_place(hexmi, oracle):
 def test_softmax_extreme_values(hexmi):
     x = torch.tensor([[1e4, 1e4 - 1, -1e4, 0.0], [-float("inf"), 0.0, 0.0, -float("inf")]], device="cuda")
     y = hexmi.softmax(x).cpu()
-    e = np.exp(-1.0)
-    assert torch.allclose(y[0], torch.tensor([1 / (1 + e), e / (1 + e), 0.0, 0.0]), atol=1e-6)
+    e = float(np.exp(-1.0))
+    assert torch.allclose(y[0], torch.tensor([1 / (1 + e), e / (1 + e), 0.0, 0.0], dtype=torch.float32), atol=1e-6)
     assert torch.allclose(y[1], torch.tensor([0.0, 0.5, 0.5, 0.0]))
 
 
