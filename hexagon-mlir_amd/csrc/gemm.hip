@@ -1,20 +1,26 @@
 // Dense GEMM C[M,N] = A[M,K] * op(B) on gfx950 matrix cores (fp16 / bf16 in, fp32 accumulate).
 //
 // Workgroup = 256 threads = 4 waves in a 2x2 arrangement; each wave owns a (WM*32) x (WN*32) block of C as
-// WM x WN accumulators of v_mfma_f32_32x32x16. The K loop walks 64-wide slabs. A slab of A (and of B) is copied
-// global -> LDS by global_load_lds_dwordx4 (no register staging), double buffered: the copy of slab k+1 is in
-// flight while slab k is multiplied. The two buffers of each operand are separate LDS objects so that the
-// compiler's wait-count tracking keeps reads of one buffer independent of copies into the other.
+// WM x WN accumulators of v_mfma_f32_32x32x16 (4x4 = 256 accumulator registers for the 256x256 tile). The K loop
+// walks 32-wide slabs through FOUR LDS stages. A slab of A (and of B) is copied global -> LDS by
+// global_load_lds_dwordx4 (no register staging); the copy of slab kt+3 is issued while slab kt is multiplied,
+// spread between the MFMAs, and one s_barrier per slab both publishes slab kt+1 and frees the stage of slab kt-1.
+// Fragments are double buffered in registers across that barrier: the LDS reads of the next 16-wide k step are
+// issued between the MFMAs of the current one (sched_group_barrier pins the interleaving). Each stage of each
+// operand is its own LDS object so the compiler's wait-count tracking keeps reads of one stage independent of
+// copies into another.
 //
 // LDS layouts (16-byte chunks, XOR swizzled through the *source* address each lane fetches, since the LDS side
 // of a global_load_lds is fixed at base + lane*16):
-//   K-contiguous operand (A, and B given as [N,K]): [row][8 chunks]; chunk c of row r sits at c ^ ((r>>1)&7).
+//   K-contiguous operand (A, and B given as [N,K]): [row][4 chunks]; chunk c of row r sits at c ^ ((r>>2)&3).
 //     A fragment is one ds_read_b128 per lane (row = lane%32, 8 consecutive k).
 //   N-contiguous operand (B given as [K,N]): [k][BN/8 chunks]; chunk c of row k sits at c ^ ((k&3)<<2).
 //     A fragment is two ds_read_b64_tr_b16: the transposing LDS read hands each lane 4 consecutive k of one column.
 //
 // The MFMA is issued with the B fragment as its first operand, so a lane's 4 consecutive accumulator registers
 // are 4 consecutive columns of one C row and go out as one 8-byte (fp16/bf16) or 16-byte (fp32) store.
+#include <type_traits>
+
 #include "hexmi_common.h"
 
 namespace hexmi {
@@ -23,7 +29,7 @@ namespace {
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 
-constexpr int BK = 64;                 // K extent of a slab (elements)
+constexpr int BK = 32;                 // K extent of a slab (elements)
 constexpr int kChunk = 8;              // elements per 16-byte chunk
 
 template <typename T> struct Mfma;
@@ -40,42 +46,62 @@ template <> struct Mfma<bf16> {
   }
 };
 
-__device__ __forceinline__ int swz_k(int row) { return (row >> 1) & 7; }      // K-contiguous tiles
+__device__ __forceinline__ int swz_k(int row) { return (row >> 2) & 3; }      // K-contiguous tiles
 __device__ __forceinline__ int swz_n(int k) { return (k & 3) << 2; }          // N-contiguous tiles
 
-// Copy a [ROWS x 64] K-contiguous slab (rows clamped to row_max) into LDS. ROWS/32 instructions per wave.
-template <typename T, int ROWS>
-__device__ __forceinline__ void copy_kmajor(const T* __restrict__ g, int64_t ld, int row0, int row_max, int k0,
-                                            T* lds, int wave, int lane) {
-#pragma unroll
-  for (int j = 0; j < ROWS / 32; ++j) {
-    const int inst = j * 4 + wave;                  // 8 rows per instruction
-    const int row = inst * 8 + lane / 8;
-    const int c = (lane % 8) ^ swz_k(row);
-    int grow = row0 + row;
-    grow = grow < row_max ? grow : row_max;
-    __builtin_amdgcn_global_load_lds(HEXMI_GLB(g + (int64_t)grow * ld + k0 + c * kChunk),
-                                     HEXMI_LDS(lds + inst * 8 * BK), 16, 0, 0);
-  }
-}
+// s_waitcnt immediate (gfx9 encoding): at most `vm` vector-memory operations outstanding, all LDS reads returned.
+constexpr int waitcnt_imm(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | (7 << 4) | (0 << 8); }
 
-// Copy a [64 x COLS] N-contiguous slab (column chunks clamped to col_max) into LDS. COLS/32 instructions per wave.
-template <typename T, int COLS>
-__device__ __forceinline__ void copy_nmajor(const T* __restrict__ g, int64_t ld, int k0, int col0, int col_max,
-                                            T* lds, int wave, int lane) {
-  constexpr int CPR = COLS / kChunk;                // chunks per row
+// global -> LDS copy of a [ROWS x 32] K-contiguous slab: ROWS/64 wave-wide instructions per wave, 16 rows each.
+// Rows past row_max are clamped (their products are never stored).
+template <typename T, int ROWS>
+struct KMajorLoader {
+  static constexpr int NI = ROWS / 64;
+  const T* ptr[NI];
+  int lds_off[NI];
+  __device__ __forceinline__ void init(const T* g, int64_t ld, int row0, int row_max, int wave, int lane) {
 #pragma unroll
-  for (int j = 0; j < COLS / 32; ++j) {
-    const int inst = j * 4 + wave;
-    const int lin = inst * 64 + lane;
-    const int k = lin / CPR;
-    const int c = (lin % CPR) ^ swz_n(k);
-    int gcol = col0 + c * kChunk;
-    gcol = gcol < col_max ? gcol : col_max;
-    __builtin_amdgcn_global_load_lds(HEXMI_GLB(g + (int64_t)(k0 + k) * ld + gcol), HEXMI_LDS(lds + inst * 64 * kChunk),
-                                     16, 0, 0);
+    for (int j = 0; j < NI; ++j) {
+      const int inst = j * 4 + wave;
+      const int row = inst * 16 + lane / 4;
+      const int c = (lane % 4) ^ swz_k(row);
+      int grow = row0 + row;
+      grow = grow < row_max ? grow : row_max;
+      ptr[j] = g + (int64_t)grow * ld + c * kChunk;
+      lds_off[j] = inst * 16 * BK;
+    }
   }
-}
+  template <int J> __device__ __forceinline__ void issue(T* lds, int k0) const {
+    __builtin_amdgcn_global_load_lds(HEXMI_GLB(ptr[J] + k0), HEXMI_LDS(lds + lds_off[J]), 16, 0, 0);
+  }
+};
+
+// global -> LDS copy of a [32 x COLS] N-contiguous slab; column chunks past col_max are clamped.
+template <typename T, int COLS>
+struct NMajorLoader {
+  static constexpr int NI = COLS / 64;
+  static constexpr int CPR = COLS / kChunk;         // chunks per row
+  const T* ptr[NI];
+  int lds_off[NI];
+  int64_t ld;
+  __device__ __forceinline__ void init(const T* g, int64_t ld_, int col0, int col_max, int wave, int lane) {
+    ld = ld_;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int inst = j * 4 + wave;
+      const int lin = inst * 64 + lane;
+      const int k = lin / CPR;
+      const int c = (lin % CPR) ^ swz_n(k);
+      int gcol = col0 + c * kChunk;
+      gcol = gcol < col_max ? gcol : col_max;
+      ptr[j] = g + (int64_t)k * ld + gcol;
+      lds_off[j] = inst * 64 * kChunk;
+    }
+  }
+  template <int J> __device__ __forceinline__ void issue(T* lds, int k0) const {
+    __builtin_amdgcn_global_load_lds(HEXMI_GLB(ptr[J] + (int64_t)k0 * ld), HEXMI_LDS(lds + lds_off[J]), 16, 0, 0);
+  }
+};
 
 template <typename T>
 __device__ __forceinline__ typename Mfma<T>::Frag read_kmajor(const T* lds, int row, int chunk) {
@@ -133,16 +159,21 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
   tn = in_group / gm;
 }
 
-template <typename T, typename OutT, int WM, int WN, bool TRANS_B>
+// K % 32 == 0. TAIL: the slab count is not a multiple of 4, so the last pass over the four stages guards its MFMAs.
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL>
 __global__ __launch_bounds__(256)
 void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restrict__ C, int M, int N, int K,
                  int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n) {
   typedef typename Mfma<T>::Frag Frag;
   constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
-  __shared__ __attribute__((aligned(16))) T a_lds0[BM * BK];
-  __shared__ __attribute__((aligned(16))) T a_lds1[BM * BK];
-  __shared__ __attribute__((aligned(16))) T b_lds0[BN * BK];
-  __shared__ __attribute__((aligned(16))) T b_lds1[BN * BK];
+  __shared__ __attribute__((aligned(16))) T a_s0[BM * BK];
+  __shared__ __attribute__((aligned(16))) T a_s1[BM * BK];
+  __shared__ __attribute__((aligned(16))) T a_s2[BM * BK];
+  __shared__ __attribute__((aligned(16))) T a_s3[BM * BK];
+  __shared__ __attribute__((aligned(16))) T b_s0[BN * BK];
+  __shared__ __attribute__((aligned(16))) T b_s1[BN * BK];
+  __shared__ __attribute__((aligned(16))) T b_s2[BN * BK];
+  __shared__ __attribute__((aligned(16))) T b_s3[BN * BK];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int wm = wave / 2, wn = wave % 2;
@@ -158,48 +189,112 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  auto load_slab = [&](int kt, T* a_dst, T* b_dst) {
-    copy_kmajor<T, BM>(A, lda, m0, M - 1, kt * BK, a_dst, wave, lane);
-    if constexpr (TRANS_B) copy_kmajor<T, BN>(B, ldb, n0, N - 1, kt * BK, b_dst, wave, lane);
-    else copy_nmajor<T, BN>(B, ldb, kt * BK, n0, N - kChunk, b_dst, wave, lane);
-  };
+  KMajorLoader<T, BM> load_a;
+  load_a.init(A, lda, m0, M - 1, wave, lane);
+  KMajorLoader<T, BN> load_bk;
+  NMajorLoader<T, BN> load_bn;
+  if constexpr (TRANS_B) load_bk.init(B, ldb, n0, N - 1, wave, lane);
+  else load_bn.init(B, ldb, n0, N - kChunk, wave, lane);
+  constexpr int NLA = BM / 64, NLB = BN / 64;       // copy instructions per wave per slab
 
-  auto multiply_slab = [&](const T* a_src, const T* b_src) {
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      Frag af[WM], bf[WN];
-#pragma unroll
-      for (int i = 0; i < WM; ++i) af[i] = read_kmajor<T>(a_src, (wm * WM + i) * 32 + lane % 32, ks * 2 + lane / 32);
-#pragma unroll
-      for (int j = 0; j < WN; ++j) {
-        if constexpr (TRANS_B) bf[j] = read_kmajor<T>(b_src, (wn * WN + j) * 32 + lane % 32, ks * 2 + lane / 32);
-        else bf[j] = read_nmajor<T, BN>(b_src, (wn * WN + j) * 32, ks, lane);
-      }
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j) acc[i][j] = Mfma<T>::run(bf[j], af[i], acc[i][j]);
+  // part 0 = the A copies of slab kt, part 1 = its B copies
+  auto issue_part = [&](int kt, T* a_dst, T* b_dst, auto part) {
+    constexpr int P = decltype(part)::value;
+    const int k0 = kt * BK;
+    if constexpr (P == 0) {
+      load_a.template issue<0>(a_dst, k0);
+      if constexpr (NLA > 1) load_a.template issue<1>(a_dst, k0);
+      if constexpr (NLA > 2) load_a.template issue<2>(a_dst, k0);
+      if constexpr (NLA > 3) load_a.template issue<3>(a_dst, k0);
+    } else if constexpr (TRANS_B) {
+      load_bk.template issue<0>(b_dst, k0);
+      if constexpr (NLB > 1) load_bk.template issue<1>(b_dst, k0);
+      if constexpr (NLB > 2) load_bk.template issue<2>(b_dst, k0);
+      if constexpr (NLB > 3) load_bk.template issue<3>(b_dst, k0);
+    } else {
+      load_bn.template issue<0>(b_dst, k0);
+      if constexpr (NLB > 1) load_bn.template issue<1>(b_dst, k0);
+      if constexpr (NLB > 2) load_bn.template issue<2>(b_dst, k0);
+      if constexpr (NLB > 3) load_bn.template issue<3>(b_dst, k0);
     }
   };
-
+  auto read_frags = [&](const T* a_src, const T* b_src, int ks, Frag* af, Frag* bf) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) af[i] = read_kmajor<T>(a_src, (wm * WM + i) * 32 + lane % 32, ks * 2 + lane / 32);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      if constexpr (TRANS_B) bf[j] = read_kmajor<T>(b_src, (wn * WN + j) * 32 + lane % 32, ks * 2 + lane / 32);
+      else bf[j] = read_nmajor<T, BN>(b_src, (wn * WN + j) * 32, ks, lane);
+    }
+  };
+  auto mfma_all = [&](const Frag* af, const Frag* bf) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j) acc[i][j] = Mfma<T>::run(bf[j], af[i], acc[i][j]);
+  };
+  // Pin the issue order of one group (NREAD LDS reads, NV copies, NMFMA MFMAs) in four identical rounds.
+  constexpr int NREAD = WM + (TRANS_B ? WN : 2 * WN);
+  constexpr int NMFMA = WM * WN;
+  auto interleave = [&](auto nvmem) {
+    constexpr int NV = decltype(nvmem)::value;
+    if constexpr (NMFMA >= 8) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                       // LDS read
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x020, (NV + 3) / 4, 0);            // VMEM read (the copies)
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (NREAD + 3) / 4 - 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / 4 - 2, 0);
+      }
+    }
+  };
+  constexpr int L = NLA + NLB;
   const int KT = K / BK;
-  load_slab(0, a_lds0, b_lds0);
-  int kt = 0;
-  for (; kt + 1 < KT; kt += 2) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();                                  // slab kt landed everywhere; buffer 1 no longer read
-    load_slab(kt + 1, a_lds1, b_lds1);
-    multiply_slab(a_lds0, b_lds0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (kt + 2 < KT) load_slab(kt + 2, a_lds0, b_lds0);
-    multiply_slab(a_lds1, b_lds1);
+  auto clampk = [&](int kt) { return kt < KT ? kt : KT - 1; };   // past the end: reload the last slab (never used)
+  std::integral_constant<int, 0> part_a;
+  std::integral_constant<int, 1> part_b;
+  std::integral_constant<int, NLA> n_a;
+  std::integral_constant<int, NLB> n_b;
+
+  Frag af[2][WM], bf[2][WN];
+  issue_part(0, a_s0, b_s0, part_a);
+  issue_part(0, a_s0, b_s0, part_b);
+  issue_part(clampk(1), a_s1, b_s1, part_a);
+  issue_part(clampk(1), a_s1, b_s1, part_b);
+  issue_part(clampk(2), a_s2, b_s2, part_a);
+  issue_part(clampk(2), a_s2, b_s2, part_b);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * L));   // slab 0 landed
+  __builtin_amdgcn_s_barrier();
+  read_frags(a_s0, b_s0, 0, af[0], bf[0]);
+
+  // One slab. Slab kt lives in stage kt%4 = (ac, bc); (an, bn) is the stage of slab kt+1; (afree, bfree) is the
+  // stage of slab kt-1, released by the barrier that preceded this body, and receives slab kt+3.
+  // At the barrier in the middle the copies still allowed in flight are slab kt+2 and the A part of slab kt+3,
+  // so slab kt+1 has landed for every wave that passes it; every wave has also issued (and, by the lgkmcnt(0)
+  // in the same wait, completed) its last LDS read of slab kt, which frees stage kt%4 for the next body.
+#define HEXMI_SLAB(ac, bc, an, bn, afree, bfree, kt)                  \
+  {                                                                   \
+    issue_part(clampk((kt) + 3), afree, bfree, part_a);               \
+    read_frags(ac, bc, 1, af[1], bf[1]);                              \
+    if (!TAIL || (kt) < KT) mfma_all(af[0], bf[0]);                   \
+    interleave(n_a);                                                  \
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(L + NLA));                 \
+    __builtin_amdgcn_s_barrier();                                     \
+    issue_part(clampk((kt) + 3), afree, bfree, part_b);               \
+    read_frags(an, bn, 0, af[0], bf[0]);                              \
+    if (!TAIL || (kt) < KT) mfma_all(af[1], bf[1]);                   \
+    interleave(n_b);                                                  \
   }
-  if (kt < KT) {                                      // odd slab count: the last slab sits in buffer 0
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    multiply_slab(a_lds0, b_lds0);
+  for (int kt = 0; kt < KT; kt += 4) {
+    HEXMI_SLAB(a_s0, b_s0, a_s1, b_s1, a_s3, b_s3, kt);
+    HEXMI_SLAB(a_s1, b_s1, a_s2, b_s2, a_s0, b_s0, kt + 1);
+    HEXMI_SLAB(a_s2, b_s2, a_s3, b_s3, a_s1, b_s1, kt + 2);
+    HEXMI_SLAB(a_s3, b_s3, a_s0, b_s0, a_s2, b_s2, kt + 3);
   }
+#undef HEXMI_SLAB
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));       // drain the trailing copies before the workgroup's LDS goes away
 
   // acc[i][j][r]: row = lane%32 of the 32x32 tile, column = 8*(r/4) + 4*(lane/32) + r%4.
 #pragma unroll
@@ -264,8 +359,12 @@ int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t 
                  int64_t ldc, hipStream_t s) {
   constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
-  hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A, B, C,
-                     (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+  if ((K / BK) % 4 == 0)
+    hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, false>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A, B,
+                       C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+  else
+    hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, true>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A, B,
+                       C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
   return launch_status();
 }
 
@@ -275,8 +374,10 @@ int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N
   const T* A = static_cast<const T*>(Av);
   const T* B = static_cast<const T*>(Bv);
   OutT* C = static_cast<OutT*>(Cv);
-  const bool fast = K % BK == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && N % 8 == 0 && M >= 1 &&
-                    aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(C, 16) && N >= 8;
+  // The tiled kernels copy 16-byte chunks and clamp (never mask) rows / column chunks, so they need whole
+  // chunks: K % 32 == 0, leading dimensions and N multiples of 8 elements, 16-byte aligned bases.
+  const bool fast = K % BK == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && N % 8 == 0 && N >= 8 &&
+                    aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(C, 16);
   if (fast) {
     const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
     if (big_tiles >= 128) return launch_tiled<T, OutT, 4, 4, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s);
