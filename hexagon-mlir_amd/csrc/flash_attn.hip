@@ -51,21 +51,53 @@ template <int D> __device__ __forceinline__ int swz_vtile(int row) {
   return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
 }
 
+// global -> LDS copy of one [64 keys][D] tile: 64*D/8/64/4 wave-wide instructions per wave. The per-lane element
+// offsets inside a tile do not change from tile to tile, so they are computed once; only a ragged last tile
+// (keys past the end of the sequence) needs its rows clamped.
 template <typename T, int D, bool IS_V>
-__device__ __forceinline__ void copy_kv_tile(const T* __restrict__ g, int key0, int key_max, T* lds, int wave,
-                                             int lane) {
-  constexpr int CPR = D / 8;                       // chunks per row
-  constexpr int INSTS = kBlockN * CPR / 64;        // wave-wide copies per tile
+struct KvTileLoader {
+  static constexpr int CPR = D / 8;                       // chunks per row
+  static constexpr int NI = kBlockN * CPR / 64 / 4;       // instructions per wave
+  int off[NI];                                            // element offset of this lane's chunk inside a tile
+  int row[NI];
+  int col[NI];
+  int lds_off[NI];
+  __device__ __forceinline__ void init(int wave, int lane) {
 #pragma unroll
-  for (int j = 0; j < INSTS / 4; ++j) {
-    const int inst = j * 4 + wave;
-    const int lin = inst * 64 + lane;
-    const int row = lin / CPR;
-    const int c = (lin % CPR) ^ (IS_V ? swz_vtile<D>(row) : swz_ktile<D>(row));
-    int key = key0 + row;
-    key = key < key_max ? key : key_max;
-    __builtin_amdgcn_global_load_lds(HEXMI_GLB(g + (int64_t)key * D + c * 8), HEXMI_LDS(lds + inst * 64 * 8), 16, 0, 0);
+    for (int j = 0; j < NI; ++j) {
+      const int inst = j * 4 + wave;
+      const int lin = inst * 64 + lane;
+      row[j] = lin / CPR;
+      col[j] = ((lin % CPR) ^ (IS_V ? swz_vtile<D>(row[j]) : swz_ktile<D>(row[j]))) * 8;
+      off[j] = row[j] * D + col[j];
+      lds_off[j] = inst * 64 * 8;
+    }
   }
+  __device__ __forceinline__ void issue(const T* __restrict__ g, int key0, int S, T* lds) const {
+    if (key0 + kBlockN <= S) {
+      const T* base = g + (int64_t)key0 * D;
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+        __builtin_amdgcn_global_load_lds(HEXMI_GLB(base + off[j]), HEXMI_LDS(lds + lds_off[j]), 16, 0, 0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        int key = key0 + row[j];
+        key = key < S ? key : S - 1;
+        __builtin_amdgcn_global_load_lds(HEXMI_GLB(g + (int64_t)key * D + col[j]), HEXMI_LDS(lds + lds_off[j]), 16, 0,
+                                         0);
+      }
+    }
+  }
+};
+
+// Value held by lane ^ 32 (v_permlane32_swap exchanges the upper half of one register with the lower half of
+// another; no LDS round trip).
+__device__ __forceinline__ float other_half(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned lo = r[0], hi = r[1];              // lo: lanes hold v[lane%32], hi: lanes hold v[lane%32 + 32]
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? lo : hi);
 }
 
 template <typename OutT>
@@ -81,7 +113,7 @@ template <> __device__ __forceinline__ void store4o<bf16>(bf16* p, float a, floa
 }
 
 template <typename T, typename OutT, int D, bool CAUSAL>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(256, 2)
 void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                       OutT* __restrict__ O, int ZH, int S, float scale_log2e) {
   typedef typename MfmaT<T>::Frag Frag;
@@ -93,7 +125,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   __shared__ __attribute__((aligned(16))) T v_lds0[kBlockN * D];
   __shared__ __attribute__((aligned(16))) T v_lds1[kBlockN * D];
 
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int nqb = (S + kBlockM - 1) / kBlockM;
   const int zh = blockIdx.x % ZH;
   const int qb = nqb - 1 - blockIdx.x / ZH;          // longest rows first
@@ -126,9 +158,13 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   const int key_end = CAUSAL ? ((qb + 1) * kBlockM < S ? (qb + 1) * kBlockM : S) : S;
   const int n_steps = (key_end + kBlockN - 1) / kBlockN;
 
+  KvTileLoader<T, D, false> k_loader;
+  KvTileLoader<T, D, true> v_loader;
+  k_loader.init(wave, lane);
+  v_loader.init(wave, lane);
   auto load_kv = [&](int step, T* k_dst, T* v_dst) {
-    copy_kv_tile<T, D, false>(k_g, step * kBlockN, S - 1, k_dst, wave, lane);
-    copy_kv_tile<T, D, true>(v_g, step * kBlockN, S - 1, v_dst, wave, lane);
+    k_loader.issue(k_g, step * kBlockN, S, k_dst);
+    v_loader.issue(v_g, step * kBlockN, S, v_dst);
   };
 
   auto process = [&](int step, const T* k_src, const T* v_src) {
@@ -136,12 +172,14 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4]
     f32x16 s[2];
 #pragma unroll
-    for (int jt = 0; jt < 2; ++jt) {
+    for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[jt][r] = 0.0f;
-      const int krow = jt * 32 + lane % 32;
 #pragma unroll
-      for (int ds = 0; ds < DS; ++ds) {
+    for (int ds = 0; ds < DS; ++ds) {                 // the two key tiles form two independent MFMA chains
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt) {
+        const int krow = jt * 32 + lane % 32;
         const int c = (ds * 2 + half) ^ swz_ktile<D>(krow);
         Frag kf = *reinterpret_cast<const Frag*>(k_src + (krow * CPR + c) * 8);
         s[jt] = MfmaT<T>::run(kf, qf[ds], s[jt]);
@@ -164,7 +202,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[jt][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    mx = fmaxf(mx, other_half(mx));
     const float m_new = fmaxf(m_i, mx * scale_log2e);
     const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
     float p[2][16];
@@ -178,10 +216,13 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       }
     l_i = l_i * alpha + sum;
     m_i = m_new;
+    // rescale the output accumulator only when some row of this wave raised its maximum (wave-uniform test)
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+        for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+    }
     // ---- O^T += V^T P^T. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
     //      which is score register hf*8 + e of this lane.
     const int g = lane / 16, i16 = lane % 16;
@@ -225,7 +266,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   }
 
   // ---- epilogue: o_acc[dt][r] is O[qrow][dt*32 + 8*(r/4) + 4*half + r%4] * l
-  const float l_tot = l_i + __shfl_xor(l_i, 32, kWave);
+  const float l_tot = l_i + other_half(l_i);
   const float inv_l = 1.0f / l_tot;
   if (qrow < S) {
     OutT* o_row = O + base + (int64_t)qrow * D;
