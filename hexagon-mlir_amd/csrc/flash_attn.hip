@@ -23,6 +23,7 @@ namespace {
 
 constexpr int kBlockM = 128;   // query rows per workgroup
 constexpr int kBlockN = 64;    // keys per step
+constexpr float kRescaleLag = 8.0f;   // how far (log2) the softmax reference maximum may trail the true one
 
 template <typename T> struct MfmaT;
 template <> struct MfmaT<f16> {
@@ -167,84 +168,93 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     v_loader.issue(v_g, step * kBlockN, S, v_dst);
   };
 
-  auto process = [&](int step, const T* k_src, const T* v_src) {
-    const int n0 = step * kBlockN;
-    // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4]
-    f32x16 s[2];
-#pragma unroll
-    for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[jt][r] = 0.0f;
-#pragma unroll
-    for (int ds = 0; ds < DS; ++ds) {                 // the two key tiles form two independent MFMA chains
-#pragma unroll
-      for (int jt = 0; jt < 2; ++jt) {
-        const int krow = jt * 32 + lane % 32;
-        const int c = (ds * 2 + half) ^ swz_ktile<D>(krow);
-        Frag kf = *reinterpret_cast<const Frag*>(k_src + (krow * CPR + c) * 8);
-        s[jt] = MfmaT<T>::run(kf, qf[ds], s[jt]);
-      }
-    }
-    // ---- mask (diagonal and ragged blocks only)
-    const bool need_mask = (CAUSAL && n0 + kBlockN - 1 > q0) || (n0 + kBlockN > S);
+  // One 32-key tile of the online softmax: mask, row max, (rare) rescale, exponentials, row sum; leaves the
+  // probabilities as the two MFMA operands pf[0], pf[1] (score registers 0..7 and 8..15 of this lane).
+  // The reference maximum m_i may lag the true running maximum by up to kRescaleLag (log2 units): softmax is
+  // shift invariant, so exponentials up to 2^kRescaleLag are as exact as ones below 1, and the output
+  // accumulator and running sum only need rescaling when a row outgrows the lag. The decision is per row (lane);
+  // the wave-uniform ballot only skips the multiplications when no row of the wave needs them.
+  auto softmax_tile = [&](int key_base, bool need_mask, f32x16& s, Frag* pf) {
     if (need_mask) {
 #pragma unroll
-      for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = n0 + jt * 32 + 8 * (r / 4) + 4 * half + r % 4;
-          if ((CAUSAL && key > qrow) || key >= S) s[jt][r] = -INFINITY;
-        }
+      for (int r = 0; r < 16; ++r) {
+        const int key = key_base + 8 * (r / 4) + 4 * half + r % 4;
+        if ((CAUSAL && key > qrow) || key >= S) s[r] = -INFINITY;
+      }
     }
-    // ---- online softmax
     float mx = -INFINITY;
 #pragma unroll
-    for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[jt][r]);
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
     mx = fmaxf(mx, other_half(mx));
-    const float m_new = fmaxf(m_i, mx * scale_log2e);
-    const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
-    float p[2][16];
-    float sum = 0.0f;
-#pragma unroll
-    for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        p[jt][r] = __builtin_amdgcn_exp2f(fmaf(s[jt][r], scale_log2e, -m_new));
-        sum += p[jt][r];
-      }
-    l_i = l_i * alpha + sum;
-    m_i = m_new;
-    // rescale the output accumulator only when some row of this wave raised its maximum (wave-uniform test)
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+    const float m_blk = mx * scale_log2e;
+    const bool grow = m_blk > m_i + kRescaleLag;
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float m_new = grow ? m_blk : m_i;
+      const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_new) : 1.0f;
+      l_i *= alpha;
+      m_i = m_new;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
     }
-    // ---- O^T += V^T P^T. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
-    //      which is score register hf*8 + e of this lane.
+    float p[16];
+    float sum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, -m_i));
+      sum += p[r];
+    }
+    l_i += sum;
+    pf[0] = MfmaT<T>::pack(&p[0]);
+    pf[1] = MfmaT<T>::pack(&p[8]);
+  };
+  // O^T += V^T P^T for one 32-key tile. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
+  // which is score register hf*8 + e of this lane, so the packed probabilities are used as they are.
+  auto pv_tile = [&](const T* v_src, int jt, const Frag* pf) {
     const int g = lane / 16, i16 = lane % 16;
 #pragma unroll
-    for (int jt = 0; jt < 2; ++jt)
+    for (int hf = 0; hf < 2; ++hf) {
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        Frag pf = MfmaT<T>::pack(&p[jt][hf * 8]);
+      for (int dt = 0; dt < DT; ++dt) {
+        union { i16x4 h[2]; Frag f; } vf;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          union { i16x4 h[2]; Frag f; } vf;
-#pragma unroll
-          for (int pp = 0; pp < 2; ++pp) {
-            const int row = jt * 32 + hf * 16 + 8 * pp + 4 * (g >> 1) + (i16 >> 2);
-            const int col = dt * 32 + (g & 1) * 16 + (i16 & 3) * 4;
-            const int c = (col / 8) ^ swz_vtile<D>(row);
-            const T* addr = v_src + (row * CPR + c) * 8 + (col % 8);
-            vf.h[pp] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
-          }
-          o_acc[dt] = MfmaT<T>::run(vf.f, pf, o_acc[dt]);
+        for (int pp = 0; pp < 2; ++pp) {
+          const int row = jt * 32 + hf * 16 + 8 * pp + 4 * (g >> 1) + (i16 >> 2);
+          const int col = dt * 32 + (g & 1) * 16 + (i16 & 3) * 4;
+          const int c = (col / 8) ^ swz_vtile<D>(row);
+          const T* addr = v_src + (row * CPR + c) * 8 + (col % 8);
+          vf.h[pp] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
         }
+        o_acc[dt] = MfmaT<T>::run(vf.f, pf[hf], o_acc[dt]);
       }
+    }
+  };
+
+  auto process = [&](int step, const T* k_src, const T* v_src) {
+    const int n0 = step * kBlockN;
+    // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4], one MFMA chain per 32-key tile
+    f32x16 s[2];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[jt][r] = 0.0f;
+      const int krow = jt * 32 + lane % 32;
+#pragma unroll
+      for (int ds = 0; ds < DS; ++ds) {
+        const int c = (ds * 2 + half) ^ swz_ktile<D>(krow);
+        Frag kf = *reinterpret_cast<const Frag*>(k_src + (krow * CPR + c) * 8);
+        s[jt] = MfmaT<T>::run(kf, qf[ds], s[jt]);
+      }
+    }
+    // The softmax of tile 0 runs on the vector ALUs while the matrix cores finish the scores of tile 1, and the
+    // softmax of tile 1 while they accumulate P V of tile 0.
+    const bool need_mask = (CAUSAL && n0 + kBlockN - 1 > q0) || (n0 + kBlockN > S);
+    Frag pf[4];
+    softmax_tile(n0, need_mask, s[0], &pf[0]);
+    pv_tile(v_src, 0, &pf[0]);
+    softmax_tile(n0 + 32, need_mask, s[1], &pf[2]);
+    pv_tile(v_src, 1, &pf[2]);
   };
 
   load_kv(0, k_lds0, v_lds0);
