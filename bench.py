@@ -233,20 +233,40 @@ ALIASES = {"norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "
            "layer_norm": "layer_norm_f16_8192x4096"}
 
 
-def measure(torch, wl, steps, warmup):
-    """Returns ms per step from HIP events around `steps` launches on the current stream."""
+def measure(torch, wl, steps, warmup, use_graph=True):
+    """ms per step from HIP events around `steps` steps on the current stream.
+
+    The steps are captured once into a HIP graph and replayed, so the figure is the GPU's time for back-to-back
+    launches and not the host's launch cadence (a Python -> ctypes launch costs more than the shortest kernels
+    here run). Falls back to direct launches if capture is unavailable."""
     for i in range(warmup):
         wl.step(i)
     torch.cuda.synchronize()
+    graph = None
+    if use_graph:
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(steps):
+                    wl.step(warmup + i)
+            graph.replay()                              # untimed: first replay pays the upload
+            torch.cuda.synchronize()
+        except Exception as exc:                        # noqa: BLE001 - report and fall back
+            print("# graph capture failed (%s); timing direct launches" % exc, file=sys.stderr)
+            graph = None
+            torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for i in range(steps):
-        wl.step(warmup + i)
+    if graph is not None:
+        graph.replay()
+    else:
+        for i in range(steps):
+            wl.step(warmup + i)
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return e0.elapsed_time(e1) / steps, wall_ms
+    return e0.elapsed_time(e1) / steps, wall_ms, graph is not None
 
 
 def report(wl, ms):
@@ -272,6 +292,7 @@ def main():
     ap.add_argument("--workload", default="norms")
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time direct launches instead of a HIP graph replay")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -289,7 +310,7 @@ def main():
     wls = make_workloads()
     primary = wls[ALIASES.get(args.workload, args.workload)]
     primary.setup(torch, hexmi)
-    ms, wall_ms = measure(torch, primary, args.steps, args.warmup)
+    ms, wall_ms, graphed = measure(torch, primary, args.steps, args.warmup, not args.no_graph)
     roof = report(primary, ms)
     unit = roof["unit"]
     line = {
@@ -298,7 +319,8 @@ def main():
         "ms_per_step": round(ms, 5), "wall_ms_per_step": round(wall_ms, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": primary.dtype, "data": "synthetic",
         "config": {"workload": primary.name, "description": primary.desc,
-                   "buffers": "%d rotated sets" % len(primary.sets)},
+                   "buffers": "%d rotated sets" % len(primary.sets),
+                   "launch": "hip graph replay" if graphed else "direct"},
         "roofline": roof,
     }
     if not args.no_cpu:
@@ -317,7 +339,7 @@ def main():
             print("# measuring %s" % name, file=sys.stderr, flush=True)
             wl.setup(torch, hexmi)
             k = steps_for(wl, args.steps)
-            wms, _ = measure(torch, wl, k, args.warmup)
+            wms, _, _ = measure(torch, wl, k, args.warmup, not args.no_graph)
             entry = {"workload": name, "ms": round(wms, 5), "steps": k}
             entry.update(report(wl, wms))
             if not args.no_cpu:

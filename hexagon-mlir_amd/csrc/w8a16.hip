@@ -10,17 +10,15 @@
 // The per-channel scale multiplies the finished fp32 sum (it is constant over k), which differs from
 // "dequantise, then multiply" only by fp32 rounding; hexmi_dequant_w8 exposes the element-wise dequantisation.
 //
-// Work split: a workgroup of 8 waves owns one tile of 16 output channels at a time; the waves split K eight ways
-// and their partial tiles are summed through LDS. Activations are staged in LDS once per workgroup when they
-// fit (16*MT rows x K fp16 <= 128 KiB), otherwise fragments are read through L2.
+// Work split: a workgroup of 4 waves owns one tile of 16 output channels; the waves split K four ways and their
+// partial tiles are summed through LDS.
 #include "hexmi_common.h"
 
 namespace hexmi {
 namespace {
 
-constexpr int kWaves = 8;
+constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * kWave;
-constexpr int kALdsBytes = 144 * 1024;     // LDS a workgroup may take for activations + reduction (of 160 KiB)
 
 // 4 int8 (one dword) -> 4 fp16 in two dwords, exact.
 __device__ __forceinline__ void cvt4(uint32_t w, uint32_t& lo, uint32_t& hi) {
@@ -46,104 +44,157 @@ __device__ __forceinline__ void cvt16(const u32x4& w, f16x8& f0, f16x8& f1) {
   f1 = b.f;
 }
 
+// One workgroup (4 waves) per tile of 16 output channels; wave w owns the K range [w*K/4, (w+1)*K/4) in steps of
+// 64 (one 16-byte weight load per lane = two MFMAs). All weight loads of a round are issued before the first
+// conversion so a wave keeps up to 8 KiB of the weight stream in flight; with every tile a separate workgroup
+// the whole grid is resident at once and nothing synchronises across tiles. Activation fragments are read
+// through L1/L2 (the activations are M*K*2 bytes, at most 128 KiB per 16 rows, shared by every workgroup).
 // MT: number of 16-row activation tiles handled per pass (rows m_base .. m_base + 16*MT).
-template <int MT, bool A_IN_LDS>
+template <int MT>
 __global__ __launch_bounds__(kThreads)
 void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
-                  f16* __restrict__ C, int M, int N, int K, int m_base, int n_tiles) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  // [16*MT][K + 8] when A_IN_LDS: the 16-byte pad per row moves consecutive rows to consecutive bank groups
-  f16* a_lds = reinterpret_cast<f16*>(smem);
-  const int KP = K + 8;
-  float* red = reinterpret_cast<float*>(smem + (A_IN_LDS ? (size_t)16 * MT * KP * 2 : 0));   // [kWaves][MT][256]
+                  f16* __restrict__ C, int M, int N, int K, int m_base) {
+  __shared__ __attribute__((aligned(16))) float red[kWaves * MT * 256];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int r16 = lane % 16, kg = lane / 16;                               // tile row / 16-byte k group of this lane
+  const int r16 = lane % 16, kg = lane / 16;               // tile row / 16-byte k group of this lane
+  const int tile = blockIdx.x;
+  const int n = tile * 16 + r16;
+  const int nc = n < N ? n : N - 1;
+  const int8_t* wrow = W + (int64_t)nc * K + kg * 16;
 
-  if constexpr (A_IN_LDS) {
-    const int chunks_per_row = K / 8;
-    for (int idx = threadIdx.x; idx < 16 * MT * chunks_per_row; idx += kThreads) {
-      const int r = idx / chunks_per_row, c = idx % chunks_per_row;
-      const int gm = m_base + r;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (gm < M) v = *reinterpret_cast<const u32x4*>(A + (int64_t)gm * K + c * 8);
-      *reinterpret_cast<u32x4*>(a_lds + (int64_t)r * KP + c * 8) = v;
-    }
-    __syncthreads();
+  const int steps = K / 64;
+  const int per_wave = (steps + kWaves - 1) / kWaves;       // consecutive steps per wave: whole 128-byte lines
+  const int s_begin = wave * per_wave;
+  const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
+
+  const f16* arow[MT];
+  bool avalid[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int gm = m_base + t * 16 + r16;
+    avalid[t] = gm < M;
+    arow[t] = A + (int64_t)(avalid[t] ? gm : 0) * K + kg * 16;
   }
 
-  // K is cut into 64-wide steps (one 16-byte weight load per lane = two MFMAs). A wave takes steps in
-  // adjacent pairs so that its loads cover whole 128-byte lines of each weight row: pair p = steps 2p, 2p+1,
-  // wave w owns pairs w, w+8, ...
-  const int steps = K / 64;
-  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-    const int n = tile * 16 + r16;
-    const int nc = n < N ? n : N - 1;
-    const int8_t* wrow = W + (int64_t)nc * K + kg * 16;
-    f32x4 acc[MT];
+  f32x4 acc[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int p0 = wave; 2 * p0 < steps; p0 += kWaves * 2) {
-      u32x4 wv[4];
+  // A round issues U weight loads and the 2*U*MT activation loads that go with them before anything is
+  // consumed, so the HBM latency of the weights and the L2 latency of the activations overlap.
+  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
+  for (int s0 = s_begin; s0 < s_end; s0 += U) {
+    u32x4 wv[U];
+    f16x8 av[U][MT][2];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int s = 2 * (p0 + (u / 2) * kWaves) + (u % 2);
-        wv[u] = u32x4{0u, 0u, 0u, 0u};
-        if (s < steps) wv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + (int64_t)s * 64));
-      }
+    for (int u = 0; u < U; ++u) {
+      wv[u] = u32x4{0u, 0u, 0u, 0u};
+      if (s0 + u < s_end) wv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + (int64_t)(s0 + u) * 64));
+    }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int s = 2 * (p0 + (u / 2) * kWaves) + (u % 2);
-        if (s < steps) {
-          f16x8 w0, w1;
-          cvt16(wv[u], w0, w1);
-          const int k = s * 64 + kg * 16;
+    for (int u = 0; u < U; ++u) {
+      const int k = (s0 + u) * 64;
 #pragma unroll
-          for (int t = 0; t < MT; ++t) {
-            f16x8 a0, a1;
-            if constexpr (A_IN_LDS) {
-              const f16* ap = a_lds + (int64_t)(t * 16 + r16) * KP + k;
-              a0 = *reinterpret_cast<const f16x8*>(ap);
-              a1 = *reinterpret_cast<const f16x8*>(ap + 8);
-            } else {
-              const int gm = m_base + t * 16 + r16;
-              if (gm < M) {
-                const f16* ap = A + (int64_t)gm * K + k;
-                a0 = *reinterpret_cast<const f16x8*>(ap);
-                a1 = *reinterpret_cast<const f16x8*>(ap + 8);
-              } else {
-                a0 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-                a1 = a0;
-              }
-            }
-            // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, a0, acc[t], 0, 0, 0);
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, a1, acc[t], 0, 0, 0);
-          }
+      for (int t = 0; t < MT; ++t) {
+        av[u][t][0] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        av[u][t][1] = av[u][t][0];
+        if (avalid[t] && s0 + u < s_end) {
+          av[u][t][0] = *reinterpret_cast<const f16x8*>(arow[t] + k);
+          av[u][t][1] = *reinterpret_cast<const f16x8*>(arow[t] + k + 8);
         }
       }
     }
-
-    // sum the K-partials of the 8 waves
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
-      *reinterpret_cast<f32x4*>(red + ((wave * MT + t) * 64 + lane) * 4) = acc[t];
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < MT * 64; idx += kThreads) {
-      const int t = idx / 64, l = idx % 64;
-      f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < U; ++u) {
+      f16x8 w0, w1;
+      cvt16(wv[u], w0, w1);                                 // a skipped step has zero weights and activations
 #pragma unroll
-      for (int w = 0; w < kWaves; ++w) sum += *reinterpret_cast<const f32x4*>(red + ((w * MT + t) * 64 + l) * 4);
-      const int gm = m_base + t * 16 + l % 16;
-      const int gn = tile * 16 + (l / 16) * 4;
-      if (gm < M) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (gn + e < N) C[(int64_t)gm * N + gn + e] = (f16)(sum[e] * (float)scales[gn + e]);
+      for (int t = 0; t < MT; ++t) {
+        // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, av[u][t][0], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, av[u][t][1], acc[t], 0, 0, 0);
       }
     }
-    __syncthreads();
+  }
+
+  // sum the K-partials of the waves
+#pragma unroll
+  for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4*>(red + ((wave * MT + t) * 64 + lane) * 4) = acc[t];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < MT * 64; idx += kThreads) {
+    const int t = idx / 64, l = idx % 64;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sum += *reinterpret_cast<const f32x4*>(red + ((w * MT + t) * 64 + l) * 4);
+    const int gm = m_base + t * 16 + l % 16;
+    const int gn = tile * 16 + (l / 16) * 4;
+    if (gm < M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (gn + e < N) C[(int64_t)gm * N + gn + e] = (f16)(sum[e] * (float)scales[gn + e]);
+    }
+  }
+}
+
+// Up to four activation rows (decode): no matrix cores. A wave owns RPW consecutive output channels and reads
+// each 4 KiB-aligned weight row with fully contiguous 16-byte loads (lane i takes bytes [1024*j + 16*i, +16) of
+// the row for j = 0..K/1024), all RPW rows in flight at once; the activations a lane needs (the same k for every
+// row) sit in registers as fp16 pairs. Products are v_dot2_f32_f16 (two exact fp16 products added into an fp32
+// accumulator), the 64 lane partials are summed with a butterfly, and lane 0 applies the channel scale.
+template <int MR, int RPW, int KJ>                          // KJ = K / 1024: 16-byte loads per lane per row
+__global__ __launch_bounds__(256)
+void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
+                       f16* __restrict__ C, int M, int N, int K) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n0 = (blockIdx.x * 4 + wave) * RPW;
+  if (n0 >= N) return;
+
+  u32x4 wv[RPW][KJ];
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    const int n = n0 + r < N ? n0 + r : N - 1;
+    const int8_t* wrow = W + (int64_t)n * K + lane * 16;
+#pragma unroll
+    for (int j = 0; j < KJ; ++j) wv[r][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + j * 1024));
+  }
+  // activations: lane needs k in [1024*j + 16*lane, +16) for every j: two 16-byte loads per (row, j)
+  f16x8 av[MR][KJ][2];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    const f16* arow = A + (int64_t)(m < M ? m : 0) * K + lane * 16;
+#pragma unroll
+    for (int j = 0; j < KJ; ++j) {
+      av[m][j][0] = *reinterpret_cast<const f16x8*>(arow + j * 1024);
+      av[m][j][1] = *reinterpret_cast<const f16x8*>(arow + j * 1024 + 8);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    float acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < KJ; ++j) {
+      f16x8 w0, w1;
+      cvt16(wv[r][j], w0, w1);
+#pragma unroll
+      for (int m = 0; m < MR; ++m) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc[m] = __builtin_amdgcn_fdot2(f16x2{w0[2 * e], w0[2 * e + 1]}, f16x2{av[m][j][0][2 * e], av[m][j][0][2 * e + 1]},
+                                          acc[m], false);
+          acc[m] = __builtin_amdgcn_fdot2(f16x2{w1[2 * e], w1[2 * e + 1]}, f16x2{av[m][j][1][2 * e], av[m][j][1][2 * e + 1]},
+                                          acc[m], false);
+        }
+      }
+    }
+    const int n = n0 + r;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const float tot = wave_sum(acc[m]);
+      if (lane == 0 && n < N && m < M) C[(int64_t)m * N + n] = (f16)(tot * (float)scales[n]);
+    }
   }
 }
 
@@ -158,24 +209,10 @@ void dequant_kernel(const int8_t* __restrict__ W, const f16* __restrict__ scales
 }
 
 template <int MT>
-int launch_pass(const f16* A, const int8_t* W, const f16* s, f16* C, int M, int N, int K, int m_base, int cus,
+int launch_pass(const f16* A, const int8_t* W, const f16* s, f16* C, int M, int N, int K, int m_base,
                 hipStream_t st) {
   const int n_tiles = (N + 15) / 16;
-  const size_t a_bytes = (size_t)16 * MT * (K + 8) * 2;
-  const size_t red_bytes = (size_t)kWaves * MT * 256 * 4;
-  const bool in_lds = a_bytes + red_bytes <= (size_t)kALdsBytes;
-  int grid = n_tiles < cus * 2 ? n_tiles : cus * 2;
-  if (in_lds) {
-    if (grid > cus) grid = cus;                       // one resident workgroup per CU (LDS bound)
-    auto kern = w8a16_kernel<MT, true>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)(a_bytes + red_bytes)) != hipSuccess)
-      return HEXMI_ELAUNCH;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), a_bytes + red_bytes, st, A, W, s, C, M, N, K, m_base, n_tiles);
-  } else {
-    hipLaunchKernelGGL((w8a16_kernel<MT, false>), dim3(grid), dim3(kThreads), red_bytes, st, A, W, s, C, M, N, K,
-                       m_base, n_tiles);
-  }
+  hipLaunchKernelGGL((w8a16_kernel<MT>), dim3(n_tiles), dim3(kThreads), 0, st, A, W, s, C, M, N, K, m_base);
   return launch_status();
 }
 
@@ -192,18 +229,26 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
   if (K == 0 || K % 64 != 0) return HEXMI_ENOTSUP;    // 16-byte weight loads, 64-wide K steps
   if (!aligned_to(A, 16) || !aligned_to(W, 16)) return HEXMI_EINVAL;
   if (M > 0x7fffffff || N > 0x7fffffff - 16 || K > 0x7fffffff) return HEXMI_ENOTSUP;
-  int cus = hexmi_num_cus();
-  if (cus <= 0) return HEXMI_ELAUNCH;
   hipStream_t st = as_stream(stream);
   const f16* a = static_cast<const f16*>(A);
   const f16* s = static_cast<const f16*>(scales);
   f16* c = static_cast<f16*>(C);
+  if ((M <= 4 && (K == 1024 || K == 2048 || K == 4096)) || (M <= 2 && K == 8192)) {
+    constexpr int RPW = 2;
+    const unsigned blocks = (unsigned)((N + 4 * RPW - 1) / (4 * RPW));
+#define HEXMI_GEMV(MR, KJ) hipLaunchKernelGGL((w8a16_gemv_kernel<MR, RPW, KJ>), dim3(blocks), dim3(256), 0, st, a, W, s, c, (int)M, (int)N, (int)K)
+#define HEXMI_GEMV_K(MR) { if (K == 1024) HEXMI_GEMV(MR, 1); else if (K == 2048) HEXMI_GEMV(MR, 2); else if (K == 4096) HEXMI_GEMV(MR, 4); else HEXMI_GEMV(MR, 8); }
+    if (M == 1) HEXMI_GEMV_K(1) else if (M == 2) HEXMI_GEMV_K(2) else { if (K == 1024) HEXMI_GEMV(4, 1); else if (K == 2048) HEXMI_GEMV(4, 2); else HEXMI_GEMV(4, 4); }
+#undef HEXMI_GEMV_K
+#undef HEXMI_GEMV
+    return launch_status();
+  }
   int rc = HEXMI_OK;
   for (int64_t m = 0; m < M && rc == HEXMI_OK; m += 64) {
     const int64_t left = M - m;
-    if (left > 32) rc = launch_pass<4>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, cus, st);
-    else if (left > 16) rc = launch_pass<2>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, cus, st);
-    else rc = launch_pass<1>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, cus, st);
+    if (left > 32) rc = launch_pass<4>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
+    else if (left > 16) rc = launch_pass<2>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
+    else rc = launch_pass<1>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
   }
   return rc;
 }
