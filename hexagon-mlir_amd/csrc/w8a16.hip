@@ -137,7 +137,89 @@ void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const
   }
 }
 
-// Up to four activation rows (decode): no matrix cores. A wave owns RPW consecutive output channels and reads
+// Up to 16 activation rows, K <= 4096: persistent workgroups of 16 waves, one per compute unit. The per-CU rate
+// of the 16-row strided weight reads is what bounds this shape, so the channel tiles are dealt round-robin over
+// exactly as many workgroups as there are CUs (workgroup b owns tiles b, b+G, b+2G). Wave w owns the K slice
+// [w*K/16, (w+1)*K/16) of every tile of its workgroup: it needs only a 16 x K/16 slice of the activations, which
+// it keeps in registers for all its tiles (no LDS staging, activations cross L2 once per workgroup), and it
+// issues the weight loads of all its tiles up front so the whole weight matrix is requested at kernel start.
+// The 16 K-partials of a tile are summed through LDS.
+constexpr int kPWaves = 16;
+constexpr int kPTiles = 3;                                  // tiles per workgroup per pass
+constexpr int kPSteps = 4;                                  // 64-wide steps per wave: K <= 16 * 4 * 64
+__global__ __launch_bounds__(1024)
+void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
+                          f16* __restrict__ C, int M, int N, int K, int n_tiles) {
+  __shared__ __attribute__((aligned(16))) float red[kPTiles * kPWaves * 256];   // [slot][wave][lane][4]
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int r16 = lane % 16, kg = lane / 16;
+  const int ksl = K / kPWaves;                              // K slice of a wave
+  const int steps = ksl / 64;                               // <= kPSteps
+  const int G = gridDim.x;
+
+  for (int t0 = blockIdx.x; t0 < n_tiles; t0 += kPTiles * G) {
+    // weights first: all tiles of this pass, every step
+    u32x4 wv[kPTiles][kPSteps];
+#pragma unroll
+    for (int q = 0; q < kPTiles; ++q) {
+      const int tile = t0 + q * G;
+      int n = (tile < n_tiles ? tile : t0) * 16 + r16;      // an absent tile re-reads the first one, unused
+      n = n < N ? n : N - 1;
+      const int8_t* wrow = W + (int64_t)n * K + (int64_t)wave * ksl + kg * 16;
+#pragma unroll
+      for (int u = 0; u < kPSteps; ++u) {
+        const int st = u < steps ? u : steps - 1;
+        wv[q][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + st * 64));
+      }
+    }
+    // this wave's activation slice: rows r16, k in [wave*ksl + u*64 + kg*16, +16)
+    f16x8 av[kPSteps][2];
+    {
+      const f16* arow = A + (int64_t)(r16 < M ? r16 : 0) * K + (int64_t)wave * ksl + kg * 16;
+#pragma unroll
+      for (int u = 0; u < kPSteps; ++u) {
+        const int st = u < steps ? u : steps - 1;
+        av[u][0] = *reinterpret_cast<const f16x8*>(arow + st * 64);
+        av[u][1] = *reinterpret_cast<const f16x8*>(arow + st * 64 + 8);
+        if (r16 >= M) {
+          av[u][0] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+          av[u][1] = av[u][0];
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < kPTiles; ++q) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < kPSteps; ++u) {
+        if (u < steps) {                                    // wave-uniform
+          f16x8 w0, w1;
+          cvt16(wv[q][u], w0, w1);
+          // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, av[u][0], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, av[u][1], acc, 0, 0, 0);
+        }
+      }
+      *reinterpret_cast<f32x4*>(red + ((q * kPWaves + wave) * 64 + lane) * 4) = acc;
+    }
+    __syncthreads();
+    if (threadIdx.x < kPTiles * 256) {
+      const int q = threadIdx.x / 256, e = threadIdx.x % 256;     // e = lane*4 + element of the accumulator
+      const int tile = t0 + q * G;
+      float sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kPWaves; ++w) sum += red[(q * kPWaves + w) * 256 + e];
+      const int l = e / 4;
+      const int gm = l % 16;
+      const int gn = tile * 16 + (l / 16) * 4 + e % 4;
+      if (tile < n_tiles && gm < M && gn < N) C[(int64_t)gm * N + gn] = (f16)(sum * (float)scales[gn]);
+    }
+    __syncthreads();
+  }
+}
+
+// One or two activation rows (decode): no matrix cores. A wave owns RPW consecutive output channels and reads
 // each 4 KiB-aligned weight row with fully contiguous 16-byte loads (lane i takes bytes [1024*j + 16*i, +16) of
 // the row for j = 0..K/1024), all RPW rows in flight at once; the activations a lane needs (the same k for every
 // row) sit in registers as fp16 pairs. Products are v_dot2_f32_f16 (two exact fp16 products added into an fp32
@@ -233,14 +315,22 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
   const f16* a = static_cast<const f16*>(A);
   const f16* s = static_cast<const f16*>(scales);
   f16* c = static_cast<f16*>(C);
-  if ((M <= 4 && (K == 1024 || K == 2048 || K == 4096)) || (M <= 2 && K == 8192)) {
+  if (M <= 2 && (K == 1024 || K == 2048 || K == 4096 || K == 8192)) {
     constexpr int RPW = 2;
     const unsigned blocks = (unsigned)((N + 4 * RPW - 1) / (4 * RPW));
 #define HEXMI_GEMV(MR, KJ) hipLaunchKernelGGL((w8a16_gemv_kernel<MR, RPW, KJ>), dim3(blocks), dim3(256), 0, st, a, W, s, c, (int)M, (int)N, (int)K)
 #define HEXMI_GEMV_K(MR) { if (K == 1024) HEXMI_GEMV(MR, 1); else if (K == 2048) HEXMI_GEMV(MR, 2); else if (K == 4096) HEXMI_GEMV(MR, 4); else HEXMI_GEMV(MR, 8); }
-    if (M == 1) HEXMI_GEMV_K(1) else if (M == 2) HEXMI_GEMV_K(2) else { if (K == 1024) HEXMI_GEMV(4, 1); else if (K == 2048) HEXMI_GEMV(4, 2); else HEXMI_GEMV(4, 4); }
+    if (M == 1) HEXMI_GEMV_K(1) else HEXMI_GEMV_K(2)
 #undef HEXMI_GEMV_K
 #undef HEXMI_GEMV
+    return launch_status();
+  }
+  if (M <= 16 && K % (kPWaves * 64) == 0 && K / (kPWaves * 64) <= kPSteps) {
+    const int cus = hexmi_num_cus();
+    if (cus <= 0) return HEXMI_ELAUNCH;
+    const int n_tiles = (int)((N + 15) / 16);
+    const int grid = n_tiles < cus ? n_tiles : cus;
+    hipLaunchKernelGGL(w8a16_persist_kernel, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, n_tiles);
     return launch_status();
   }
   int rc = HEXMI_OK;
