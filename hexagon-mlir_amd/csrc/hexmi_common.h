@@ -35,16 +35,50 @@ template <> __device__ __forceinline__ f16 from_f32<f16>(float v) { return (f16)
 template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return (bf16)v; }  // round-to-nearest-even
 
 // ---- wavefront reductions -----------------------------------------------
-// Butterfly over the 64 lanes; every lane ends with the full result.
+// Butterfly over the 64 lanes on the vector ALU (no LDS round trips): DPP exchanges inside a row of 16 lanes
+// (quad permutes for lane^1 and lane^2; the half-row and row mirrors stand in for lane^4 and lane^8 because the
+// partial results are already uniform inside groups of 4 and 8), then v_permlane16_swap / v_permlane32_swap
+// for the exchanges between rows. Every lane ends with the full result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  const int i = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xF, 0xF, false));
+}
+// {a, b} with a = value of the partner row (16 lanes) / half (32 lanes) and b = own, in some order that is the
+// same for both partners up to exchange: callers combine them with a commutative operation.
+__device__ __forceinline__ void swap16(float v, float& a, float& b) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  a = __builtin_bit_cast(float, (unsigned)r[0]);
+  b = __builtin_bit_cast(float, (unsigned)r[1]);
+}
+__device__ __forceinline__ void swap32(float v, float& a, float& b) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  a = __builtin_bit_cast(float, (unsigned)r[0]);
+  b = __builtin_bit_cast(float, (unsigned)r[1]);
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
+  v += dpp_move<0xB1>(v);      // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E>(v);      // quad_perm [2,3,0,1]
+  v += dpp_move<0x141>(v);     // row_half_mirror
+  v += dpp_move<0x140>(v);     // row_mirror
+  float a, b;
+  swap16(v, a, b);
+  v = a + b;
+  swap32(v, a, b);
+  return a + b;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-  return v;
+  v = fmaxf(v, dpp_move<0xB1>(v));
+  v = fmaxf(v, dpp_move<0x4E>(v));
+  v = fmaxf(v, dpp_move<0x141>(v));
+  v = fmaxf(v, dpp_move<0x140>(v));
+  float a, b;
+  swap16(v, a, b);
+  v = fmaxf(a, b);
+  swap32(v, a, b);
+  return fmaxf(a, b);
 }
 
 // ---- host helpers ---------------------------------------------------------

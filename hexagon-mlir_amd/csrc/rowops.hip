@@ -1,10 +1,10 @@
-// Row reductions: softmax, RMSNorm, LayerNorm. Single pass over HBM: a row is
-// loaded once with 16-byte accesses, kept in registers in fp32-convertible
-// form, reduced with wavefront butterflies (and one LDS exchange when a row
-// spans several waves), and stored once.
+// Row reductions: softmax, RMSNorm, LayerNorm. Single pass over HBM: a row is loaded once with 16-byte
+// non-temporal accesses, kept in registers as fp32, reduced with wavefront butterflies (plus one LDS exchange per
+// reduction when a row spans several waves), and stored once.
 //
-//   rows up to 16 KiB : one 64-lane wave per row, no LDS, no barrier
-//   rows up to 128 KiB: one 1024-thread workgroup per row, LDS reduction
+//   rows up to 4 KiB  : one 64-lane wave per row, four rows per workgroup, no LDS, no barrier
+//   rows up to 128 KiB: 256 .. 1024 threads per row with two to eight 16-byte chunks per thread (more, shorter
+//                       waves keep more of HBM busy than one long wave per row)
 //   anything else (or misaligned): generic strided kernel, row re-read from L2
 #include "hexmi_common.h"
 
@@ -39,15 +39,14 @@ __device__ __forceinline__ void store16_stream(T* p, const Vec16<T>& r) {
   __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(r.v), reinterpret_cast<u32x4*>(p));
 }
 
-// Reduce across the waves of a workgroup through LDS. `red` holds one float
-// per wave; every thread returns the combined value.
+// Reduce across the WAVES waves that share a row through LDS. `red` holds one float per wave and must not be
+// reused by another reduction of the same kernel (each reduction gets its own slots, so one barrier suffices);
+// every thread returns the combined value.
 template <bool IS_MAX, int WAVES>
-__device__ __forceinline__ float block_reduce(float v, float* red) {
+__device__ __forceinline__ float block_reduce(float v, float* red, int wave_in_row) {
   v = IS_MAX ? wave_max(v) : wave_sum(v);
   if constexpr (WAVES == 1) return v;
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  __syncthreads();                                  // previous use of `red` finished
-  if (lane == 0) red[wave] = v;
+  if (threadIdx.x % kWave == 0) red[wave_in_row] = v;
   __syncthreads();
   float r = red[0];
 #pragma unroll
@@ -67,10 +66,18 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
                 int64_t rows, int cols, int64_t ld_x, int64_t ld_y, float eps) {
   constexpr int N = Vec16<T>::N;
   constexpr int WAVES = THREADS / kWave;
-  __shared__ float red[WAVES > 1 ? WAVES : 1];
+  __shared__ float red_a[ROWS_PER_BLOCK][WAVES];     // first reduction (max / mean)
+  __shared__ float red_b[ROWS_PER_BLOCK][WAVES];     // second reduction (sum / variance)
   const int t = threadIdx.x % THREADS;
-  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / THREADS;
-  if (row >= rows) return;                          // whole waves leave together (THREADS % 64 == 0)
+  const int row_in_block = threadIdx.x / THREADS;
+  const int wave_in_row = t / kWave;
+  int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + row_in_block;
+  // Rows past the end are computed on the last row and not stored, so every wave reaches the barriers.
+  const bool row_valid = row < rows;
+  if (!row_valid) {
+    if constexpr (WAVES == 1) return;               // no barrier in this configuration: whole waves may leave
+    row = rows - 1;
+  }
 
   const T* xr = x + row * ld_x;
   T* yr = y + row * ld_y;
@@ -94,18 +101,18 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
     for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
       for (int i = 0; i < N; ++i) m = fmaxf(m, v[c][i]);
-    m = block_reduce<true, WAVES>(m, red);
+    m = block_reduce<true, WAVES>(m, red_a[row_in_block], wave_in_row);
     float s = 0.0f;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
       for (int i = 0; i < N; ++i) { v[c][i] = __expf(v[c][i] - m); s += v[c][i]; }
-    s = block_reduce<false, WAVES>(s, red);
+    s = block_reduce<false, WAVES>(s, red_b[row_in_block], wave_in_row);
     const float inv = 1.0f / s;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
       const int col = (c * THREADS + t) * N;
-      if (col < cols) {
+      if (col < cols && row_valid) {
         Vec16<T> o;
 #pragma unroll
         for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i] * inv);
@@ -120,22 +127,21 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
 #pragma unroll
       for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
-        for (int i = 0; i < N; ++i) s += v[c][i];
-      mean = block_reduce<false, WAVES>(s, red) * inv_n;
+        for (int i = 0; i < N; ++i) s += v[c][i];     // masked slots hold 0
+      mean = block_reduce<false, WAVES>(s, red_a[row_in_block], wave_in_row) * inv_n;
     }
     float q = 0.0f;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
-      const int col = (c * THREADS + t) * N;
-      if (col < cols) {
+      if ((c * THREADS + t) * N < cols) {
 #pragma unroll
         for (int i = 0; i < N; ++i) { v[c][i] -= mean; q += v[c][i] * v[c][i]; }
       }
     }
-    q = block_reduce<false, WAVES>(q, red);
+    q = block_reduce<false, WAVES>(q, red_b[row_in_block], wave_in_row);
     const float rstd = 1.0f / sqrtf(q * inv_n + eps);
     if constexpr (OP == kLayerNorm) {
-      if (t == 0) {
+      if (t == 0 && row_valid) {
         if (mean_out) mean_out[row] = mean;
         if (rstd_out) rstd_out[row] = rstd;
       }
@@ -143,7 +149,7 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
       const int col = (c * THREADS + t) * N;
-      if (col < cols) {
+      if (col < cols && row_valid) {
         Vec16<T> o;
         if (w) {
           Vec16<T> wv = load16(w + col);
@@ -174,7 +180,9 @@ void row_kernel_generic(const T* __restrict__ x, T* __restrict__ y, const T* __r
                         const T* __restrict__ b, float* __restrict__ mean_out, float* __restrict__ rstd_out,
                         int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps) {
   constexpr int WAVES = 4;
-  __shared__ float red[WAVES];
+  __shared__ float red_a[WAVES];
+  __shared__ float red_b[WAVES];
+  const int wave_in_row = threadIdx.x / kWave;
   const int64_t row = blockIdx.x;
   const T* xr = x + row * ld_x;
   T* yr = y + row * ld_y;
@@ -182,10 +190,10 @@ void row_kernel_generic(const T* __restrict__ x, T* __restrict__ y, const T* __r
   if constexpr (OP == kSoftmax) {
     float m = -INFINITY;
     for (int64_t i = t; i < cols; i += 256) m = fmaxf(m, to_f32<T>(xr[i]));
-    m = block_reduce<true, WAVES>(m, red);
+    m = block_reduce<true, WAVES>(m, red_a, wave_in_row);
     float s = 0.0f;
     for (int64_t i = t; i < cols; i += 256) s += __expf(to_f32<T>(xr[i]) - m);
-    s = block_reduce<false, WAVES>(s, red);
+    s = block_reduce<false, WAVES>(s, red_b, wave_in_row);
     const float inv = 1.0f / s;
     for (int64_t i = t; i < cols; i += 256) yr[i] = from_f32<T>(__expf(to_f32<T>(xr[i]) - m) * inv);
   } else {
@@ -194,11 +202,11 @@ void row_kernel_generic(const T* __restrict__ x, T* __restrict__ y, const T* __r
     if constexpr (OP == kLayerNorm) {
       float s = 0.0f;
       for (int64_t i = t; i < cols; i += 256) s += to_f32<T>(xr[i]);
-      mean = block_reduce<false, WAVES>(s, red) * inv_n;
+      mean = block_reduce<false, WAVES>(s, red_a, wave_in_row) * inv_n;
     }
     float q = 0.0f;
     for (int64_t i = t; i < cols; i += 256) { float d = to_f32<T>(xr[i]) - mean; q += d * d; }
-    q = block_reduce<false, WAVES>(q, red);
+    q = block_reduce<false, WAVES>(q, red_b, wave_in_row);
     const float rstd = 1.0f / sqrtf(q * inv_n + eps);
     if constexpr (OP == kLayerNorm) {
       if (t == 0) {
@@ -237,12 +245,13 @@ int dispatch_rows(const void* xv, void* yv, const void* wv, const void* bv, floa
   const int64_t chunks = (cols + N - 1) / N;        // 16-byte chunks per row
 #define HEXMI_TILE(C, TH, RPB) return launch_tile<T, OP, C, TH, RPB>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s)
   if (vec_ok && rows <= 0x7fffffff) {
+    // about two to four 16-byte chunks per thread; rows narrower than 4 KiB stay inside one wave (no barrier)
     if (chunks <= 64 * 1) HEXMI_TILE(1, 64, 4);
     if (chunks <= 64 * 2) HEXMI_TILE(2, 64, 4);
     if (chunks <= 64 * 4) HEXMI_TILE(4, 64, 4);
-    if (chunks <= 64 * 8) HEXMI_TILE(8, 64, 4);
+    if (chunks <= 256 * 2) HEXMI_TILE(2, 256, 1);
     if (chunks <= 256 * 4) HEXMI_TILE(4, 256, 1);
-    if (chunks <= 256 * 8) HEXMI_TILE(8, 256, 1);
+    if (chunks <= 512 * 4) HEXMI_TILE(4, 512, 1);
     if (chunks <= 1024 * 4) HEXMI_TILE(4, 1024, 1);
     if (chunks <= 1024 * 8) HEXMI_TILE(8, 1024, 1);
   }

@@ -19,10 +19,10 @@ def _gen(seed):
     return torch.Generator().manual_seed(seed)
 
 
-def _check(got, want, dtype, atol16=1e-6):
+def _check(got, want, dtype, atol16=1e-6, atol32=1e-7):
     got = got.cpu()
     if dtype == torch.float32:
-        assert torch.allclose(got, want, rtol=F32_RTOL, atol=1e-7), (got - want).abs().max()
+        assert torch.allclose(got, want, rtol=F32_RTOL, atol=atol32), (got - want).abs().max()
     else:
         assert close16(got, want, max_ulp=1, atol=atol16)
 
@@ -121,7 +121,7 @@ def test_layer_norm_parity(hexmi, oracle, dtype, shape):
     m = torch.empty(shape[0], device="cuda")
     r = torch.empty(shape[0], device="cuda")
     got = hexmi.layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-5, mean=m, rstd=r)
-    _check(got, want, dtype, atol16=2e-6)
+    _check(got, want, dtype, atol16=2e-6, atol32=2e-6)      # x_hat*w + b near zero carries the rounding of its terms
     assert torch.allclose(m.cpu(), torch.from_numpy(mean), rtol=1e-5, atol=1e-6)
     assert torch.allclose(r.cpu(), torch.from_numpy(rstd), rtol=1e-5)
 
