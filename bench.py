@@ -58,6 +58,28 @@ def _sets(torch, tensors, bytes_per_set, rotate=True):
     return out
 
 
+class CopyCalibration(Workload):
+    """Plain device copy of a known size (64 MiB read + 64 MiB written per step): the reference reading for scaling
+    the FETCH_SIZE / WRITE_SIZE hardware counters to bytes. Not part of the suite."""
+    name, bound, dtype, kernel = "copy_64MiB", "hbm", "u8", "elementwise copy (torch)"
+    desc = "torch Tensor.copy_ of 64 MiB, 5 rotated sets"
+
+    def setup(self, torch, hexmi):
+        n = 64 << 20
+        self.work = 2 * n
+        self.sets = [{"x": torch.zeros(n, dtype=torch.uint8, device="cuda"),
+                      "out": torch.empty(n, dtype=torch.uint8, device="cuda")} for _ in range(5)]
+
+    def step(self, i):
+        s = self.sets[i % len(self.sets)]
+        s["out"].copy_(s["x"])
+
+    def cpu(self, torch):
+        a = torch.zeros(64 << 20, dtype=torch.uint8)
+        b = torch.empty_like(a)
+        return _time_cpu(lambda: b.copy_(a), 3), "64 MiB memcpy on CPU"
+
+
 class Softmax(Workload):
     name, bound, dtype, kernel = "softmax_f32_4096x1024", "hbm", "f32", "row_kernel"
     desc = "row softmax fp32 [4096,1024] N(0,1) seed 0"
@@ -224,10 +246,11 @@ def _time_cpu(fn, iters):
 def make_workloads():
     return {w.name: w for w in (
         Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
-        W8A16(1), W8A16(16), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128))}
+        W8A16(1), W8A16(16), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128),
+        CopyCalibration())}
 
 
-ALIASES = {"norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "gemm": "gemm_f16_4096",
+ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "gemm": "gemm_f16_4096",
            "gemm_bf16": "gemm_bf16_8192", "attn": "attn_causal_f16_4x32x4096x128",
            "attn_long": "attn_causal_f16_1x32x16384x128", "rms_norm": "rms_norm_f16_8192x4096",
            "layer_norm": "layer_norm_f16_8192x4096"}
@@ -269,13 +292,33 @@ def measure(torch, wl, steps, warmup, use_graph=True):
     return e0.elapsed_time(e1) / steps, wall_ms, graph is not None
 
 
+PROFILE_KEYS = {"norms_f16_8192x4096": "norms", "softmax_f32_4096x1024": "softmax", "gemm_f16_4096": "gemm",
+                "gemm_bf16_8192": "gemm_bf16", "w8a16_m1": "w8a16_m1", "w8a16_m16": "w8a16_m16",
+                "w8a16_m256": "w8a16_m256", "attn_causal_f16_4x32x4096x128": "attn",
+                "attn_causal_f16_1x32x16384x128": "attn_long"}
+
+
+def measured_traffic(wl):
+    """HBM bytes per step from the committed rocprofv3 counter runs (profiles/traffic.json), or None."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            table = json.load(f)["traffic"]
+        per_kernel = table[PROFILE_KEYS[wl.name]]
+        if wl.name == "w8a16_m256":                       # four passes of the same kernel per step
+            return 4 * sum(per_kernel.values())
+        return sum(per_kernel.values())
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def report(wl, ms):
     if wl.bound == "hbm":
         achieved, peak, unit = wl.work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
     else:
         achieved, peak, unit = wl.work / (ms * 1e-3) / 1e12, MFMA_PEAK_TFLOPS, "TFLOP/s"
     return {"bound": wl.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": None, "kernel": wl.kernel, "work_per_step": wl.work}
+            "frac": round(achieved / peak, 4), "traffic": measured_traffic(wl), "kernel": wl.kernel,
+            "work_per_step": wl.work}
 
 
 def steps_for(wl, steps):
@@ -334,7 +377,7 @@ def main():
     if not args.no_suite:
         suite = []
         for name, wl in wls.items():
-            if wl is primary or name in ("norms_f16_8192x4096",):
+            if wl is primary or name in ("norms_f16_8192x4096", "copy_64MiB"):
                 continue
             print("# measuring %s" % name, file=sys.stderr, flush=True)
             wl.setup(torch, hexmi)

@@ -128,8 +128,17 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
 
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int nqb = (S + kBlockM - 1) / kBlockM;
-  const int zh = blockIdx.x % ZH;
-  const int qb = nqb - 1 - blockIdx.x / ZH;          // longest rows first
+  // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each). Give every XCD whole heads and let it walk
+  // them one after the other, longest query blocks first, so the K/V of the head in progress stays in its L2.
+  int zh, qb;
+  if (ZH % 8 == 0) {
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    zh = xcd + 8 * (slot / nqb);
+    qb = nqb - 1 - slot % nqb;
+  } else {
+    zh = blockIdx.x % ZH;
+    qb = nqb - 1 - blockIdx.x / ZH;
+  }
   const int64_t base = (int64_t)zh * S * D;
   const T* q_g = Q + base;
   const T* k_g = K + base;
