@@ -103,6 +103,55 @@ struct NMajorLoader {
   }
 };
 
+// Weight-only quantised B: a [ROWS x 32] int8 K-contiguous slab is copied global -> LDS raw (16-byte chunk
+// (row, half) at linear position row*2 + half, no swizzle), and one slab later converted LDS -> LDS into the same
+// swizzled fp16 K-contiguous tile a global_load_lds copy of fp16 data would have filled. All global traffic stays
+// on the asynchronous copy path, so one in-order counter paces A and B alike.
+template <int ROWS>
+struct I8Loader {
+  static constexpr int NI = ROWS / 128 > 0 ? ROWS / 128 : 1;   // copy instructions per wave per slab
+  static constexpr int NC = ROWS * 2 / 256;                    // 16-byte chunks converted per thread per slab
+  const int8_t* ptr[NI];
+  int raw_off[NI];
+  int cv_raw[NC];                                             // raw byte offset of this thread's chunk
+  int cv_el[NC][2];                                           // fp16 element offsets of the two chunks it expands to
+  __device__ __forceinline__ void init(const int8_t* g, int64_t ld, int row0, int row_max, int wave, int lane,
+                                       int tid) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int inst = j * 4 + wave;
+      const int idx = inst * 64 + lane;
+      const int row = idx / 2, half = idx % 2;
+      int grow = row0 + row;
+      grow = grow < row_max ? grow : row_max;
+      ptr[j] = g + (int64_t)grow * ld + half * 16;
+      raw_off[j] = inst * 64 * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      const int idx = j * 256 + tid;
+      const int row = idx / 2, half = idx % 2;
+      cv_raw[j] = idx * 16;
+      cv_el[j][0] = row * BK + (((half * 2 + 0) ^ swz_k(row)) * kChunk);
+      cv_el[j][1] = row * BK + (((half * 2 + 1) ^ swz_k(row)) * kChunk);
+    }
+  }
+  template <int J> __device__ __forceinline__ void issue(int8_t* raw, int k0) const {
+    if constexpr (J < NI)
+      __builtin_amdgcn_global_load_lds(HEXMI_GLB(ptr[J] + k0), HEXMI_LDS(raw + raw_off[J]), 16, 0, 0);
+  }
+  __device__ __forceinline__ void convert(const int8_t* raw, f16* lds) const {
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      const u32x4 r = *reinterpret_cast<const u32x4*>(raw + cv_raw[j]);
+      f16x8 w0, w1;
+      cvt16(r, w0, w1);
+      *reinterpret_cast<f16x8*>(lds + cv_el[j][0]) = w0;
+      *reinterpret_cast<f16x8*>(lds + cv_el[j][1]) = w1;
+    }
+  }
+};
+
 template <typename T>
 __device__ __forceinline__ typename Mfma<T>::Frag read_kmajor(const T* lds, int row, int chunk) {
   typedef typename Mfma<T>::Frag Frag;
@@ -160,10 +209,14 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
 }
 
 // K % 32 == 0. TAIL: the slab count is not a multiple of 4, so the last pass over the four stages guards its MFMAs.
-template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL>
+// B_I8: B is int8 [N,K] (weight-only quantisation, needs TRANS_B and T = fp16); its slabs are copied raw into
+// LDS, converted to fp16 LDS -> LDS one slab later, and the result is multiplied by scales[column].
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false>
 __global__ __launch_bounds__(256)
-void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restrict__ C, int M, int N, int K,
-                 int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n) {
+void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __restrict__ C, int M, int N, int K,
+                 int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
+                 const f16* __restrict__ scales = nullptr) {
+  const T* B = static_cast<const T*>(Bv);
   typedef typename Mfma<T>::Frag Frag;
   constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
   __shared__ __attribute__((aligned(16))) T a_s0[BM * BK];
@@ -174,6 +227,11 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
   __shared__ __attribute__((aligned(16))) T b_s1[BN * BK];
   __shared__ __attribute__((aligned(16))) T b_s2[BN * BK];
   __shared__ __attribute__((aligned(16))) T b_s3[BN * BK];
+  // raw int8 B slabs on their way to fp16 (weight-only quantised B only)
+  __shared__ __attribute__((aligned(16))) int8_t r_s0[B_I8 ? BN * BK : 16];
+  __shared__ __attribute__((aligned(16))) int8_t r_s1[B_I8 ? BN * BK : 16];
+  __shared__ __attribute__((aligned(16))) int8_t r_s2[B_I8 ? BN * BK : 16];
+  __shared__ __attribute__((aligned(16))) int8_t r_s3[B_I8 ? BN * BK : 16];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int wm = wave / 2, wn = wave % 2;
@@ -193,9 +251,12 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
   load_a.init(A, lda, m0, M - 1, wave, lane);
   KMajorLoader<T, BN> load_bk;
   NMajorLoader<T, BN> load_bn;
-  if constexpr (TRANS_B) load_bk.init(B, ldb, n0, N - 1, wave, lane);
+  I8Loader<BN> load_b8;
+  if constexpr (B_I8) load_b8.init(static_cast<const int8_t*>(Bv), ldb, n0, N - 1, wave, lane, threadIdx.x);
+  else if constexpr (TRANS_B) load_bk.init(B, ldb, n0, N - 1, wave, lane);
   else load_bn.init(B, ldb, n0, N - kChunk, wave, lane);
-  constexpr int NLA = BM / 64, NLB = BN / 64;       // copy instructions per wave per slab
+  constexpr int NLA = BM / 64;                      // copy instructions per wave per slab (A)
+  constexpr int NLB = B_I8 ? I8Loader<BN>::NI : BN / 64;   // B copies per wave per slab
 
   // part 0 = the A copies of slab kt, part 1 = its B copies
   auto issue_part = [&](int kt, T* a_dst, T* b_dst, auto part) {
@@ -206,6 +267,8 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
       if constexpr (NLA > 1) load_a.template issue<1>(a_dst, k0);
       if constexpr (NLA > 2) load_a.template issue<2>(a_dst, k0);
       if constexpr (NLA > 3) load_a.template issue<3>(a_dst, k0);
+    } else if constexpr (B_I8) {
+      // nothing: int8 B goes through registers (see the slab body)
     } else if constexpr (TRANS_B) {
       load_bk.template issue<0>(b_dst, k0);
       if constexpr (NLB > 1) load_bk.template issue<1>(b_dst, k0);
@@ -223,7 +286,7 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
     for (int i = 0; i < WM; ++i) af[i] = read_kmajor<T>(a_src, (wm * WM + i) * 32 + lane % 32, ks * 2 + lane / 32);
 #pragma unroll
     for (int j = 0; j < WN; ++j) {
-      if constexpr (TRANS_B) bf[j] = read_kmajor<T>(b_src, (wn * WN + j) * 32 + lane % 32, ks * 2 + lane / 32);
+      if constexpr (TRANS_B || B_I8) bf[j] = read_kmajor<T>(b_src, (wn * WN + j) * 32 + lane % 32, ks * 2 + lane / 32);
       else bf[j] = read_nmajor<T, BN>(b_src, (wn * WN + j) * 32, ks, lane);
     }
   };
@@ -234,7 +297,7 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
       for (int j = 0; j < WN; ++j) acc[i][j] = Mfma<T>::run(bf[j], af[i], acc[i][j]);
   };
   // Pin the issue order of one group (NREAD LDS reads, NV copies, NMFMA MFMAs) in four identical rounds.
-  constexpr int NREAD = WM + (TRANS_B ? WN : 2 * WN);
+  constexpr int NREAD = WM + ((TRANS_B || B_I8) ? WN : 2 * WN);
   constexpr int NMFMA = WM * WN;
   auto interleave = [&](auto nvmem) {
     constexpr int NV = decltype(nvmem)::value;
@@ -259,13 +322,27 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
   std::integral_constant<int, NLB> n_b;
 
   Frag af[2][WM], bf[2][WN];
+  auto issue_raw = [&](int kt, int8_t* raw) {
+    load_b8.template issue<0>(raw, kt * BK);
+    load_b8.template issue<1>(raw, kt * BK);
+  };
   issue_part(0, a_s0, b_s0, part_a);
   issue_part(0, a_s0, b_s0, part_b);
   issue_part(clampk(1), a_s1, b_s1, part_a);
   issue_part(clampk(1), a_s1, b_s1, part_b);
   issue_part(clampk(2), a_s2, b_s2, part_a);
   issue_part(clampk(2), a_s2, b_s2, part_b);
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * L));   // slab 0 landed
+  if constexpr (B_I8) {
+    // raw slabs 0..2 are in flight; 0 and 1 are converted before the loop, 2 by the first slab body
+    issue_raw(0, r_s0);
+    issue_raw(clampk(1), r_s1);
+    issue_raw(clampk(2), r_s2);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(NLB));            // A 0..2 and raw 0, 1 landed
+    __builtin_amdgcn_s_barrier();
+    load_b8.convert(r_s0, reinterpret_cast<f16*>(b_s0));
+    load_b8.convert(r_s1, reinterpret_cast<f16*>(b_s1));
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(B_I8 ? NLB : 2 * L));   // slab 0 landed (and the conversions written)
   __builtin_amdgcn_s_barrier();
   read_frags(a_s0, b_s0, 0, af[0], bf[0]);
 
@@ -274,24 +351,29 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
   // At the barrier in the middle the copies still allowed in flight are slab kt+2 and the A part of slab kt+3,
   // so slab kt+1 has landed for every wave that passes it; every wave has also issued (and, by the lgkmcnt(0)
   // in the same wait, completed) its last LDS read of slab kt, which frees stage kt%4 for the next body.
-#define HEXMI_SLAB(ac, bc, an, bn, afree, bfree, kt)                  \
+  // int8 B: the raw copy of slab kt+3 goes to rfree with the A copies; the barrier in the middle then only lets
+  // this body's own copies stay in flight, so raw slab kt+2 (r2) has landed and is converted into its fp16 stage
+  // b2 in the second half -- a stage freed two barriers ago and first read after the next body's barrier.
+#define HEXMI_SLAB(ac, bc, an, bn, afree, bfree, rfree, r2, b2, kt)   \
   {                                                                   \
     issue_part(clampk((kt) + 3), afree, bfree, part_a);               \
+    if constexpr (B_I8) issue_raw(clampk((kt) + 3), rfree);           \
     read_frags(ac, bc, 1, af[1], bf[1]);                              \
     if (!TAIL || (kt) < KT) mfma_all(af[0], bf[0]);                   \
     interleave(n_a);                                                  \
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(L + NLA));                 \
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(B_I8 ? NLA + NLB : L + NLA));   \
     __builtin_amdgcn_s_barrier();                                     \
     issue_part(clampk((kt) + 3), afree, bfree, part_b);               \
+    if constexpr (B_I8) load_b8.convert(r2, reinterpret_cast<f16*>(b2));   \
     read_frags(an, bn, 0, af[0], bf[0]);                              \
     if (!TAIL || (kt) < KT) mfma_all(af[1], bf[1]);                   \
     interleave(n_b);                                                  \
   }
   for (int kt = 0; kt < KT; kt += 4) {
-    HEXMI_SLAB(a_s0, b_s0, a_s1, b_s1, a_s3, b_s3, kt);
-    HEXMI_SLAB(a_s1, b_s1, a_s2, b_s2, a_s0, b_s0, kt + 1);
-    HEXMI_SLAB(a_s2, b_s2, a_s3, b_s3, a_s1, b_s1, kt + 2);
-    HEXMI_SLAB(a_s3, b_s3, a_s0, b_s0, a_s2, b_s2, kt + 3);
+    HEXMI_SLAB(a_s0, b_s0, a_s1, b_s1, a_s3, b_s3, r_s3, r_s2, b_s2, kt);
+    HEXMI_SLAB(a_s1, b_s1, a_s2, b_s2, a_s0, b_s0, r_s0, r_s3, b_s3, kt + 1);
+    HEXMI_SLAB(a_s2, b_s2, a_s3, b_s3, a_s1, b_s1, r_s1, r_s0, b_s0, kt + 2);
+    HEXMI_SLAB(a_s3, b_s3, a_s0, b_s0, a_s2, b_s2, r_s2, r_s1, b_s1, kt + 3);
   }
 #undef HEXMI_SLAB
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));       // drain the trailing copies before the workgroup's LDS goes away
@@ -306,9 +388,15 @@ void gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, OutT* __restr
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int col = n0 + (wn * WN + j) * 32 + 8 * q + 4 * (lane / 32);
-        if (col < N)
-          store4<OutT>(C + (int64_t)row * ldc + col, acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1],
-                       acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+        if (col < N) {
+          float s0 = 1.0f, s1 = 1.0f, s2 = 1.0f, s3 = 1.0f;
+          if constexpr (B_I8) {
+            const f16x4 sc = *reinterpret_cast<const f16x4*>(scales + col);
+            s0 = (float)sc[0]; s1 = (float)sc[1]; s2 = (float)sc[2]; s3 = (float)sc[3];
+          }
+          store4<OutT>(C + (int64_t)row * ldc + col, acc[i][j][q * 4 + 0] * s0, acc[i][j][q * 4 + 1] * s1,
+                       acc[i][j][q * 4 + 2] * s2, acc[i][j][q * 4 + 3] * s3);
+        }
       }
     }
   }
@@ -397,7 +485,30 @@ int dispatch_trans(bool trans_b, const void* A, const void* B, void* C, int64_t 
                  : dispatch_gemm<T, OutT, false>(A, B, C, M, N, K, lda, ldb, ldc, s);
 }
 
+template <int WM, int WN>
+int launch_w8a16(const f16* A, const int8_t* W, const f16* scales, f16* C, int64_t M, int64_t N, int64_t K,
+                 hipStream_t s) {
+  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+  if ((K / BK) % 4 == 0)
+    hipLaunchKernelGGL((gemm_kernel<f16, f16, WM, WN, true, false, true>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A,
+                       static_cast<const void*>(W), C, (int)M, (int)N, (int)K, K, K, N, tiles_m, tiles_n, scales);
+  else
+    hipLaunchKernelGGL((gemm_kernel<f16, f16, WM, WN, true, true, true>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A,
+                       static_cast<const void*>(W), C, (int)M, (int)N, (int)K, K, K, N, tiles_m, tiles_n, scales);
+  return launch_status();
+}
+
 }  // namespace
+
+// K % 32 == 0, N % 8 == 0, 16-byte aligned A / W / C / scales (checked by the caller).
+int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,
+                     hipStream_t stream) {
+  const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  if (big_tiles >= 128) return launch_w8a16<4, 4>(A, W, scales, C, M, N, K, stream);
+  return launch_w8a16<2, 2>(A, W, scales, C, M, N, K, stream);
+}
+
 }  // namespace hexmi
 
 using namespace hexmi;

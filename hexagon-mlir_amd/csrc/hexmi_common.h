@@ -81,6 +81,33 @@ __device__ __forceinline__ float wave_max(float v) {
   return fmaxf(a, b);
 }
 
+// ---- int8 -> fp16 (weight-only quantisation) --------------------------------
+// int8 -> fp16 is exact: byte b = w ^ 0x80 placed in the low mantissa bits of 0x6400 is the fp16 number
+// 1024 + b, and subtracting 1152 leaves w.
+// 4 int8 (one dword) -> 4 fp16 in two dwords, exact.
+__device__ __forceinline__ void cvt4(uint32_t w, uint32_t& lo, uint32_t& hi) {
+  const uint32_t b = w ^ 0x80808080u;                         // bytes now w + 128 in [1, 255]
+  // v_perm_b32 byte selectors: 0..3 pick bytes of the second source, 4..7 of the first.
+  uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, b, 0x07010700u);   // {0x64, b1, 0x64, b0}
+  uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, b, 0x07030702u);   // {0x64, b3, 0x64, b2}
+  const f16x2 bias = {(f16)1152.0f, (f16)1152.0f};
+  f16x2 h0 = *reinterpret_cast<f16x2*>(&p0) - bias;
+  f16x2 h1 = *reinterpret_cast<f16x2*>(&p1) - bias;
+  lo = *reinterpret_cast<uint32_t*>(&h0);
+  hi = *reinterpret_cast<uint32_t*>(&h1);
+}
+
+// 16 int8 -> two 8-element fp16 fragments (bytes 0..7 and 8..15).
+__device__ __forceinline__ void cvt16(const u32x4& w, f16x8& f0, f16x8& f1) {
+  union { uint32_t u[4]; f16x8 f; } a, b;
+  cvt4(w[0], a.u[0], a.u[1]);
+  cvt4(w[1], a.u[2], a.u[3]);
+  cvt4(w[2], b.u[0], b.u[1]);
+  cvt4(w[3], b.u[2], b.u[3]);
+  f0 = a.f;
+  f1 = b.f;
+}
+
 // ---- host helpers ---------------------------------------------------------
 inline hipStream_t as_stream(hexmi_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
@@ -98,5 +125,9 @@ inline int dtype_size(int dtype) {
     default: return 0;
   }
 }
+
+// Tiled W8A16 GEMM for many activation rows (gemm.hip): C[M,N] = (A[M,K] * W[N,K]^T) * scales[N].
+int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,
+                     hipStream_t stream);
 
 }  // namespace hexmi

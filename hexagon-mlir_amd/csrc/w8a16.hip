@@ -20,30 +20,6 @@ namespace {
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * kWave;
 
-// 4 int8 (one dword) -> 4 fp16 in two dwords, exact.
-__device__ __forceinline__ void cvt4(uint32_t w, uint32_t& lo, uint32_t& hi) {
-  const uint32_t b = w ^ 0x80808080u;                         // bytes now w + 128 in [1, 255]
-  // v_perm_b32 byte selectors: 0..3 pick bytes of the second source, 4..7 of the first.
-  uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, b, 0x07010700u);   // {0x64, b1, 0x64, b0}
-  uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, b, 0x07030702u);   // {0x64, b3, 0x64, b2}
-  const f16x2 bias = {(f16)1152.0f, (f16)1152.0f};
-  f16x2 h0 = *reinterpret_cast<f16x2*>(&p0) - bias;
-  f16x2 h1 = *reinterpret_cast<f16x2*>(&p1) - bias;
-  lo = *reinterpret_cast<uint32_t*>(&h0);
-  hi = *reinterpret_cast<uint32_t*>(&h1);
-}
-
-// 16 int8 -> two 8-element fp16 fragments (bytes 0..7 and 8..15).
-__device__ __forceinline__ void cvt16(const u32x4& w, f16x8& f0, f16x8& f1) {
-  union { uint32_t u[4]; f16x8 f; } a, b;
-  cvt4(w[0], a.u[0], a.u[1]);
-  cvt4(w[1], a.u[2], a.u[3]);
-  cvt4(w[2], b.u[0], b.u[1]);
-  cvt4(w[3], b.u[2], b.u[3]);
-  f0 = a.f;
-  f1 = b.f;
-}
-
 // One workgroup (4 waves) per tile of 16 output channels; wave w owns the K range [w*K/4, (w+1)*K/4) in steps of
 // 64 (one 16-byte weight load per lane = two MFMAs). All weight loads of a round are issued before the first
 // conversion so a wave keeps up to 8 KiB of the weight stream in flight; with every tile a separate workgroup
@@ -333,6 +309,8 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     hipLaunchKernelGGL(w8a16_persist_kernel, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, n_tiles);
     return launch_status();
   }
+  if (M > 64 && K % 32 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8))
+    return gemm_w8a16_tiled(M, N, K, a, W, s, c, st);
   int rc = HEXMI_OK;
   for (int64_t m = 0; m < M && rc == HEXMI_OK; m += 64) {
     const int64_t left = M - m;
