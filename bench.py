@@ -304,8 +304,6 @@ def measured_traffic(wl):
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
             table = json.load(f)["traffic"]
         per_kernel = table[PROFILE_KEYS[wl.name]]
-        if wl.name == "w8a16_m256":                       # four passes of the same kernel per step
-            return 4 * sum(per_kernel.values())
         return sum(per_kernel.values())
     except (OSError, KeyError, ValueError):
         return None

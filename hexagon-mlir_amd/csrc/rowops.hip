@@ -7,6 +7,7 @@
 //                       waves keep more of HBM busy than one long wave per row)
 //   anything else (or misaligned): generic strided kernel, row re-read from L2
 #include "hexmi_common.h"
+#include <type_traits>
 
 namespace hexmi {
 namespace {
@@ -59,117 +60,177 @@ enum RowOp { kSoftmax = 0, kRmsNorm = 1, kLayerNorm = 2 };
 // THREADS threads cooperate on one row (THREADS == 64: a wave per row, several
 // rows per workgroup). Each thread owns CHUNKS 16-byte chunks, chunk c of
 // thread t covering elements [(c*THREADS + t)*N, +N).
-template <typename T, int OP, int CHUNKS, int THREADS, int ROWS_PER_BLOCK>
+//
+// PIPE (large problems whose shape fills the tile exactly: cols == CHUNKS * THREADS * N and
+// rows % ROWS_PER_BLOCK == 0, so no access is masked): the grid is a few workgroups per CU and each walks row
+// groups blockIdx.x, +gridDim.x, ...; the loads of the next group are issued before the current one is reduced,
+// so every wave always has a row in flight and HBM sees a steady stream instead of load / reduce / store phases.
+// Weight and bias stay in registers for the walk. The stores of a group are unconditional, so the wait for the
+// prefetched loads that follows them can leave exactly those stores outstanding; a store under a condition would
+// turn that wait into a wait for everything, write acknowledgements included. For the same reason LayerNorm's
+// per-row mean / rstd (one lane stores them) are written one group late, between the wait for the loads and the
+// issue of the next ones.
+// Without PIPE a workgroup handles exactly one row group (gridDim.x == number of groups) and accesses are masked.
+template <typename T, int OP, int CHUNKS, int THREADS, int ROWS_PER_BLOCK, bool PIPE>
 __global__ __launch_bounds__(THREADS * ROWS_PER_BLOCK)
 void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict__ w,
                 const T* __restrict__ b, float* __restrict__ mean_out, float* __restrict__ rstd_out,
                 int64_t rows, int cols, int64_t ld_x, int64_t ld_y, float eps) {
+  constexpr bool FULL = PIPE;
   constexpr int N = Vec16<T>::N;
   constexpr int WAVES = THREADS / kWave;
-  __shared__ float red_a[ROWS_PER_BLOCK][WAVES];     // first reduction (max / mean)
-  __shared__ float red_b[ROWS_PER_BLOCK][WAVES];     // second reduction (sum / variance)
+  constexpr int SLOTS = PIPE ? 2 : 1;                // consecutive groups alternate slots: a fast wave may start
+                                                     // the next group while a slow one still reads this one's sums
+  __shared__ float red_a[SLOTS][ROWS_PER_BLOCK][WAVES];     // first reduction (max / mean)
+  __shared__ float red_b[SLOTS][ROWS_PER_BLOCK][WAVES];     // second reduction (sum / variance)
   const int t = threadIdx.x % THREADS;
   const int row_in_block = threadIdx.x / THREADS;
   const int wave_in_row = t / kWave;
-  int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + row_in_block;
-  // Rows past the end are computed on the last row and not stored, so every wave reaches the barriers.
-  const bool row_valid = row < rows;
-  if (!row_valid) {
-    if constexpr (WAVES == 1) return;               // no barrier in this configuration: whole waves may leave
-    row = rows - 1;
-  }
+  const int64_t groups = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  const float inv_n = 1.0f / (float)cols;
 
-  const T* xr = x + row * ld_x;
-  T* yr = y + row * ld_y;
-  float v[CHUNKS][N];
-#pragma unroll
-  for (int c = 0; c < CHUNKS; ++c) {
-    const int col = (c * THREADS + t) * N;
-    if (col < cols) {
-      Vec16<T> raw = load16_stream(xr + col);
-#pragma unroll
-      for (int i = 0; i < N; ++i) v[c][i] = to_f32<T>(raw.v[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < N; ++i) v[c][i] = (OP == kSoftmax) ? -INFINITY : 0.0f;
-    }
-  }
-
-  if constexpr (OP == kSoftmax) {
-    float m = -INFINITY;
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c)
-#pragma unroll
-      for (int i = 0; i < N; ++i) m = fmaxf(m, v[c][i]);
-    m = block_reduce<true, WAVES>(m, red_a[row_in_block], wave_in_row);
-    float s = 0.0f;
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c)
-#pragma unroll
-      for (int i = 0; i < N; ++i) { v[c][i] = __expf(v[c][i] - m); s += v[c][i]; }
-    s = block_reduce<false, WAVES>(s, red_b[row_in_block], wave_in_row);
-    const float inv = 1.0f / s;
+  Vec16<T> wv[CHUNKS], bv[CHUNKS];
+  if constexpr (PIPE && OP != kSoftmax) {
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
       const int col = (c * THREADS + t) * N;
-      if (col < cols && row_valid) {
-        Vec16<T> o;
-#pragma unroll
-        for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i] * inv);
-        store16_stream(yr + col, o);
+      if (col < cols) {
+        if (w) wv[c] = load16(w + col);
+        if (OP == kLayerNorm && b) bv[c] = load16(b + col);
       }
     }
-  } else {
-    const float inv_n = 1.0f / (float)cols;
-    float mean = 0.0f;
+  }
+
+  // Rows past the end (last group only) are computed on the last row and not stored, so every wave reaches the
+  // barriers.
+  auto row_of = [&](int64_t g) {
+    const int64_t r = g * ROWS_PER_BLOCK + row_in_block;
+    return r < rows ? r : rows - 1;
+  };
+  // Chunks past the end of the row load column 0 instead (and are ignored): the loads stay free of branches,
+  // which lets them be issued back to back and waited for only where their values are used.
+  int load_col[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) load_col[c] = (c * THREADS + t) * N < cols ? (c * THREADS + t) * N : 0;
+  Vec16<T> raw[CHUNKS];
+  {
+    const T* xr = x + row_of(blockIdx.x) * ld_x;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) raw[c] = load16_stream(xr + load_col[c]);
+  }
+
+  int slot = 0;
+  int64_t g = blockIdx.x;
+  float stat_mean = 0.0f, stat_rstd = 0.0f;           // LayerNorm statistics of the previous group, not yet stored
+  int64_t stat_row = -1;
+  auto flush_stats = [&]() {
     if constexpr (OP == kLayerNorm) {
+      if (t == 0 && stat_row >= 0) {
+        if (mean_out) mean_out[stat_row] = stat_mean;
+        if (rstd_out) rstd_out[stat_row] = stat_rstd;
+      }
+    }
+  };
+  // One row group; PREFETCH (a compile-time flag, so the walk below has no branch around the loads) issues the
+  // loads of group g + gridDim.x before the reductions of group g.
+  auto process = [&](auto prefetch_tag) {
+    constexpr bool PREFETCH = decltype(prefetch_tag)::value;
+    const int64_t row = g * ROWS_PER_BLOCK + row_in_block;
+    const bool row_valid = FULL || row < rows;
+    T* yr = y + (row_valid ? row : rows - 1) * ld_y;
+    float v[CHUNKS][N];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const bool in = FULL || (c * THREADS + t) * N < cols;
+#pragma unroll
+      for (int i = 0; i < N; ++i) v[c][i] = in ? to_f32<T>(raw[c].v[i]) : (OP == kSoftmax ? -INFINITY : 0.0f);
+    }
+    flush_stats();
+    if constexpr (PREFETCH) {
+      const T* xn = x + row_of(g + gridDim.x) * ld_x;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) raw[c] = load16_stream(xn + load_col[c]);
+    }
+
+    if constexpr (OP == kSoftmax) {
+      float m = -INFINITY;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+        for (int i = 0; i < N; ++i) m = fmaxf(m, v[c][i]);
+      m = block_reduce<true, WAVES>(m, red_a[slot][row_in_block], wave_in_row);
       float s = 0.0f;
 #pragma unroll
       for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
-        for (int i = 0; i < N; ++i) s += v[c][i];     // masked slots hold 0
-      mean = block_reduce<false, WAVES>(s, red_a[row_in_block], wave_in_row) * inv_n;
-    }
-    float q = 0.0f;
+        for (int i = 0; i < N; ++i) { v[c][i] = __expf(v[c][i] - m); s += v[c][i]; }
+      s = block_reduce<false, WAVES>(s, red_b[slot][row_in_block], wave_in_row);
+      const float inv = 1.0f / s;
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      if ((c * THREADS + t) * N < cols) {
+      for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * THREADS + t) * N;
+        if (FULL || (col < cols && row_valid)) {
+          Vec16<T> o;
 #pragma unroll
-        for (int i = 0; i < N; ++i) { v[c][i] -= mean; q += v[c][i] * v[c][i]; }
-      }
-    }
-    q = block_reduce<false, WAVES>(q, red_b[row_in_block], wave_in_row);
-    const float rstd = 1.0f / sqrtf(q * inv_n + eps);
-    if constexpr (OP == kLayerNorm) {
-      if (t == 0 && row_valid) {
-        if (mean_out) mean_out[row] = mean;
-        if (rstd_out) rstd_out[row] = rstd;
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      const int col = (c * THREADS + t) * N;
-      if (col < cols && row_valid) {
-        Vec16<T> o;
-        if (w) {
-          Vec16<T> wv = load16(w + col);
-#pragma unroll
-          for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd * to_f32<T>(wv.v[i]);
-        } else {
-#pragma unroll
-          for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd;
+          for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i] * inv);
+          store16_stream(yr + col, o);
         }
-        if (OP == kLayerNorm && b) {
-          Vec16<T> bv = load16(b + col);
+      }
+    } else {
+      float mean = 0.0f;
+      if constexpr (OP == kLayerNorm) {
+        float s = 0.0f;
 #pragma unroll
-          for (int i = 0; i < N; ++i) v[c][i] += to_f32<T>(bv.v[i]);
+        for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+          for (int i = 0; i < N; ++i) s += v[c][i];     // masked slots hold 0
+        mean = block_reduce<false, WAVES>(s, red_a[slot][row_in_block], wave_in_row) * inv_n;
+      }
+      float q = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) {
+        if (FULL || (c * THREADS + t) * N < cols) {
+#pragma unroll
+          for (int i = 0; i < N; ++i) { v[c][i] -= mean; q += v[c][i] * v[c][i]; }
         }
+      }
+      q = block_reduce<false, WAVES>(q, red_b[slot][row_in_block], wave_in_row);
+      const float rstd = 1.0f / sqrtf(q * inv_n + eps);
+      if constexpr (OP == kLayerNorm) {
+        stat_mean = mean;
+        stat_rstd = rstd;
+        stat_row = row_valid ? row : -1;
+      }
 #pragma unroll
-        for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i]);
-        store16_stream(yr + col, o);
+      for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * THREADS + t) * N;
+        if (FULL || (col < cols && row_valid)) {
+          Vec16<T> o;
+          if (w) {
+            if constexpr (!PIPE) wv[c] = load16(w + col);
+#pragma unroll
+            for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd * to_f32<T>(wv[c].v[i]);
+          } else {
+#pragma unroll
+            for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd;
+          }
+          if (OP == kLayerNorm && b) {
+            if constexpr (!PIPE) bv[c] = load16(b + col);
+#pragma unroll
+            for (int i = 0; i < N; ++i) v[c][i] += to_f32<T>(bv[c].v[i]);
+          }
+#pragma unroll
+          for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i]);
+          store16_stream(yr + col, o);
+        }
       }
     }
+  };
+  if constexpr (PIPE) {
+    for (; g + gridDim.x < groups; g += gridDim.x, slot ^= 1) process(std::true_type{});
   }
+  if (g < groups) process(std::false_type{});
+  flush_stats();
 }
 
 // Any shape / alignment: 256 threads per row, scalar accesses, the row is read
@@ -223,13 +284,39 @@ void row_kernel_generic(const T* __restrict__ x, T* __restrict__ y, const T* __r
   }
 }
 
-template <typename T, int OP, int CHUNKS, int THREADS, int RPB>
-int launch_tile(const T* x, T* y, const T* w, const T* b, float* mean, float* rstd, int64_t rows,
+// Grid of a pipelined launch: about 32 KiB of loads in flight per CU (2048 / CHUNKS threads, each with CHUNKS
+// 16-byte loads outstanding) measured fastest on MI355X: more resident workgroups shorten each one's walk and
+// bring the load / reduce / store phases back, fewer leave HBM idle. A problem too small for every workgroup to
+// walk at least four groups is launched with one group per workgroup instead.
+constexpr int kPipeChunksPerCu = 2048;
+constexpr int kPipeMinWalk = 4;
+
+template <typename T, int OP, int CHUNKS, int THREADS, int RPB, bool PIPE>
+int launch_grid(int64_t blocks, const T* x, T* y, const T* w, const T* b, float* mean, float* rstd, int64_t rows,
                 int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s) {
-  const int64_t blocks = (rows + RPB - 1) / RPB;
-  hipLaunchKernelGGL((row_kernel<T, OP, CHUNKS, THREADS, RPB>), dim3((unsigned)blocks), dim3(THREADS * RPB), 0, s,
-                     x, y, w, b, mean, rstd, rows, (int)cols, ld_x, ld_y, eps);
+  hipLaunchKernelGGL((row_kernel<T, OP, CHUNKS, THREADS, RPB, PIPE>), dim3((unsigned)blocks), dim3(THREADS * RPB), 0,
+                     s, x, y, w, b, mean, rstd, rows, (int)cols, ld_x, ld_y, eps);
   return launch_status();
+}
+
+// MAY_PIPE: whether the tile has a pipelined instantiation at all (the widest tiles do not: one workgroup of
+// 1024 threads per CU leaves nothing to overlap with). threads_per_cu <= 0 selects the default.
+template <typename T, int OP, int CHUNKS, int THREADS, int RPB, bool MAY_PIPE>
+int launch_tile(const T* x, T* y, const T* w, const T* b, float* mean, float* rstd, int64_t rows,
+                int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s, int threads_per_cu = 0) {
+  constexpr int N = 16 / sizeof(T);
+  const int64_t groups = (rows + RPB - 1) / RPB;
+  if constexpr (MAY_PIPE) {
+    if (cols == (int64_t)CHUNKS * THREADS * N && rows % RPB == 0) {
+      if (threads_per_cu <= 0) threads_per_cu = kPipeChunksPerCu / CHUNKS;
+      const int per_cu = threads_per_cu / (THREADS * RPB) > 0 ? threads_per_cu / (THREADS * RPB) : 1;
+      const int64_t resident = (int64_t)hexmi_num_cus() * per_cu;
+      if (resident > 0 && groups >= kPipeMinWalk * resident)
+        return launch_grid<T, OP, CHUNKS, THREADS, RPB, true>(resident, x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y,
+                                                              eps, s);
+    }
+  }
+  return launch_grid<T, OP, CHUNKS, THREADS, RPB, false>(groups, x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s);
 }
 
 template <typename T, int OP>
@@ -243,17 +330,18 @@ int dispatch_rows(const void* xv, void* yv, const void* wv, const void* bv, floa
   const bool vec_ok = cols % N == 0 && ld_x % N == 0 && ld_y % N == 0 && aligned_to(x, 16) && aligned_to(y, 16) &&
                       (!w || aligned_to(w, 16)) && (!b || aligned_to(b, 16));
   const int64_t chunks = (cols + N - 1) / N;        // 16-byte chunks per row
-#define HEXMI_TILE(C, TH, RPB) return launch_tile<T, OP, C, TH, RPB>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s)
+#define HEXMI_TILE(C, TH, RPB, PIPE) \
+  return launch_tile<T, OP, C, TH, RPB, PIPE>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s)
   if (vec_ok && rows <= 0x7fffffff) {
     // about two to four 16-byte chunks per thread; rows narrower than 4 KiB stay inside one wave (no barrier)
-    if (chunks <= 64 * 1) HEXMI_TILE(1, 64, 4);
-    if (chunks <= 64 * 2) HEXMI_TILE(2, 64, 4);
-    if (chunks <= 64 * 4) HEXMI_TILE(4, 64, 4);
-    if (chunks <= 256 * 2) HEXMI_TILE(2, 256, 1);
-    if (chunks <= 256 * 4) HEXMI_TILE(4, 256, 1);
-    if (chunks <= 512 * 4) HEXMI_TILE(4, 512, 1);
-    if (chunks <= 1024 * 4) HEXMI_TILE(4, 1024, 1);
-    if (chunks <= 1024 * 8) HEXMI_TILE(8, 1024, 1);
+    if (chunks <= 64 * 1) HEXMI_TILE(1, 64, 4, true);
+    if (chunks <= 64 * 2) HEXMI_TILE(2, 64, 4, true);
+    if (chunks <= 64 * 4) HEXMI_TILE(4, 64, 4, true);
+    if (chunks <= 256 * 2) HEXMI_TILE(2, 256, 1, true);
+    if (chunks <= 256 * 4) HEXMI_TILE(4, 256, 1, true);
+    if (chunks <= 512 * 4) HEXMI_TILE(4, 512, 1, true);
+    if (chunks <= 1024 * 4) HEXMI_TILE(4, 1024, 1, false);
+    if (chunks <= 1024 * 8) HEXMI_TILE(8, 1024, 1, false);
   }
 #undef HEXMI_TILE
   if (rows > 0x7fffffff) return HEXMI_ENOTSUP;

@@ -142,6 +142,37 @@ def test_norm_config_shape(hexmi, oracle):
     assert close16(got_r2, got_r, 1, 1e-6)
 
 
+# Shapes that fill a tile exactly and are tall enough for the persistent walk (a few workgroups per CU, each
+# walking several row groups with the next group's loads in flight); row counts chosen so that workgroups walk
+# unequal numbers of groups.
+WALK_SHAPES = [(torch.float16, 32772, 512), (torch.float16, 16388, 1024), (torch.float32, 8204, 1024),
+               (torch.float16, 4100, 4096), (torch.bfloat16, 2051, 8192), (torch.float32, 1030, 8192)]
+
+
+@pytest.mark.parametrize("dtype,rows,cols", WALK_SHAPES)
+def test_persistent_walk(hexmi, oracle, dtype, rows, cols):
+    g = _gen(11)
+    x = (torch.randn(rows, cols, generator=g) + 0.25).to(dtype)
+    w = (1 + 0.1 * torch.randn(cols, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(cols, generator=g)).to(dtype)
+    a, tag = to_np(x)
+    wn, _ = to_np(w)
+    bn, _ = to_np(b)
+    xd, wd, bd = x.cuda(), w.cuda(), b.cuda()
+    _check(hexmi.softmax(xd), from_np(oracle.softmax(a, dtype=tag), dtype), dtype, atol16=1e-7)
+    _check(hexmi.rms_norm(xd, wd, 1e-5), from_np(oracle.rms_norm(a, wn, 1e-5, dtype=tag), dtype), dtype)
+    _check(hexmi.rms_norm(xd, None, 1e-5), from_np(oracle.rms_norm(a, None, 1e-5, dtype=tag), dtype), dtype)
+    want, mean, rstd = oracle.layer_norm(a, wn, bn, 1e-5, dtype=tag)
+    m = torch.full((rows,), float("nan"), device="cuda")
+    r = torch.full((rows,), float("nan"), device="cuda")
+    got = hexmi.layer_norm(xd, wd, bd, 1e-5, mean=m, rstd=r)
+    _check(got, from_np(want, dtype), dtype, atol16=2e-6, atol32=2e-6)
+    assert torch.allclose(m.cpu(), torch.from_numpy(mean), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(r.cpu(), torch.from_numpy(rstd), rtol=1e-5)
+    want_plain = oracle.layer_norm(a, None, None, 1e-5, dtype=tag)[0]
+    _check(hexmi.layer_norm(xd, None, None, 1e-5), from_np(want_plain, dtype), dtype, atol16=2e-6, atol32=2e-6)
+
+
 def test_norm_reference_call_sites(hexmi, oracle):
     g = _gen(5)
     # test_rms_norm.py:65-89
