@@ -196,8 +196,9 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float a, float
 // tiles resident on one XCD share A and B panels.
 __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int total = tiles_m * tiles_n;
-  int logical = pid;
-  if (total % 8 == 0) logical = (pid % 8) * (total / 8) + pid / 8;
+  // XCD x runs ids x, x + 8, ...: total/8 of them, one more on the first total%8 XCDs
+  const int xcd = pid % 8, per = total / 8, extra = total % 8;
+  const int logical = xcd * per + (xcd < extra ? xcd : extra) + pid / 8;
   constexpr int GROUP_M = 4;
   const int group_size = GROUP_M * tiles_n;
   const int group = logical / group_size;
