@@ -15,6 +15,7 @@ current stream, which hexmi passes to the C ABI).
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -232,6 +233,42 @@ class Attention(Workload):
         return t * (Z * H / heads), "%d of %d heads, fp32 F.scaled_dot_product_attention(is_causal=True) on CPU, time scaled" % (heads, Z * H)
 
 
+class MaskedAttention(Workload):
+    """tm_tensor.attention with an additive mask (the next row after the causal kernel): [B,S,D] operands."""
+    bound, dtype, kernel = "mfma", "f16", "flash_fwd_kernel"
+
+    def __init__(self, B, S, D):
+        self.shape = (B, S, D)
+        self.name = "attn_masked_f16_%dx%dx%d" % self.shape
+        self.desc = ("tm_tensor.attention fp16 q,k,v [%d,%d,%d] N(0,1), additive mask [%d,%d,%d] N(0,1) with 30%% -inf, "
+                     "scale 1/sqrt(%d)" % (B, S, D, B, S, S, D))
+
+    def setup(self, torch, hexmi):
+        B, S, D = self.shape
+        g = torch.Generator().manual_seed(0)
+        q, k, v = (torch.randn(B, S, D, generator=g).half() for _ in range(3))
+        mask = torch.randn(B, S, S, generator=g)
+        mask[torch.rand(B, S, S, generator=g) < 0.3] = float("-inf")
+        mask[:, :, 0] = 0.0
+        self.hexmi, self.host = hexmi, {"q": q, "k": k, "v": v, "mask": mask.half()}
+        self.work = 4 * B * S * S * D                     # QK^T and PV, every key of every query
+        self.sets = _sets(torch, self.host, 0, rotate=False)
+        self.sets[0]["out"] = torch.empty_like(self.sets[0]["q"])
+
+    def step(self, i):
+        s = self.sets[0]
+        self.hexmi.attention(s["q"], s["k"], s["v"], s["mask"], out=s["out"])
+
+    def cpu(self, torch):
+        from oracle import torch_cpu
+        B, S, D = self.shape
+        n = 4
+        h = self.host
+        t = _time_cpu(lambda: torch_cpu.attention_masked(h["q"][:n], h["k"][:n], h["v"][:n], h["mask"][:n],
+                                                         1.0 / math.sqrt(D)), 1)
+        return t * (B / n), "%d of %d batch entries, fp32 F.scaled_dot_product_attention(attn_mask=...) on CPU, time scaled" % (n, B)
+
+
 def _time_cpu(fn, iters):
     fn()                                                # warm-up
     ts = []
@@ -246,13 +283,13 @@ def _time_cpu(fn, iters):
 def make_workloads():
     return {w.name: w for w in (
         Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
-        W8A16(1), W8A16(16), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128),
+        W8A16(1), W8A16(16), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128),
         CopyCalibration())}
 
 
 ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "gemm": "gemm_f16_4096",
            "gemm_bf16": "gemm_bf16_8192", "attn": "attn_causal_f16_4x32x4096x128",
-           "attn_long": "attn_causal_f16_1x32x16384x128", "rms_norm": "rms_norm_f16_8192x4096",
+           "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128", "rms_norm": "rms_norm_f16_8192x4096",
            "layer_norm": "layer_norm_f16_8192x4096"}
 
 

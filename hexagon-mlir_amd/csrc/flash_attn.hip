@@ -113,10 +113,16 @@ template <> __device__ __forceinline__ void store4o<bf16>(bf16* p, float a, floa
   *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)a, (bf16)b, (bf16)c, (bf16)d};
 }
 
-template <typename T, typename OutT, int D, bool CAUSAL>
+// GENERAL: the number of keys (Skv) may differ from the number of queries (S) and an additive mask
+// [ZH, S, Skv] (same dtype as Q; may be null) is added to the scaled scores before the softmax, as
+// tm_tensor.attention does (qcom_hexagon_backend/lib/Transforms/LowerTmTensor.cpp:157-160); Skv % 4 == 0.
+template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false>
 __global__ __launch_bounds__(256, 2)
 void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
-                      OutT* __restrict__ O, int ZH, int S, float scale_log2e) {
+                      OutT* __restrict__ O, int ZH, int S, float scale_log2e, const T* __restrict__ Mk = nullptr,
+                      int Skv_arg = 0, float mask_factor = 0.0f) {
+  static_assert(!(CAUSAL && GENERAL), "the causal kernel has as many keys as queries and no mask");
+  const int Skv = GENERAL ? Skv_arg : S;
   typedef typename MfmaT<T>::Frag Frag;
   constexpr int DS = D / 16;                        // 16-wide steps over the head dimension
   constexpr int DT = D / 32;                        // 32-wide output tiles over the head dimension
@@ -140,9 +146,10 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     qb = nqb - 1 - blockIdx.x / ZH;
   }
   const int64_t base = (int64_t)zh * S * D;
+  const int64_t kv_base = (int64_t)zh * Skv * D;
   const T* q_g = Q + base;
-  const T* k_g = K + base;
-  const T* v_g = V + base;
+  const T* k_g = K + kv_base;
+  const T* v_g = V + kv_base;
 
   const int q0 = qb * kBlockM + wave * 32;           // first query row of this wave
   const int qrow = q0 + lane % 32;                    // the query row this lane's scores belong to
@@ -165,7 +172,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   float m_i = -INFINITY;                              // running max (already multiplied by scale*log2e)
   float l_i = 0.0f;                                   // this lane's share of the running sum
 
-  const int key_end = CAUSAL ? ((qb + 1) * kBlockM < S ? (qb + 1) * kBlockM : S) : S;
+  const int key_end = CAUSAL ? ((qb + 1) * kBlockM < S ? (qb + 1) * kBlockM : S) : Skv;
   const int n_steps = (key_end + kBlockN - 1) / kBlockN;
 
   KvTileLoader<T, D, false> k_loader;
@@ -173,8 +180,8 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   k_loader.init(wave, lane);
   v_loader.init(wave, lane);
   auto load_kv = [&](int step, T* k_dst, T* v_dst) {
-    k_loader.issue(k_g, step * kBlockN, S, k_dst);
-    v_loader.issue(v_g, step * kBlockN, S, v_dst);
+    k_loader.issue(k_g, step * kBlockN, Skv, k_dst);
+    v_loader.issue(v_g, step * kBlockN, Skv, v_dst);
   };
 
   // One 32-key tile of the online softmax: mask, row max, (rare) rescale, exponentials, row sum; leaves the
@@ -188,7 +195,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int key = key_base + 8 * (r / 4) + 4 * half + r % 4;
-        if ((CAUSAL && key > qrow) || key >= S) s[r] = -INFINITY;
+        if ((CAUSAL && key > qrow) || key >= Skv) s[r] = -INFINITY;
       }
     }
     float mx = -INFINITY;
@@ -240,8 +247,29 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     }
   };
 
+  // mask row of this lane's query (GENERAL with a mask only)
+  const T* mask_row = nullptr;
+  if constexpr (GENERAL) {
+    if (Mk) mask_row = Mk + ((int64_t)zh * S + (qrow < S ? qrow : S - 1)) * Skv;
+  }
+
   auto process = [&](int step, const T* k_src, const T* v_src) {
     const int n0 = step * kBlockN;
+    // mask values of this lane's 32 scores: four runs of four consecutive keys per 32-key tile
+    typedef T MaskRun __attribute__((ext_vector_type(4)));
+    MaskRun mk[2][4];
+    if constexpr (GENERAL) {
+      if (mask_row) {
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            int key = n0 + jt * 32 + 8 * g4 + 4 * half;
+            key = key + 4 <= Skv ? key : Skv - 4;          // past the end: any valid run, those scores are dropped
+            mk[jt][g4] = *reinterpret_cast<const MaskRun*>(mask_row + key);
+          }
+      }
+    }
     // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4], one MFMA chain per 32-key tile
     f32x16 s[2];
 #pragma unroll
@@ -258,7 +286,16 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     }
     // The softmax of tile 0 runs on the vector ALUs while the matrix cores finish the scores of tile 1, and the
     // softmax of tile 1 while they accumulate P V of tile 0.
-    const bool need_mask = (CAUSAL && n0 + kBlockN - 1 > q0) || (n0 + kBlockN > S);
+    if constexpr (GENERAL) {
+      if (mask_row) {
+        // softmax(scale*s + mask) = softmax(scale * (s + mask/scale)): fold the mask into the raw scores
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s[jt][r] = fmaf(to_f32<T>(mk[jt][r / 4][r % 4]), mask_factor, s[jt][r]);
+      }
+    }
+    const bool need_mask = (CAUSAL && n0 + kBlockN - 1 > q0) || (n0 + kBlockN > Skv);
     Frag pf[4];
     softmax_tile(n0, need_mask, s[0], &pf[0]);
     pv_tile(v_src, 0, &pf[0]);
@@ -305,7 +342,8 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
 template <typename T, typename OutT, int DMAX>
 __global__ __launch_bounds__(256)
 void flash_fwd_rowwise(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
-                       OutT* __restrict__ O, int64_t rows_total, int S, int D, float scale_log2e, int causal) {
+                       OutT* __restrict__ O, int64_t rows_total, int S, int D, float scale_log2e, int causal,
+                       const T* __restrict__ Mk, int Skv) {
   __shared__ float q_s[4][DMAX];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int64_t row = (int64_t)blockIdx.x * 4 + wave;      // over ZH*S
@@ -313,21 +351,24 @@ void flash_fwd_rowwise(const T* __restrict__ Q, const T* __restrict__ K, const T
   const int64_t zh = row / S;
   const int qi = (int)(row % S);
   const T* q = Q + row * D;
-  const T* k = K + zh * S * D;
-  const T* v = V + zh * S * D;
+  const T* k = K + zh * Skv * D;
+  const T* v = V + zh * Skv * D;
+  const T* mrow = Mk ? Mk + row * Skv : nullptr;         // additive mask row [Skv] of this query
   for (int d = lane; d < D; d += kWave) q_s[wave][d] = to_f32<T>(q[d]);
   __builtin_amdgcn_wave_barrier();
   float o[DMAX];
 #pragma unroll
   for (int d = 0; d < DMAX; ++d) o[d] = 0.0f;
   float m = -INFINITY, l = 0.0f;
-  const int kend = causal ? qi + 1 : S;
+  const int kend = causal ? qi + 1 : Skv;
   for (int j = lane; j < kend; j += kWave) {
     const T* kj = k + (int64_t)j * D;
     float sdot = 0.0f;
     for (int d = 0; d < D; ++d) sdot = fmaf(q_s[wave][d], to_f32<T>(kj[d]), sdot);
-    const float sv = sdot * scale_log2e;
+    float sv = sdot * scale_log2e;
+    if (mrow) sv = fmaf(to_f32<T>(mrow[j]), 1.44269504088896340736f, sv);
     const float m_new = fmaxf(m, sv);
+    if (m_new == -INFINITY) continue;                      // masked out so far: nothing to accumulate
     const float alpha = exp2f(m - m_new);
     const float p = exp2f(sv - m_new);
     l = l * alpha + p;
@@ -367,25 +408,57 @@ int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH
   return launch_status();
 }
 
+template <typename T, typename OutT, int D>
+int launch_mfma_general(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
+                        int64_t Skv, float scale_log2e, hipStream_t st) {
+  const int64_t nqb = (S + kBlockM - 1) / kBlockM;
+  const int64_t blocks = nqb * ZH;
+  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  const float mask_factor = 1.44269504088896340736f / scale_log2e;     // mask / sm_scale
+  hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, false, true>), dim3((unsigned)blocks), dim3(256), 0, st,
+                     static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                     static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e, static_cast<const T*>(mask), (int)Skv,
+                     mask_factor);
+  return launch_status();
+}
+
 template <typename T, typename OutT>
-int launch_rowwise(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, int64_t D,
-                   float scale_log2e, bool causal, hipStream_t st) {
+int launch_rowwise(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
+                   int64_t Skv, int64_t D, float scale_log2e, bool causal, hipStream_t st) {
   const int64_t rows = ZH * S;
   const int64_t blocks = (rows + 3) / 4;
   if (blocks > 0x7fffffff || D > 128) return HEXMI_ENOTSUP;
   hipLaunchKernelGGL((flash_fwd_rowwise<T, OutT, 128>), dim3((unsigned)blocks), dim3(256), 0, st,
                      static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
-                     static_cast<OutT*>(O), rows, (int)S, (int)D, scale_log2e, causal ? 1 : 0);
+                     static_cast<OutT*>(O), rows, (int)S, (int)D, scale_log2e, causal ? 1 : 0,
+                     static_cast<const T*>(mask), (int)Skv);
   return launch_status();
 }
 
+// mask == nullptr and Skv == S: the tuned kernels; otherwise the general ones.
 template <typename T, typename OutT>
-int dispatch_half(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, int64_t D,
-                  float scale_log2e, bool causal, hipStream_t st) {
+int dispatch_half(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
+                  int64_t Skv, int64_t D, float scale_log2e, bool causal, hipStream_t st) {
   const bool ok = aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16);
-  if (ok && D == 128) return launch_mfma<T, OutT, 128>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
-  if (ok && D == 64) return launch_mfma<T, OutT, 64>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
-  return launch_rowwise<T, OutT>(Q, K, V, O, ZH, S, D, scale_log2e, causal, st);
+  const bool plain = !mask && Skv == S;
+  if (ok && plain && D == 128) return launch_mfma<T, OutT, 128>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
+  if (ok && plain && D == 64) return launch_mfma<T, OutT, 64>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
+  const bool general_ok = ok && !causal && Skv % 4 == 0 && Skv >= 4 && scale_log2e != 0.0f && (!mask || aligned_to(mask, 8));
+  if (general_ok && D == 128) return launch_mfma_general<T, OutT, 128>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
+  if (general_ok && D == 64) return launch_mfma_general<T, OutT, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
+  return launch_rowwise<T, OutT>(Q, K, V, mask, O, ZH, S, Skv, D, scale_log2e, causal, st);
+}
+
+int attention_any(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
+                  int64_t Skv, int64_t D, float sm_scale, bool cz, int in_dtype, int out_dtype, hipStream_t st) {
+  const float c = sm_scale * 1.44269504088896340736f;
+  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F16) return dispatch_half<f16, f16>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
+  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F32) return dispatch_half<f16, float>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
+  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_BF16) return dispatch_half<bf16, bf16>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
+  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_F32) return dispatch_half<bf16, float>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
+  if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32)
+    return launch_rowwise<float, float>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
+  return HEXMI_ENOTSUP;
 }
 
 }  // namespace
@@ -400,14 +473,18 @@ extern "C" int hexmi_flash_attn_fwd(const void* Q, const void* K, const void* V,
   if (Z == 0 || H == 0 || S == 0 || D == 0) return HEXMI_OK;
   if (!Q || !K || !V || !O) return HEXMI_EINVAL;
   if (S > 0x7fffffff / 2 || Z * H > 0x7fffffff) return HEXMI_ENOTSUP;
-  const float c = sm_scale * 1.44269504088896340736f;
-  hipStream_t st = as_stream(stream);
-  const bool cz = causal != 0;
-  const int64_t ZH = Z * H;
-  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F16) return dispatch_half<f16, f16>(Q, K, V, O, ZH, S, D, c, cz, st);
-  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F32) return dispatch_half<f16, float>(Q, K, V, O, ZH, S, D, c, cz, st);
-  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_BF16) return dispatch_half<bf16, bf16>(Q, K, V, O, ZH, S, D, c, cz, st);
-  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_F32) return dispatch_half<bf16, float>(Q, K, V, O, ZH, S, D, c, cz, st);
-  if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) return launch_rowwise<float, float>(Q, K, V, O, ZH, S, D, c, cz, st);
-  return HEXMI_ENOTSUP;
+  return attention_any(Q, K, V, nullptr, O, Z * H, S, S, D, sm_scale, causal != 0, in_dtype, out_dtype,
+                       as_stream(stream));
+}
+
+extern "C" int hexmi_attention(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t batch,
+                               int64_t seq_q, int64_t seq_kv, int64_t head_dim, float sm_scale, int in_dtype,
+                               int out_dtype, hexmi_stream_t stream) {
+  if (batch < 0 || seq_q < 0 || seq_kv < 0 || head_dim < 0) return HEXMI_EINVAL;
+  if (batch == 0 || seq_q == 0 || head_dim == 0) return HEXMI_OK;
+  if (seq_kv == 0) return HEXMI_EINVAL;                    // a softmax over no keys is undefined
+  if (!Q || !K || !V || !O) return HEXMI_EINVAL;
+  if (seq_q > 0x7fffffff / 2 || seq_kv > 0x7fffffff / 2 || batch > 0x7fffffff) return HEXMI_ENOTSUP;
+  return attention_any(Q, K, V, mask, O, batch, seq_q, seq_kv, head_dim, sm_scale, false, in_dtype, out_dtype,
+                       as_stream(stream));
 }

@@ -36,6 +36,7 @@ SIGNATURES = {
     "hexmi_gemm_w8a16": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_dequant_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_flash_attn_fwd": (_int, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _ptr]),
+    "hexmi_attention": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _ptr]),
 }
 
 _lib = None

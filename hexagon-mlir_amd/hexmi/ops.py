@@ -47,6 +47,7 @@ _LIBDEF.define("matmul(Tensor a, Tensor b, bool trans_b, Tensor(a!) out) -> ()")
 _LIBDEF.define("w8a16_matmul(Tensor a, Tensor w, Tensor scales, Tensor(a!) out) -> ()")
 _LIBDEF.define("dequant_w8(Tensor w, Tensor scales, Tensor(a!) out) -> ()")
 _LIBDEF.define("flash_attention(Tensor q, Tensor k, Tensor v, float sm_scale, bool causal, Tensor(a!) out) -> ()")
+_LIBDEF.define("attention(Tensor q, Tensor k, Tensor v, Tensor? mask, float sm_scale, Tensor(a!) out) -> ()")
 
 
 def _softmax_impl(x, out):
@@ -100,9 +101,17 @@ def _flash_impl(q, k, v, sm_scale, causal, out):
                    "hexmi_flash_attn_fwd")
 
 
+def _attention_impl(q, k, v, mask, sm_scale, out):
+    B, Sq, D = q.shape
+    Skv = k.shape[1]
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().hexmi_attention(_p(q), _p(k), _p(v), _p(mask), _p(out), B, Sq, Skv, D, sm_scale,
+                                              _dt(q), _dt(out), _stream()), "hexmi_attention")
+
+
 for _name, _fn in (("softmax", _softmax_impl), ("rms_norm", _rms_norm_impl), ("layer_norm", _layer_norm_impl),
                    ("matmul", _matmul_impl), ("w8a16_matmul", _w8a16_impl), ("dequant_w8", _dequant_impl),
-                   ("flash_attention", _flash_impl)):
+                   ("flash_attention", _flash_impl), ("attention", _attention_impl)):
     _LIBDEF.impl(_name, _fn, "CUDA")
 
 
@@ -259,4 +268,27 @@ def flash_attention(q, k, v, sm_scale=None, causal=False, out=None, out_dtype=No
     qd, kd, vd = _stage(q, dev), _stage(k, dev), _stage(v, dev)
     od = _out_like(out, q.shape, out_dtype, dev)
     torch.ops.hexmi.flash_attention(qd, kd, vd, float(sm_scale), bool(causal), od)
+    return _finish(od, out)
+
+
+def attention(q, k, v, mask=None, sm_scale=None, out=None, out_dtype=None):
+    """tm_tensor.attention: softmax(Q K^T / sqrt(d) + mask) V for q [B,Sq,D], k / v [B,Skv,D] and an additive
+    mask [B,Sq,Skv] (or None) (include/hexagon/Dialect/TmTensor/IR/TmTensorOps.td:28-56,
+    lib/Transforms/LowerTmTensor.cpp:70-235); `F.scaled_dot_product_attention(q, k, v, attn_mask=mask)`."""
+    if q.dim() != 3 or k.dim() != 3 or v.shape != k.shape or q.shape[0] != k.shape[0] or q.shape[2] != k.shape[2]:
+        raise ValueError("hexmi.attention: q [B,Sq,D], k and v [B,Skv,D]")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("hexmi.attention: q, k, v dtypes differ")
+    B, Sq, D = q.shape
+    Skv = k.shape[1]
+    if mask is not None and (tuple(mask.shape) != (B, Sq, Skv) or mask.dtype != q.dtype):
+        raise ValueError("hexmi.attention: mask must be [%d,%d,%d] of %s" % (B, Sq, Skv, q.dtype))
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    if out_dtype is None:
+        out_dtype = out.dtype if out is not None else q.dtype
+    dev = _device() if q.device.type != "cuda" else q.device
+    qd, kd, vd, md = _stage(q, dev), _stage(k, dev), _stage(v, dev), _stage(mask, dev)
+    od = _out_like(out, q.shape, out_dtype, dev)
+    torch.ops.hexmi.attention(qd, kd, vd, md, float(sm_scale), od)
     return _finish(od, out)

@@ -139,6 +139,23 @@ int hexmi_flash_attn_fwd(const void *Q, const void *K, const void *V, void *O,
                          float sm_scale, int causal, int in_dtype,
                          int out_dtype, hexmi_stream_t stream);
 
+/* tm_tensor.attention: O = softmax(sm_scale * Q K^T + mask) V per batch entry,
+ * "Equivalent to : softmax(QK^T / sqrt(d_k) + mask) * V"
+ * (include/hexagon/Dialect/TmTensor/IR/TmTensorOps.td:28-56; lowering
+ * lib/Transforms/LowerTmTensor.cpp:70-235: scale `:120-123`, additive mask
+ * `:157-160`, max / sub / exp / sum / div `:164-222`, P V `:225-229`).
+ * Q: [batch, seq_q, head_dim]; K, V: [batch, seq_kv, head_dim];
+ * mask: [batch, seq_q, seq_kv] of in_dtype, added to the scaled scores, or
+ * NULL; O: [batch, seq_q, head_dim]. The reference fixes
+ * sm_scale = 1/sqrt(head_dim); here the caller passes it. -inf mask entries
+ * remove a key; a row whose keys are all removed yields NaN, as the
+ * reference's max / sub / exp / div sequence does.
+ * in_dtype / out_dtype as for hexmi_flash_attn_fwd. */
+int hexmi_attention(const void *Q, const void *K, const void *V,
+                    const void *mask, void *O, int64_t batch, int64_t seq_q,
+                    int64_t seq_kv, int64_t head_dim, float sm_scale,
+                    int in_dtype, int out_dtype, hexmi_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,6 +20,9 @@
  *       power-of-two scale patterns, one-hot scales, edge weights +-127 / 0.
  *   attention (brute force) : F.scaled_dot_product_attention on CPU (fp32 and
  *       fp64), causal and full; row 0 of a causal result == V[0].
+ *   attention_masked        : F.scaled_dot_product_attention(attn_mask=...) on CPU,
+ *                             rectangular (Sq != Skv) and -inf masks; reduces to
+ *                             `attention` when mask == NULL and Sq == Skv
  *   attention_online        : the recurrence of the reference kernel, checked
  *       against the brute-force form.
  *
@@ -294,6 +297,39 @@ void oracle_attention(const void *Q, const void *K, const void *V, void *O, int6
       for (int64_t j = 0; j < jend; ++j)
         for (int64_t d = 0; d < D; ++d) acc[d] += p[j] * load_el(V, base + j * D + d, in_dtype);
       for (int64_t d = 0; d < D; ++d) store_el(O, base + i * D + d, out_dtype, acc[d] / l);
+      free(p);
+      free(acc);
+    }
+  }
+}
+
+/* tm_tensor.attention with its mask operand and separate query / key lengths
+ * (qcom_hexagon_backend/lib/Transforms/LowerTmTensor.cpp:88-99 shapes, :120-123 scale, :157-160 additive mask,
+ * :164-222 softmax, :225-229 P V). Q: [B, Sq, D]; K, V: [B, Skv, D]; mask: [B, Sq, Skv] of in_dtype or NULL. */
+void oracle_attention_masked(const void *Q, const void *K, const void *V, const void *mask, void *O, int64_t B,
+                             int64_t Sq, int64_t Skv, int64_t D, double scale, int in_dtype, int out_dtype) {
+#pragma omp parallel for schedule(dynamic, 4) collapse(2)
+  for (int64_t b = 0; b < B; ++b) {
+    for (int64_t i = 0; i < Sq; ++i) {
+      const int64_t qb = b * Sq * D, kb = b * Skv * D, mb = (b * Sq + i) * Skv;
+      double *p = (double *)malloc(sizeof(double) * (size_t)Skv);
+      double *acc = (double *)calloc((size_t)D, sizeof(double));
+      double m = -INFINITY;
+      for (int64_t j = 0; j < Skv; ++j) {
+        double s = 0.0;
+        for (int64_t d = 0; d < D; ++d)
+          s += load_el(Q, qb + i * D + d, in_dtype) * load_el(K, kb + j * D + d, in_dtype);
+        p[j] = s * scale + (mask ? load_el(mask, mb + j, in_dtype) : 0.0);
+        if (p[j] > m) m = p[j];
+      }
+      double l = 0.0;
+      for (int64_t j = 0; j < Skv; ++j) {
+        p[j] = exp(p[j] - m);                  /* m == -inf (every key removed): exp(nan), as the reference */
+        l += p[j];
+      }
+      for (int64_t j = 0; j < Skv; ++j)
+        for (int64_t d = 0; d < D; ++d) acc[d] += p[j] * load_el(V, kb + j * D + d, in_dtype);
+      for (int64_t d = 0; d < D; ++d) store_el(O, qb + i * D + d, out_dtype, acc[d] / l);
       free(p);
       free(acc);
     }

@@ -156,6 +156,25 @@ def attention(q, k, v, scale, causal, out_dtype=None, dtype=None):
     return o
 
 
+def attention_masked(q, k, v, mask, scale, out_dtype=None, dtype=None):
+    """q: [B,Sq,D]; k, v: [B,Skv,D]; mask: [B,Sq,Skv] or None; softmax(scale*QK^T + mask) V in double."""
+    q, k, v = _c(q), _c(k), _c(v)
+    B, Sq, D = q.shape
+    Skv = k.shape[1]
+    code_in = _code(q, dtype)
+    if mask is not None:
+        mask = _c(mask)
+        assert mask.shape == (B, Sq, Skv) and mask.dtype == q.dtype
+    if out_dtype is None:
+        o, code_out = np.empty_like(q), code_in
+    else:
+        o = np.empty(q.shape, out_dtype)
+        code_out = _code(o)
+    _l().oracle_attention_masked(_ptr(q), _ptr(k), _ptr(v), _ptr(mask) if mask is not None else None, _ptr(o),
+                                 _i64(B), _i64(Sq), _i64(Skv), _i64(D), _dbl(scale), _int(code_in), _int(code_out))
+    return o
+
+
 def attention_online_f32(q, k, v, sm_scale, block_n):
     q, k, v = _c(q), _c(k), _c(v)
     assert q.dtype == np.float32

@@ -43,3 +43,9 @@ def w8a16_matmul(a, w_int8, scales):
 def attention(q, k, v, scale, causal):
     """test/python/triton/test_flash_attention.py:212: F.scaled_dot_product_attention(q, k, v, scale=SCALE)."""
     return F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal, scale=scale)
+
+
+def attention_masked(q, k, v, mask, scale):
+    """tm_tensor.attention as torch states it: softmax(QK^T * scale + mask) V with an additive float mask."""
+    m = None if mask is None else mask.float()
+    return F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=m, scale=scale)

@@ -19,7 +19,7 @@ def _declared():
 def test_header_declares_expected_entry_points():
     names = _declared()
     for must in ("hexmi_softmax", "hexmi_rms_norm", "hexmi_layer_norm", "hexmi_matmul_f16f16_f32", "hexmi_gemm",
-                 "hexmi_gemm_w8a16", "hexmi_dequant_w8", "hexmi_flash_attn_fwd"):
+                 "hexmi_gemm_w8a16", "hexmi_dequant_w8", "hexmi_flash_attn_fwd", "hexmi_attention"):
         assert must in names
 
 

@@ -138,3 +138,85 @@ def test_attention_errors(hexmi):
     assert hexmi.flash_attention(torch.empty(1, 2, 0, 64, device="cuda", dtype=torch.float16),
                                  torch.empty(1, 2, 0, 64, device="cuda", dtype=torch.float16),
                                  torch.empty(1, 2, 0, 64, device="cuda", dtype=torch.float16)).shape == (1, 2, 0, 64)
+
+
+# ---- tm_tensor.attention: [B, S, D] operands, rectangular scores, additive mask -----------------------------
+def _oracle_masked(oracle, q, k, v, mask, scale):
+    qn, tag = to_np(q)
+    kn, _ = to_np(k)
+    vn, _ = to_np(v)
+    mn = None if mask is None else to_np(mask)[0]
+    return torch.from_numpy(oracle.attention_masked(qn, kn, vn, mn, scale, out_dtype=np.float32, dtype=tag))
+
+
+def _mask(B, Sq, Skv, dtype, seed, drop=0.3):
+    g = _gen(seed)
+    m = torch.randn(B, Sq, Skv, generator=g)
+    m[torch.rand(B, Sq, Skv, generator=g) < drop] = float("-inf")
+    m[:, :, 0] = 0.0                                   # every row keeps a key
+    return m.to(dtype)
+
+
+MASKED_CASES = [(2, 128, 128, 128), (3, 200, 72, 64), (1, 1, 64, 128), (2, 77, 516, 128), (1, 300, 4, 64),
+                (1, 130, 1024, 128), (2, 65, 66, 64), (1, 40, 100, 80)]   # the last two: Skv % 4 != 0 / other D
+
+
+@pytest.mark.parametrize("with_mask", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", MASKED_CASES)
+def test_masked_attention_parity_half(hexmi, oracle, case, dtype, with_mask):
+    B, Sq, Skv, D = case
+    g = _gen(21)
+    q = torch.randn(B, Sq, D, generator=g).to(dtype)
+    k, v = torch.randn(B, Skv, D, generator=g).to(dtype), torch.randn(B, Skv, D, generator=g).to(dtype)
+    mask = _mask(B, Sq, Skv, dtype, 22) if with_mask else None
+    scale = 1.0 / math.sqrt(D)
+    got = hexmi.attention(q.cuda(), k.cuda(), v.cuda(), None if mask is None else mask.cuda()).cpu()
+    want = _oracle_masked(oracle, q, k, v, mask, scale)
+    assert got.dtype == dtype and got.shape == (B, Sq, D)
+    assert (got.float() - want).abs().max() <= (2e-2 if dtype == torch.float16 else 4e-2)
+    got32 = hexmi.attention(q.cuda(), k.cuda(), v.cuda(), None if mask is None else mask.cuda(),
+                            out_dtype=torch.float32).cpu()
+    assert (got32 - want).abs().max() <= (5e-3 if dtype == torch.float16 else 3e-2)
+
+
+@pytest.mark.parametrize("case", [(2, 50, 70, 32), (1, 64, 64, 128), (1, 33, 129, 64)])
+def test_masked_attention_parity_fp32(hexmi, oracle, case):
+    B, Sq, Skv, D = case
+    g = _gen(23)
+    q, k, v = torch.rand(B, Sq, D, generator=g), torch.rand(B, Skv, D, generator=g), torch.rand(B, Skv, D, generator=g)
+    mask = _mask(B, Sq, Skv, torch.float32, 24)
+    got = hexmi.attention(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).cpu()
+    want = _oracle_masked(oracle, q, k, v, mask, 1.0 / math.sqrt(D))
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_masked_attention_properties(hexmi):
+    # a causal additive mask reproduces the causal kernel; a constant added to the mask changes nothing;
+    # host tensors are staged and `out` is filled in place
+    B, S, D = 2, 256, 128
+    g = _gen(25)
+    q, k, v = (torch.randn(B, S, D, generator=g).half() for _ in range(3))
+    tri = torch.full((S, S), float("-inf")).triu(1).half().expand(B, S, S).contiguous()
+    got = hexmi.attention(q.cuda(), k.cuda(), v.cuda(), tri.cuda()).cpu()
+    causal = hexmi.flash_attention(q.view(B, 1, S, D).cuda(), k.view(B, 1, S, D).cuda(), v.view(B, 1, S, D).cuda(),
+                                   None, True).cpu().view(B, S, D)
+    assert (got.float() - causal.float()).abs().max() <= 2e-3
+    shifted = hexmi.attention(q.cuda(), k.cuda(), v.cuda(), (tri + 2.0).cuda()).cpu()
+    assert (shifted.float() - got.float()).abs().max() <= 2e-3
+    out = torch.empty(B, S, D, dtype=torch.float16)
+    ret = hexmi.attention(q, k, v, tri, out=out)
+    assert ret is out and torch.equal(out, got)
+    with pytest.raises(ValueError):
+        hexmi.attention(q, k, v, tri[:, :, :-4])
+
+
+def test_masked_attention_fully_masked_row_is_nan(hexmi):
+    # LowerTmTensor.cpp:164-222: max = -inf, x - max = nan, exp / sum / div propagate it
+    B, S, D = 1, 64, 64
+    g = _gen(26)
+    q, k, v = (torch.randn(B, S, D, generator=g).half() for _ in range(3))
+    mask = torch.zeros(B, S, S).half()
+    mask[0, 5, :] = float("-inf")
+    got = hexmi.attention(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).cpu()
+    assert torch.isnan(got[0, 5]).all() and not torch.isnan(got[0, :5]).any() and not torch.isnan(got[0, 6:]).any()

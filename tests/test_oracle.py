@@ -282,6 +282,32 @@ def test_attention_causal_invariants(oracle):
     assert o16.dtype == np.float32 and np.allclose(o16, o, atol=2e-2)
 
 
+def test_attention_masked_vs_sdpa(oracle):
+    # tm_tensor.attention (LowerTmTensor.cpp:70-235): rectangular scores, additive mask with -inf entries
+    g = torch.Generator().manual_seed(18)
+    B, Sq, Skv, D = 3, 40, 72, 32
+    q = torch.randn(B, Sq, D, generator=g)
+    k, v = torch.randn(B, Skv, D, generator=g), torch.randn(B, Skv, D, generator=g)
+    mask = torch.randn(B, Sq, Skv, generator=g)
+    mask[torch.rand(B, Sq, Skv, generator=g) < 0.3] = float("-inf")
+    mask[:, :, 0] = 0.0                                                        # no row loses every key
+    scale = 1.0 / np.sqrt(D)
+    got = oracle.attention_masked(q.numpy(), k.numpy(), v.numpy(), mask.numpy(), scale)
+    want = F.scaled_dot_product_attention(q.double(), k.double(), v.double(), attn_mask=mask.double(), scale=scale)
+    assert np.allclose(got, want.numpy(), rtol=1e-5, atol=1e-6)
+    assert np.allclose(got, torch_cpu.attention_masked(q, k, v, mask, scale).numpy(), rtol=1e-4, atol=1e-5)
+    # no mask and Sq == Skv: the plain oracle; a causal additive mask: the causal oracle
+    q2 = torch.randn(B, Skv, D, generator=g)
+    plain = oracle.attention_masked(q2.numpy(), k.numpy(), v.numpy(), None, scale)
+    assert np.allclose(plain, oracle.attention(q2.numpy(), k.numpy(), v.numpy(), scale, False), rtol=1e-12, atol=0)
+    tri = torch.full((Skv, Skv), float("-inf")).triu(1).expand(B, Skv, Skv).contiguous()
+    causal = oracle.attention_masked(q2.numpy(), k.numpy(), v.numpy(), tri.numpy(), scale)
+    assert np.allclose(causal, oracle.attention(q2.numpy(), k.numpy(), v.numpy(), scale, True), rtol=1e-12, atol=0)
+    # a constant added to a whole mask row changes nothing (shift invariance of the softmax)
+    shifted = oracle.attention_masked(q.numpy(), k.numpy(), v.numpy(), (mask + 3.0).numpy(), scale)
+    assert np.allclose(shifted, got, rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize("block_n", [16, 64])
 def test_attention_online_recurrence(oracle, block_n):
     g = torch.Generator().manual_seed(17)
