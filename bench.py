@@ -233,6 +233,70 @@ class Attention(Workload):
         return t * (Z * H / heads), "%d of %d heads, fp32 F.scaled_dot_product_attention(is_causal=True) on CPU, time scaled" % (heads, Z * H)
 
 
+class Elementwise(Workload):
+    """The reference's small tutorial kernels at a size that needs HBM: GELU-tanh / SiLU over fp16 [8192,4096],
+    RoPE over fp16 [4,4096,32,128], one sum per 4096-element program over fp32 [8192*4096]."""
+    bound = "hbm"
+
+    def __init__(self, which):
+        self.which = which
+        self.name = {"gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096", "rope": "rope_f16_4x4096x32x128",
+                     "sum": "block_sum_f32_8192x4096"}[which]
+        self.kernel = {"gelu": "unary_kernel", "silu": "unary_kernel", "rope": "rope_kernel", "sum": "block_sum_kernel"}[which]
+        self.dtype = "f32" if which == "sum" else "f16"
+        self.desc = {"gelu": "GELU-tanh fp16 [8192,4096] N(0,1)", "silu": "SiLU fp16 [8192,4096] N(0,1)",
+                     "rope": "RoPE fp16 [batch 4, seq 4096, heads 32, features 128] N(0,1), theta 1e4",
+                     "sum": "8192 programs x 4096 fp32 elements, one sum each"}[which]
+
+    def setup(self, torch, hexmi):
+        g = torch.Generator().manual_seed(0)
+        self.hexmi = hexmi
+        if self.which == "rope":
+            x = torch.randn(4, 4096, 32, 128, generator=g).half()
+        elif self.which == "sum":
+            x = torch.randn(8192 * 4096, generator=g)
+        else:
+            x = torch.randn(8192, 4096, generator=g).half()
+        self.host = {"x": x}
+        n_bytes = x.numel() * x.element_size()
+        self.work = n_bytes + 8192 * 4 if self.which == "sum" else 2 * n_bytes
+        self.sets = _sets(torch, self.host, self.work)
+        for s in self.sets:
+            s["out"] = torch.empty(8192, device="cuda") if self.which == "sum" else torch.empty_like(s["x"])
+
+    def step(self, i):
+        s = self.sets[i % len(self.sets)]
+        if self.which == "gelu":
+            self.hexmi.gelu(s["x"], out=s["out"])
+        elif self.which == "silu":
+            self.hexmi.silu(s["x"], out=s["out"])
+        elif self.which == "rope":
+            self.hexmi.rope(s["x"], 10000.0, out=s["out"])
+        else:
+            self.hexmi.block_sum(s["x"], 4096, out=s["out"])
+
+    def cpu(self, torch):
+        import torch.nn.functional as F
+        x = self.host["x"]
+        if self.which == "gelu":
+            return _time_cpu(lambda: F.gelu(x, approximate="tanh"), 3), "full tensor, F.gelu(approximate='tanh') on CPU"
+        if self.which == "silu":
+            return _time_cpu(lambda: F.silu(x), 3), "full tensor, F.silu on CPU"
+        if self.which == "sum":
+            return _time_cpu(lambda: x.view(8192, 4096).sum(1), 3), "full tensor, torch.sum(dim=1) on CPU"
+        D, L = 128, 4096
+        idx = torch.arange(D, dtype=torch.float32)
+        steps = torch.where(idx % 2 == 0, idx, idx - 1)
+        ang = torch.arange(L, dtype=torch.float32)[:, None] * (1.0 / (10000.0 ** (steps / D)))[None, :]
+        cos, sin = torch.cos(ang).reshape(1, L, 1, D), torch.sin(ang).reshape(1, L, 1, D)
+        even = (torch.arange(D) % 2 == 0).view(1, 1, 1, D)
+        xs = x[:1]
+
+        def run():
+            torch.where(even, xs * cos - torch.roll(xs, -1, 3) * sin, torch.roll(xs, 1, 3) * sin + xs * cos)
+        return _time_cpu(run, 1) * 4, "1 of 4 batch entries, the reference's torch RoPE formula on CPU, time scaled"
+
+
 class MaskedAttention(Workload):
     """tm_tensor.attention with an additive mask (the next row after the causal kernel): [B,S,D] operands."""
     bound, dtype, kernel = "mfma", "f16", "flash_fwd_kernel"
@@ -283,13 +347,15 @@ def _time_cpu(fn, iters):
 def make_workloads():
     return {w.name: w for w in (
         Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
-        W8A16(1), W8A16(16), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128),
+        W8A16(1), W8A16(16), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
+        Elementwise("sum"),
         CopyCalibration())}
 
 
 ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "gemm": "gemm_f16_4096",
            "gemm_bf16": "gemm_bf16_8192", "attn": "attn_causal_f16_4x32x4096x128",
-           "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128", "rms_norm": "rms_norm_f16_8192x4096",
+           "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
+           "rope": "rope_f16_4x4096x32x128", "sum": "block_sum_f32_8192x4096", "rms_norm": "rms_norm_f16_8192x4096",
            "layer_norm": "layer_norm_f16_8192x4096"}
 
 

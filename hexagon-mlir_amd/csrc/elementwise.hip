@@ -1,0 +1,393 @@
+// Element-wise operators, block sums and rotary embedding: the small tutorial kernels of the reference
+// (GELU-tanh, SiLU, rsqrt / sin / cos / exp, vector add / sub / mul / div, sum reduction, RoPE). All are one pass
+// over HBM with 16-byte non-temporal accesses, four chunks in flight per thread, fp32 arithmetic.
+#include "hexmi_common.h"
+
+namespace hexmi {
+namespace {
+
+template <typename T> struct Chunk {                // one 16-byte global access
+  static constexpr int N = 16 / sizeof(T);
+  T v[N];
+};
+template <typename T>
+__device__ __forceinline__ Chunk<T> load_chunk(const T* p) {
+  Chunk<T> r;
+  *reinterpret_cast<u32x4*>(r.v) = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return r;
+}
+template <typename T>
+__device__ __forceinline__ void store_chunk(T* p, const Chunk<T>& r) {
+  __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(r.v), reinterpret_cast<u32x4*>(p));
+}
+
+// ---- unary ---------------------------------------------------------------------------------------------------
+template <int OP>
+__device__ __forceinline__ float unary(float x) {
+  if constexpr (OP == HEXMI_GELU_TANH) {
+    // 0.5*x*(1 + tanh(u)), u = 0.797885*x + 0.035677*x^3, tanh(u) = (1 - e^-2u) / (1 + e^-2u)
+    // (test/python/triton/test_gelu.py:26-30,54). 0.5*(1 + tanh(u)) = 1 / (1 + e^-2u): the same function without
+    // the cancellation in 1 + tanh(u) for negative u, and e^-2u = inf gives 0 instead of inf/inf.
+    // v_exp_f32 and v_rcp_f32 (1 ulp each) keep the kernel bound by HBM rather than by the vector ALUs
+    const float u = 0.797885f * x + 0.035677f * x * x * x;
+    return x * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
+  } else if constexpr (OP == HEXMI_SILU) {
+    return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x));   // x / (1 + e^-x), test/python/triton/test_silu.py:50
+  } else if constexpr (OP == HEXMI_RSQRT) {
+    return 1.0f / sqrtf(x);                          // test/python/triton/test_rsqrt.py:20-24
+  } else if constexpr (OP == HEXMI_SIN) {
+    return sinf(x);                                  // test/python/triton/test_math_ops.py:33-38
+  } else if constexpr (OP == HEXMI_COS) {
+    return cosf(x);                                  // test/python/triton/test_math_ops.py:25-30
+  } else {
+    return expf(x);
+  }
+}
+
+constexpr int kEwThreads = 256;
+constexpr int kEwChunks = 4;                         // 16-byte chunks per thread
+
+template <typename T, int OP>
+__global__ __launch_bounds__(kEwThreads)
+void unary_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n) {
+  constexpr int N = Chunk<T>::N;
+  const int64_t chunks = n / N;
+  const int64_t c0 = (int64_t)blockIdx.x * (kEwThreads * kEwChunks) + threadIdx.x;
+  Chunk<T> in[kEwChunks];
+#pragma unroll
+  for (int u = 0; u < kEwChunks; ++u) {
+    const int64_t c = c0 + u * kEwThreads;
+    in[u] = load_chunk(x + (c < chunks ? c : 0) * N);           // branch-free: out-of-range lanes re-read chunk 0
+  }
+#pragma unroll
+  for (int u = 0; u < kEwChunks; ++u) {
+    const int64_t c = c0 + u * kEwThreads;
+    Chunk<T> out;
+#pragma unroll
+    for (int i = 0; i < N; ++i) out.v[i] = from_f32<T>(unary<OP>(to_f32<T>(in[u].v[i])));
+    if (c < chunks) store_chunk(y + c * N, out);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < n % N) {                  // the few elements past the last whole chunk
+    const int64_t i = chunks * N + threadIdx.x;
+    y[i] = from_f32<T>(unary<OP>(to_f32<T>(x[i])));
+  }
+}
+
+// misaligned buffers: one element per thread
+template <typename T, int OP>
+__global__ __launch_bounds__(kEwThreads)
+void unary_scalar_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+  if (i < n) y[i] = from_f32<T>(unary<OP>(to_f32<T>(x[i])));
+}
+
+// ---- binary --------------------------------------------------------------------------------------------------
+template <int OP>
+__device__ __forceinline__ float binary(float a, float b) {
+  if constexpr (OP == HEXMI_ADD) return a + b;       // test/python/triton/test_vec_add.py
+  else if constexpr (OP == HEXMI_SUB) return a - b;
+  else if constexpr (OP == HEXMI_MUL) return a * b;
+  else return a / b;                                 // test/python/triton/test_vec_div_2d.py:52-55
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(kEwThreads)
+void binary_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ y, int64_t n) {
+  constexpr int N = Chunk<T>::N;
+  constexpr int CH = kEwChunks / 2;                  // two operands: the same number of loads in flight
+  const int64_t chunks = n / N;
+  const int64_t c0 = (int64_t)blockIdx.x * (kEwThreads * CH) + threadIdx.x;
+  Chunk<T> ia[CH], ib[CH];
+#pragma unroll
+  for (int u = 0; u < CH; ++u) {
+    const int64_t c = c0 + u * kEwThreads;
+    ia[u] = load_chunk(a + (c < chunks ? c : 0) * N);
+    ib[u] = load_chunk(b + (c < chunks ? c : 0) * N);
+  }
+#pragma unroll
+  for (int u = 0; u < CH; ++u) {
+    const int64_t c = c0 + u * kEwThreads;
+    Chunk<T> out;
+#pragma unroll
+    for (int i = 0; i < N; ++i) out.v[i] = from_f32<T>(binary<OP>(to_f32<T>(ia[u].v[i]), to_f32<T>(ib[u].v[i])));
+    if (c < chunks) store_chunk(y + c * N, out);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < n % N) {
+    const int64_t i = chunks * N + threadIdx.x;
+    y[i] = from_f32<T>(binary<OP>(to_f32<T>(a[i]), to_f32<T>(b[i])));
+  }
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(kEwThreads)
+void binary_scalar_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ y, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+  if (i < n) y[i] = from_f32<T>(binary<OP>(to_f32<T>(a[i]), to_f32<T>(b[i])));
+}
+
+// ---- block sums ----------------------------------------------------------------------------------------------
+// out[p] = sum(x[p*block .. (p+1)*block)), one workgroup per program of the reference's launch grid
+// (test/python/triton/test_sum.py:30-36: `tl.store(output_ptr + pid, tl.sum(x))`). fp32 accumulation in a fixed
+// order (per-thread strided partials, wave butterfly, waves in order): the result does not depend on timing.
+constexpr int kSumThreads = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(kSumThreads)
+void block_sum_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t block, int64_t n) {
+  constexpr int N = Chunk<T>::N;
+  __shared__ float part[kSumThreads / kWave];
+  const int64_t begin = (int64_t)blockIdx.x * block;
+  const int64_t end = begin + block < n ? begin + block : n;
+  const T* xb = x + begin;
+  const int64_t len = end - begin;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool vec = reinterpret_cast<uintptr_t>(xb) % 16 == 0;
+  const int64_t chunks = vec ? len / N : 0;
+  int64_t c = threadIdx.x;
+  for (; c + 3 * kSumThreads < chunks; c += 4 * kSumThreads) {   // four loads in flight
+    Chunk<T> v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = load_chunk(xb + (c + u * kSumThreads) * N);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < N; ++i) acc[u] += to_f32<T>(v[u].v[i]);
+  }
+  for (; c < chunks; c += kSumThreads) {
+    const Chunk<T> v = load_chunk(xb + c * N);
+#pragma unroll
+    for (int i = 0; i < N; ++i) acc[0] += to_f32<T>(v.v[i]);
+  }
+  for (int64_t i = chunks * N + threadIdx.x; i < len; i += kSumThreads) acc[1] += to_f32<T>(xb[i]);
+  float s = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
+  if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSumThreads / kWave; ++w) t += part[w];
+    out[blockIdx.x] = from_f32<T>(t);
+  }
+}
+
+// ---- rotary embedding ----------------------------------------------------------------------------------------
+// x, y: [batch, seq, heads, feat] contiguous; features are rotated in adjacent pairs (2i, 2i+1) by the angle
+// m * theta^(-2i/feat), m the sequence position (test/python/triton/test_rope.py:43-57 compute_thetas,
+// :60-95 rope_reference_pytorch, :174-184 even / odd cases):
+//   y[2i] = x[2i] cos - x[2i+1] sin,   y[2i+1] = x[2i] sin + x[2i+1] cos.
+// A workgroup owns one sequence position; a thread owns one 16-byte chunk of the feature vector, computes the
+// sines and cosines of its pairs once (in double: the angle m*freq is accurate to fp32 for any m) and walks all
+// (batch, head) rows with them.
+template <typename T>
+__global__ __launch_bounds__(256)
+void rope_kernel(const T* __restrict__ x, T* __restrict__ y, int batch, int seq, int heads, int feat, double log2_theta) {
+  constexpr int N = Chunk<T>::N;                     // elements per chunk (even)
+  const int chunks = feat / N;                       // chunks per feature vector (feat % N == 0 on this path)
+  const int rows_per_pass = 256 / chunks;            // (batch, head) rows handled side by side
+  const int m = blockIdx.x;
+  const int ch = threadIdx.x % chunks;
+  const int r0 = threadIdx.x / chunks;
+  if (r0 >= rows_per_pass) return;
+  float cs[N / 2], sn[N / 2];
+#pragma unroll
+  for (int p = 0; p < N / 2; ++p) {
+    const int i2 = ch * N + 2 * p;                   // even feature index = the reference's `steps`
+    const double freq = exp2(-((double)i2 / (double)feat) * log2_theta);
+    double s, c;
+    sincos((double)m * freq, &s, &c);
+    cs[p] = (float)c;
+    sn[p] = (float)s;
+  }
+  const int64_t rows = (int64_t)batch * heads;
+  for (int64_t r = r0 + (int64_t)blockIdx.y * rows_per_pass; r < rows; r += (int64_t)rows_per_pass * gridDim.y) {
+    const int64_t b = r / heads, h = r % heads;
+    const int64_t off = (((b * seq + m) * heads) + h) * feat + ch * N;
+    const Chunk<T> in = load_chunk(x + off);
+    Chunk<T> out;
+#pragma unroll
+    for (int p = 0; p < N / 2; ++p) {
+      const float e = to_f32<T>(in.v[2 * p]), o = to_f32<T>(in.v[2 * p + 1]);
+      out.v[2 * p] = from_f32<T>(e * cs[p] - o * sn[p]);
+      out.v[2 * p + 1] = from_f32<T>(e * sn[p] + o * cs[p]);
+    }
+    store_chunk(y + off, out);
+  }
+}
+
+// any feat (even), any alignment: one pair per thread
+template <typename T>
+__global__ __launch_bounds__(256)
+void rope_pair_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t pairs_total, int seq, int heads, int feat,
+                      double log2_theta) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= pairs_total) return;
+  const int half = feat / 2;
+  const int p = (int)(idx % half);
+  const int64_t row = idx / half;                    // (b*seq + m)*heads + h
+  const int m = (int)((row / heads) % seq);
+  const double freq = exp2(-((double)(2 * p) / (double)feat) * log2_theta);
+  double s, c;
+  sincos((double)m * freq, &s, &c);
+  const int64_t off = row * feat + 2 * p;
+  const float e = to_f32<T>(x[off]), o = to_f32<T>(x[off + 1]);
+  y[off] = from_f32<T>(e * (float)c - o * (float)s);
+  y[off + 1] = from_f32<T>(e * (float)s + o * (float)c);
+}
+
+// ---- dispatch ------------------------------------------------------------------------------------------------
+template <typename T, int OP>
+int launch_unary(const void* xv, void* yv, int64_t n, hipStream_t s) {
+  const T* x = static_cast<const T*>(xv);
+  T* y = static_cast<T*>(yv);
+  constexpr int N = 16 / sizeof(T);
+  if (aligned_to(x, 16) && aligned_to(y, 16) && n >= N) {
+    const int64_t chunks = n / N;
+    const int64_t blocks = (chunks + kEwThreads * kEwChunks - 1) / (kEwThreads * kEwChunks);
+    if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+    hipLaunchKernelGGL((unary_kernel<T, OP>), dim3((unsigned)blocks), dim3(kEwThreads), 0, s, x, y, n);
+  } else {
+    const int64_t blocks = (n + kEwThreads - 1) / kEwThreads;
+    if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+    hipLaunchKernelGGL((unary_scalar_kernel<T, OP>), dim3((unsigned)blocks), dim3(kEwThreads), 0, s, x, y, n);
+  }
+  return launch_status();
+}
+
+template <typename T>
+int dispatch_unary(int op, const void* x, void* y, int64_t n, hipStream_t s) {
+  switch (op) {
+    case HEXMI_GELU_TANH: return launch_unary<T, HEXMI_GELU_TANH>(x, y, n, s);
+    case HEXMI_SILU: return launch_unary<T, HEXMI_SILU>(x, y, n, s);
+    case HEXMI_RSQRT: return launch_unary<T, HEXMI_RSQRT>(x, y, n, s);
+    case HEXMI_SIN: return launch_unary<T, HEXMI_SIN>(x, y, n, s);
+    case HEXMI_COS: return launch_unary<T, HEXMI_COS>(x, y, n, s);
+    case HEXMI_EXP: return launch_unary<T, HEXMI_EXP>(x, y, n, s);
+    default: return HEXMI_EINVAL;
+  }
+}
+
+template <typename T, int OP>
+int launch_binary(const void* av, const void* bv, void* yv, int64_t n, hipStream_t s) {
+  const T* a = static_cast<const T*>(av);
+  const T* b = static_cast<const T*>(bv);
+  T* y = static_cast<T*>(yv);
+  constexpr int N = 16 / sizeof(T);
+  if (aligned_to(a, 16) && aligned_to(b, 16) && aligned_to(y, 16) && n >= N) {
+    const int64_t chunks = n / N;
+    const int64_t per_block = kEwThreads * (kEwChunks / 2);
+    const int64_t blocks = (chunks + per_block - 1) / per_block;
+    if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+    hipLaunchKernelGGL((binary_kernel<T, OP>), dim3((unsigned)blocks), dim3(kEwThreads), 0, s, a, b, y, n);
+  } else {
+    const int64_t blocks = (n + kEwThreads - 1) / kEwThreads;
+    if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+    hipLaunchKernelGGL((binary_scalar_kernel<T, OP>), dim3((unsigned)blocks), dim3(kEwThreads), 0, s, a, b, y, n);
+  }
+  return launch_status();
+}
+
+template <typename T>
+int dispatch_binary(int op, const void* a, const void* b, void* y, int64_t n, hipStream_t s) {
+  switch (op) {
+    case HEXMI_ADD: return launch_binary<T, HEXMI_ADD>(a, b, y, n, s);
+    case HEXMI_SUB: return launch_binary<T, HEXMI_SUB>(a, b, y, n, s);
+    case HEXMI_MUL: return launch_binary<T, HEXMI_MUL>(a, b, y, n, s);
+    case HEXMI_DIV: return launch_binary<T, HEXMI_DIV>(a, b, y, n, s);
+    default: return HEXMI_EINVAL;
+  }
+}
+
+template <typename T>
+int launch_block_sum(const void* x, void* out, int64_t n, int64_t block, hipStream_t s) {
+  const int64_t programs = (n + block - 1) / block;
+  if (programs > 0x7fffffff) return HEXMI_ENOTSUP;
+  hipLaunchKernelGGL((block_sum_kernel<T>), dim3((unsigned)programs), dim3(kSumThreads), 0, s,
+                     static_cast<const T*>(x), static_cast<T*>(out), block, n);
+  return launch_status();
+}
+
+template <typename T>
+int launch_rope(const void* xv, void* yv, int64_t batch, int64_t seq, int64_t heads, int64_t feat, double theta,
+                hipStream_t s) {
+  const T* x = static_cast<const T*>(xv);
+  T* y = static_cast<T*>(yv);
+  constexpr int N = 16 / sizeof(T);
+  const double log2_theta = log2(theta);
+  if (aligned_to(x, 16) && aligned_to(y, 16) && feat % N == 0 && feat / N <= 256) {
+    // enough workgroups to fill the chip when the sequence is short: split the (batch, head) rows over grid.y
+    const int64_t passes = (batch * heads + 256 / (feat / N) - 1) / (256 / (feat / N));
+    int64_t split = (2048 + seq - 1) / seq;
+    split = split < passes ? split : passes;
+    split = split < 65535 ? split : 65535;
+    hipLaunchKernelGGL((rope_kernel<T>), dim3((unsigned)seq, (unsigned)split), dim3(256), 0, s, x, y, (int)batch,
+                       (int)seq, (int)heads, (int)feat, log2_theta);
+  } else {
+    const int64_t pairs = batch * seq * heads * (feat / 2);
+    const int64_t blocks = (pairs + 255) / 256;
+    if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+    hipLaunchKernelGGL((rope_pair_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, x, y, pairs, (int)seq,
+                       (int)heads, (int)feat, log2_theta);
+  }
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace hexmi
+
+using namespace hexmi;
+
+extern "C" int hexmi_unary(int op, const void* x, void* y, int64_t n, int dtype, hexmi_stream_t stream) {
+  if (n < 0 || op < 0 || op > HEXMI_EXP) return HEXMI_EINVAL;
+  if (n == 0) return HEXMI_OK;
+  if (!x || !y) return HEXMI_EINVAL;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case HEXMI_F32: return dispatch_unary<float>(op, x, y, n, s);
+    case HEXMI_F16: return dispatch_unary<f16>(op, x, y, n, s);
+    case HEXMI_BF16: return dispatch_unary<bf16>(op, x, y, n, s);
+    default: return HEXMI_ENOTSUP;
+  }
+}
+
+extern "C" int hexmi_binary(int op, const void* a, const void* b, void* y, int64_t n, int dtype,
+                            hexmi_stream_t stream) {
+  if (n < 0 || op < 0 || op > HEXMI_DIV) return HEXMI_EINVAL;
+  if (n == 0) return HEXMI_OK;
+  if (!a || !b || !y) return HEXMI_EINVAL;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case HEXMI_F32: return dispatch_binary<float>(op, a, b, y, n, s);
+    case HEXMI_F16: return dispatch_binary<f16>(op, a, b, y, n, s);
+    case HEXMI_BF16: return dispatch_binary<bf16>(op, a, b, y, n, s);
+    default: return HEXMI_ENOTSUP;
+  }
+}
+
+extern "C" int hexmi_block_sum(const void* x, void* out, int64_t n, int64_t block, int dtype,
+                               hexmi_stream_t stream) {
+  if (n < 0 || block <= 0) return HEXMI_EINVAL;
+  if (n == 0) return HEXMI_OK;
+  if (!x || !out) return HEXMI_EINVAL;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case HEXMI_F32: return launch_block_sum<float>(x, out, n, block, s);
+    case HEXMI_F16: return launch_block_sum<f16>(x, out, n, block, s);
+    case HEXMI_BF16: return launch_block_sum<bf16>(x, out, n, block, s);
+    default: return HEXMI_ENOTSUP;
+  }
+}
+
+extern "C" int hexmi_rope(const void* x, void* y, int64_t batch, int64_t seq, int64_t heads, int64_t feat,
+                          double theta, int dtype, hexmi_stream_t stream) {
+  if (batch < 0 || seq < 0 || heads < 0 || feat < 0 || feat % 2 != 0 || !(theta > 0.0)) return HEXMI_EINVAL;
+  if (batch == 0 || seq == 0 || heads == 0 || feat == 0) return HEXMI_OK;
+  if (!x || !y) return HEXMI_EINVAL;
+  if (batch > 0x7fffffff || seq > 0x7fffffff || heads > 0x7fffffff || feat > 0x7fffffff) return HEXMI_ENOTSUP;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case HEXMI_F32: return launch_rope<float>(x, y, batch, seq, heads, feat, theta, s);
+    case HEXMI_F16: return launch_rope<f16>(x, y, batch, seq, heads, feat, theta, s);
+    case HEXMI_BF16: return launch_rope<bf16>(x, y, batch, seq, heads, feat, theta, s);
+    default: return HEXMI_ENOTSUP;
+  }
+}

@@ -21,7 +21,7 @@ class HexmiError(RuntimeError):
 
 
 _c = ctypes
-_i64, _int, _f32, _ptr = _c.c_int64, _c.c_int, _c.c_float, _c.c_void_p
+_i64, _int, _f32, _f64, _ptr = _c.c_int64, _c.c_int, _c.c_float, _c.c_double, _c.c_void_p
 
 # name -> (restype, argtypes); must list every symbol of include/hexmi.h
 SIGNATURES = {
@@ -36,6 +36,10 @@ SIGNATURES = {
     "hexmi_gemm_w8a16": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_dequant_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_flash_attn_fwd": (_int, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _ptr]),
+    "hexmi_unary": (_int, [_int, _ptr, _ptr, _i64, _int, _ptr]),
+    "hexmi_binary": (_int, [_int, _ptr, _ptr, _ptr, _i64, _int, _ptr]),
+    "hexmi_block_sum": (_int, [_ptr, _ptr, _i64, _i64, _int, _ptr]),
+    "hexmi_rope": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _f64, _int, _ptr]),
     "hexmi_attention": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _ptr]),
 }
 

@@ -114,3 +114,100 @@ def attention_fwd_kernel(pid1, Q, K, V, sm_scale, Out, H, N_CTX, BLOCK_M=None, B
     if STAGE not in (1, 3):
         raise ValueError("attention_fwd_kernel: STAGE must be 1 (full) or 3 (causal)")
     ops.flash_attention(Q, K, V, sm_scale, causal=(STAGE == 3), out=Out)
+
+
+def _check_block(name, t, BLOCK_SIZE, programs):
+    if BLOCK_SIZE is not None and BLOCK_SIZE * programs < t.numel():
+        raise ValueError("%s: grid of %d programs x BLOCK_SIZE %d does not cover %d elements"
+                         % (name, programs, BLOCK_SIZE, t.numel()))
+
+
+@Kernel
+def gelu_kernel(x_ptr, output_ptr, BLOCK_SIZE=None):
+    """test/python/triton/test_gelu.py:43-54."""
+    ops.unary("gelu_tanh", x_ptr, out=output_ptr)
+
+
+@Kernel
+def silu_kernel(x_ptr, output_ptr, BLOCK_SIZE=None):
+    """test/python/triton/test_silu.py:43-52."""
+    ops.unary("silu", x_ptr, out=output_ptr)
+
+
+@Kernel
+def rsqrt_kernel(x_ptr, output_ptr, BLOCK_SIZE=None):
+    """test/python/triton/test_rsqrt.py:20-24."""
+    ops.unary("rsqrt", x_ptr, out=output_ptr)
+
+
+@Kernel
+def sin_kernel(x_ptr, output_ptr, BLOCK_SIZE=None):
+    """test/python/triton/test_math_ops.py:33-38."""
+    ops.unary("sin", x_ptr, out=output_ptr)
+
+
+@Kernel
+def cos_kernel(x_ptr, output_ptr, BLOCK_SIZE=None):
+    """test/python/triton/test_math_ops.py:25-30."""
+    ops.unary("cos", x_ptr, out=output_ptr)
+
+
+@Kernel
+def add_kernel(x_ptr, y_ptr, output_ptr, n_elements=None, BLOCK_SIZE=None):
+    """test/python/triton/test_vec_add.py (and test_vec_add_with_scalar.py:32-46: n_elements masks the tail)."""
+    if n_elements is not None and n_elements != x_ptr.numel():
+        ops.binary("add", x_ptr.reshape(-1)[:n_elements], y_ptr.reshape(-1)[:n_elements],
+                   out=output_ptr.reshape(-1)[:n_elements])
+    else:
+        ops.binary("add", x_ptr, y_ptr, out=output_ptr)
+
+
+add_kernel_scalar = add_kernel
+
+
+@Kernel
+def div_kernel(x_ptr, y_ptr, output_ptr, NUM_ROWS=None, NUM_COLS=None):
+    """test/python/triton/test_vec_div_2d.py:21-55."""
+    if NUM_ROWS is not None and NUM_COLS is not None:
+        _check_2d("div_kernel", x_ptr, NUM_ROWS, NUM_COLS)
+    ops.binary("div", x_ptr, y_ptr, out=output_ptr)
+
+
+class _SumKernel(Kernel):
+    """`sum_kernel[grid](x, out, BLOCK_SIZE=...)` writes one sum per program, so the launch needs the grid."""
+
+    def __getitem__(self, grid):
+        launch = super().__getitem__(grid)
+        g = tuple(grid) if isinstance(grid, (tuple, list)) else (grid,)
+        programs = math.prod(int(v) for v in g)
+
+        def with_grid(*args, **kwargs):
+            return launch(*args, _programs=programs, **kwargs)
+
+        return with_grid
+
+
+@_SumKernel
+def sum_kernel(x_ptr, output_ptr, BLOCK_SIZE=None, _programs=1):
+    """test/python/triton/test_sum.py:30-36: program p stores the sum of elements [p*BLOCK_SIZE, (p+1)*BLOCK_SIZE)."""
+    if BLOCK_SIZE is None:
+        BLOCK_SIZE = x_ptr.numel()
+    _check_block("sum_kernel", x_ptr, BLOCK_SIZE, _programs)
+    if output_ptr.numel() < _programs:
+        raise ValueError("sum_kernel: output must hold one element per program")
+    n = min(x_ptr.numel(), BLOCK_SIZE * _programs)
+    used = (n + BLOCK_SIZE - 1) // BLOCK_SIZE
+    ops.block_sum(x_ptr.reshape(-1)[:n], BLOCK_SIZE, out=output_ptr.reshape(-1)[:used])
+
+
+@Kernel
+def rope_kernel(x_ptr, output_ptr, BATCH_SIZE, BATCH_SIZE_STRIDE, SEQ_LEN, SEQ_LEN_STRIDE, N_HEADS, N_HEADS_STRIDE,
+                N_FEATURES, N_FEATURES_STRIDE, BLOCK_SIZE=None, THETA=10000.0):
+    """test/python/triton/test_rope.py:97-197; only the contiguous [B, L, H, F] strides are supported."""
+    want = (SEQ_LEN * N_HEADS * N_FEATURES, N_HEADS * N_FEATURES, N_FEATURES, 1)
+    if (BATCH_SIZE_STRIDE, SEQ_LEN_STRIDE, N_HEADS_STRIDE, N_FEATURES_STRIDE) != want:
+        raise ValueError("rope_kernel: only the contiguous strides %s are supported" % (want,))
+    if x_ptr.numel() != BATCH_SIZE * want[0]:
+        raise ValueError("rope_kernel: tensor does not have BATCH_SIZE*SEQ_LEN*N_HEADS*N_FEATURES elements")
+    shape = (BATCH_SIZE, SEQ_LEN, N_HEADS, N_FEATURES)
+    ops.rope(x_ptr.view(shape), THETA, out=output_ptr.view(shape))

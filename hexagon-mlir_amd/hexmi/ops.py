@@ -47,6 +47,10 @@ _LIBDEF.define("matmul(Tensor a, Tensor b, bool trans_b, Tensor(a!) out) -> ()")
 _LIBDEF.define("w8a16_matmul(Tensor a, Tensor w, Tensor scales, Tensor(a!) out) -> ()")
 _LIBDEF.define("dequant_w8(Tensor w, Tensor scales, Tensor(a!) out) -> ()")
 _LIBDEF.define("flash_attention(Tensor q, Tensor k, Tensor v, float sm_scale, bool causal, Tensor(a!) out) -> ()")
+_LIBDEF.define("unary(int op, Tensor x, Tensor(a!) out) -> ()")
+_LIBDEF.define("binary(int op, Tensor a, Tensor b, Tensor(a!) out) -> ()")
+_LIBDEF.define("block_sum(Tensor x, int block, Tensor(a!) out) -> ()")
+_LIBDEF.define("rope(Tensor x, float theta, Tensor(a!) out) -> ()")
 _LIBDEF.define("attention(Tensor q, Tensor k, Tensor v, Tensor? mask, float sm_scale, Tensor(a!) out) -> ()")
 
 
@@ -109,9 +113,32 @@ def _attention_impl(q, k, v, mask, sm_scale, out):
                                               _dt(q), _dt(out), _stream()), "hexmi_attention")
 
 
+def _unary_impl(op, x, out):
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().hexmi_unary(op, _p(x), _p(out), x.numel(), _dt(x), _stream()), "hexmi_unary")
+
+
+def _binary_impl(op, a, b, out):
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().hexmi_binary(op, _p(a), _p(b), _p(out), a.numel(), _dt(a), _stream()), "hexmi_binary")
+
+
+def _block_sum_impl(x, block, out):
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().hexmi_block_sum(_p(x), _p(out), x.numel(), block, _dt(x), _stream()), "hexmi_block_sum")
+
+
+def _rope_impl(x, theta, out):
+    B, L, H, D = x.shape
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().hexmi_rope(_p(x), _p(out), B, L, H, D, theta, _dt(x), _stream()), "hexmi_rope")
+
+
 for _name, _fn in (("softmax", _softmax_impl), ("rms_norm", _rms_norm_impl), ("layer_norm", _layer_norm_impl),
                    ("matmul", _matmul_impl), ("w8a16_matmul", _w8a16_impl), ("dequant_w8", _dequant_impl),
-                   ("flash_attention", _flash_impl), ("attention", _attention_impl)):
+                   ("flash_attention", _flash_impl), ("attention", _attention_impl),
+                   ("unary", _unary_impl), ("binary", _binary_impl), ("block_sum", _block_sum_impl),
+                   ("rope", _rope_impl)):
     _LIBDEF.impl(_name, _fn, "CUDA")
 
 
@@ -291,4 +318,72 @@ def attention(q, k, v, mask=None, sm_scale=None, out=None, out_dtype=None):
     qd, kd, vd, md = _stage(q, dev), _stage(k, dev), _stage(v, dev), _stage(mask, dev)
     od = _out_like(out, q.shape, out_dtype, dev)
     torch.ops.hexmi.attention(qd, kd, vd, md, float(sm_scale), od)
+    return _finish(od, out)
+
+
+UNARY_OPS = {"gelu_tanh": 0, "silu": 1, "rsqrt": 2, "sin": 3, "cos": 4, "exp": 5}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def unary(op, x, out=None):
+    """Element-wise `op` in UNARY_OPS ("gelu_tanh": test/python/triton/test_gelu.py:43-54, "silu": test_silu.py:43-52,
+    "rsqrt": test_rsqrt.py:20-24, "sin" / "cos": test_math_ops.py:25-38, "exp")."""
+    if op not in UNARY_OPS:
+        raise ValueError("hexmi.unary: unknown op %r" % (op,))
+    dev = _device() if x.device.type != "cuda" else x.device
+    xd = _stage(x, dev)
+    od = _out_like(out, x.shape, x.dtype, dev)
+    torch.ops.hexmi.unary(UNARY_OPS[op], xd, od)
+    return _finish(od, out)
+
+
+def gelu(x, out=None):
+    """`F.gelu(x, approximate="tanh")` (test/python/triton/test_gelu.py:73)."""
+    return unary("gelu_tanh", x, out)
+
+
+def silu(x, out=None):
+    """`F.silu(x)` (test/python/triton/test_silu.py:69)."""
+    return unary("silu", x, out)
+
+
+def binary(op, a, b, out=None):
+    """Element-wise a (op) b for same-shape tensors, op in BINARY_OPS (test/python/triton/test_vec_add.py,
+    test_vec_div_2d.py:21-55)."""
+    if op not in BINARY_OPS:
+        raise ValueError("hexmi.binary: unknown op %r" % (op,))
+    if a.shape != b.shape or a.dtype != b.dtype:
+        raise ValueError("hexmi.binary: operands must share shape and dtype")
+    dev = _device() if a.device.type != "cuda" else a.device
+    ad, bd = _stage(a, dev), _stage(b, dev)
+    od = _out_like(out, a.shape, a.dtype, dev)
+    torch.ops.hexmi.binary(BINARY_OPS[op], ad, bd, od)
+    return _finish(od, out)
+
+
+def block_sum(x, block=None, out=None):
+    """out[p] = sum of the p-th run of `block` elements of x (flattened); block=None sums everything into out[0]
+    (`torch.sum(x)`, test/python/triton/test_sum.py:30-47)."""
+    n = x.numel()
+    if block is None:
+        block = max(n, 1)
+    if block < 1:
+        raise ValueError("hexmi.block_sum: block must be positive")
+    programs = (n + block - 1) // block
+    dev = _device() if x.device.type != "cuda" else x.device
+    xd = _stage(x, dev).reshape(-1)
+    od = _out_like(out, (programs,), x.dtype, dev)
+    torch.ops.hexmi.block_sum(xd, int(block), od)
+    return _finish(od, out)
+
+
+def rope(x, theta=10000.0, out=None):
+    """Rotary embedding of x [batch, seq, heads, features] over adjacent feature pairs
+    (`rope_reference_pytorch`, test/python/triton/test_rope.py:60-95)."""
+    if x.dim() != 4 or x.shape[-1] % 2 != 0:
+        raise ValueError("hexmi.rope: x must be [batch, seq, heads, features] with an even feature count")
+    dev = _device() if x.device.type != "cuda" else x.device
+    xd = _stage(x, dev)
+    od = _out_like(out, x.shape, x.dtype, dev)
+    torch.ops.hexmi.rope(xd, float(theta), od)
     return _finish(od, out)

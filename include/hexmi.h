@@ -156,6 +156,55 @@ int hexmi_attention(const void *Q, const void *K, const void *V,
                     int64_t seq_kv, int64_t head_dim, float sm_scale,
                     int in_dtype, int out_dtype, hexmi_stream_t stream);
 
+/* Element-wise operators, sum reduction, rotary embedding ------------------ */
+
+/* y[i] = f(x[i]), fp32 arithmetic, result rounded to `dtype`.
+ * HEXMI_GELU_TANH: 0.5*x*(1 + tanh(0.797885*x + 0.035677*x^3)), the `gelu_kernel`
+ *   of test/python/triton/test_gelu.py:43-54 (checked there against
+ *   F.gelu(x, approximate="tanh"));
+ * HEXMI_SILU: x / (1 + exp(-x)), `silu_kernel` of test/python/triton/test_silu.py:43-52;
+ * HEXMI_RSQRT: test/python/triton/test_rsqrt.py:20-24;
+ * HEXMI_SIN / HEXMI_COS: test/python/triton/test_math_ops.py:25-38; HEXMI_EXP. */
+typedef enum hexmi_unary_op {
+  HEXMI_GELU_TANH = 0,
+  HEXMI_SILU = 1,
+  HEXMI_RSQRT = 2,
+  HEXMI_SIN = 3,
+  HEXMI_COS = 4,
+  HEXMI_EXP = 5
+} hexmi_unary_op;
+int hexmi_unary(int op, const void *x, void *y, int64_t n, int dtype,
+                hexmi_stream_t stream);
+
+/* y[i] = a[i] (+ - * /) b[i]: `add_kernel` of test/python/triton/test_vec_add.py
+ * (and test_vec_add_with_scalar.py:32-46, test_vec_add_2d.py), `div_kernel` of
+ * test/python/triton/test_vec_div_2d.py:21-55. 2-D contiguous operands are the
+ * same call with n = rows*cols. */
+typedef enum hexmi_binary_op {
+  HEXMI_ADD = 0,
+  HEXMI_SUB = 1,
+  HEXMI_MUL = 2,
+  HEXMI_DIV = 3
+} hexmi_binary_op;
+int hexmi_binary(int op, const void *a, const void *b, void *y, int64_t n,
+                 int dtype, hexmi_stream_t stream);
+
+/* out[p] = sum(x[p*block .. min((p+1)*block, n))) for p < ceil(n/block): the
+ * `sum_kernel` of test/python/triton/test_sum.py:30-36 launched on a grid of
+ * ceil(n/block) programs with BLOCK_SIZE = block (the test uses one program over
+ * 1024*1024 elements). fp32 accumulation in a fixed order; out has `dtype`. */
+int hexmi_block_sum(const void *x, void *out, int64_t n, int64_t block,
+                    int dtype, hexmi_stream_t stream);
+
+/* Rotary position embedding of x [batch, seq, heads, feat] (contiguous, feat
+ * even): adjacent feature pairs (2i, 2i+1) are rotated by m * theta^(-2i/feat),
+ * m the sequence position: `rope_kernel` of test/python/triton/test_rope.py:97-197
+ * (angles `compute_thetas` :43-57, even / odd cases :174-184, torch form
+ * `rope_reference_pytorch` :60-95). */
+int hexmi_rope(const void *x, void *y, int64_t batch, int64_t seq,
+               int64_t heads, int64_t feat, double theta, int dtype,
+               hexmi_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,11 @@
  *                             `attention` when mask == NULL and Sq == Skv
  *   attention_online        : the recurrence of the reference kernel, checked
  *       against the brute-force form.
+ *   unary (gelu_tanh, silu, rsqrt, sin, cos, exp), binary, block_sum, rope :
+ *       F.gelu(approximate="tanh") / F.silu / torch.rsqrt / sin / cos on CPU (the
+ *       reference tests' own oracles and tolerances); torch.sum; the reference's
+ *       rope_reference_pytorch formula re-stated with torch ops in the test and
+ *       the closed forms "position 0 is the identity" / "pairs keep their norm".
  *
  * Storage types: fp16 and bf16 travel as uint16_t bit patterns.
  */
@@ -380,4 +385,62 @@ void oracle_attention_online_f32(const float *Q, const float *K, const float *V,
   }
   free(acc);
   free(qk);
+}
+
+/* ---- element-wise operators, block sums, rotary embedding -------------------
+ * op codes as hexmi_unary_op / hexmi_binary_op. */
+void oracle_unary(int op, const void *x, void *y, int64_t n, int dtype) {
+#pragma omp parallel for
+  for (int64_t i = 0; i < n; ++i) {
+    const double v = load_el(x, i, dtype);
+    double r;
+    switch (op) {
+      case 0: { /* gelu_kernel, test/python/triton/test_gelu.py:26-30,54 (its own constants) */
+        const double u = 0.797885 * v + 0.035677 * v * v * v;
+        r = 0.5 * v * (1.0 + tanh(u));
+        break;
+      }
+      case 1: r = v / (1.0 + exp(-v)); break;            /* test_silu.py:50 */
+      case 2: r = 1.0 / sqrt(v); break;                  /* test_rsqrt.py:20-24 */
+      case 3: r = sin(v); break;                         /* test_math_ops.py:33-38 */
+      case 4: r = cos(v); break;                         /* test_math_ops.py:25-30 */
+      default: r = exp(v); break;
+    }
+    store_el(y, i, dtype, r);
+  }
+}
+
+void oracle_binary(int op, const void *a, const void *b, void *y, int64_t n, int dtype) {
+#pragma omp parallel for
+  for (int64_t i = 0; i < n; ++i) {
+    const double u = load_el(a, i, dtype), v = load_el(b, i, dtype);
+    store_el(y, i, dtype, op == 0 ? u + v : op == 1 ? u - v : op == 2 ? u * v : u / v);
+  }
+}
+
+/* sum_kernel, test/python/triton/test_sum.py:30-36: out[pid] = sum of program pid's BLOCK_SIZE elements */
+void oracle_block_sum(const void *x, void *out, int64_t n, int64_t block, int dtype) {
+  const int64_t programs = (n + block - 1) / block;
+  for (int64_t p = 0; p < programs; ++p) {
+    const int64_t end = (p + 1) * block < n ? (p + 1) * block : n;
+    double s = 0.0;
+    for (int64_t i = p * block; i < end; ++i) s += load_el(x, i, dtype);
+    store_el(out, p, dtype, s);
+  }
+}
+
+/* rope_kernel, test/python/triton/test_rope.py:43-57 (angles), :174-184 (even / odd cases):
+ * x [batch, seq, heads, feat]; pair (2i, 2i+1) at position m turns by m / theta^(2i/feat). */
+void oracle_rope(const void *x, void *y, int64_t batch, int64_t seq, int64_t heads, int64_t feat, double theta,
+                 int dtype) {
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t m = 0; m < seq; ++m)
+      for (int64_t h = 0; h < heads; ++h)
+        for (int64_t i = 0; i < feat; i += 2) {
+          const int64_t off = ((b * seq + m) * heads + h) * feat + i;
+          const double ang = (double)m / pow(theta, (double)i / (double)feat);
+          const double e = load_el(x, off, dtype), o = load_el(x, off + 1, dtype);
+          store_el(y, off, dtype, e * cos(ang) - o * sin(ang));
+          store_el(y, off + 1, dtype, e * sin(ang) + o * cos(ang));
+        }
 }

@@ -185,6 +185,41 @@ def attention_online_f32(q, k, v, sm_scale, block_n):
     return o
 
 
+UNARY_OPS = {"gelu_tanh": 0, "silu": 1, "rsqrt": 2, "sin": 3, "cos": 4, "exp": 5}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def unary(op, x, dtype=None):
+    x = _c(x)
+    y = np.empty_like(x)
+    _l().oracle_unary(_int(UNARY_OPS[op]), _ptr(x), _ptr(y), _i64(x.size), _int(_code(x, dtype)))
+    return y
+
+
+def binary(op, a, b, dtype=None):
+    a, b = _c(a), _c(b)
+    assert a.shape == b.shape and a.dtype == b.dtype
+    y = np.empty_like(a)
+    _l().oracle_binary(_int(BINARY_OPS[op]), _ptr(a), _ptr(b), _ptr(y), _i64(a.size), _int(_code(a, dtype)))
+    return y
+
+
+def block_sum(x, block, dtype=None):
+    x = _c(x).reshape(-1)
+    out = np.empty(((x.size + block - 1) // block,), x.dtype)
+    _l().oracle_block_sum(_ptr(x), _ptr(out), _i64(x.size), _i64(block), _int(_code(x, dtype)))
+    return out
+
+
+def rope(x, theta, dtype=None):
+    """x: [batch, seq, heads, feat]."""
+    x = _c(x)
+    B, L, H, D = x.shape
+    y = np.empty_like(x)
+    _l().oracle_rope(_ptr(x), _ptr(y), _i64(B), _i64(L), _i64(H), _i64(D), _dbl(theta), _int(_code(x, dtype)))
+    return y
+
+
 def f32_to_f16_bits(v):
     return _l().oracle_f32_to_f16(ctypes.c_float(v))
 

@@ -315,3 +315,66 @@ def test_attention_online_recurrence(oracle, block_n):
     got = oracle.attention_online_f32(q, k, v, 0.5, block_n)
     want = oracle.attention(q, k, v, 0.5, False)
     assert np.allclose(got, want, rtol=2e-5, atol=1e-6)
+
+
+# ---- element-wise operators, block sums, rotary embedding ---------------------------------------------------
+def test_unary_ops_vs_torch(oracle):
+    g = torch.Generator().manual_seed(30)
+    x = torch.randn(16384, generator=g, dtype=torch.float64).float() * 3
+    xn = x.numpy()
+    # test_gelu.py:73-76 (atol 1e-5 in fp32: the kernel's rounded constants differ from torch's in the 7th digit)
+    assert np.allclose(oracle.unary("gelu_tanh", xn), F.gelu(x, approximate="tanh").numpy(), atol=1e-5)
+    assert np.allclose(oracle.unary("silu", xn), F.silu(x.double()).numpy(), rtol=1e-6, atol=1e-7)   # test_silu.py:69
+    pos = torch.rand(1024, generator=g) + 1e-3
+    assert np.allclose(oracle.unary("rsqrt", pos.numpy()), torch.rsqrt(pos.double()).numpy(), rtol=1e-6)
+    lin = torch.linspace(0, 3.14, 1024)                                          # test_math_ops.py:42
+    assert np.allclose(oracle.unary("sin", lin.numpy()), torch.sin(lin.double()).numpy(), atol=1e-7)
+    assert np.allclose(oracle.unary("cos", lin.numpy()), torch.cos(lin.double()).numpy(), atol=1e-7)
+    assert np.allclose(oracle.unary("exp", xn), torch.exp(x.double()).numpy(), rtol=1e-6)
+    # fp16 storage: computed in double, rounded once
+    h = x.half()
+    want = F.silu(h.double()).half()
+    assert np.array_equal(oracle.unary("silu", h.numpy()), want.numpy())
+    # closed forms: gelu(0) = 0, silu(0) = 0, gelu(x) -> x for large x and -> 0 for very negative x (no NaN)
+    edge = np.array([0.0, 30.0, -30.0, 1e4, -1e4], np.float32)
+    assert np.allclose(oracle.unary("gelu_tanh", edge), [0.0, 30.0, 0.0, 1e4, 0.0], atol=1e-6)
+
+
+def test_binary_ops_and_block_sum(oracle):
+    g = torch.Generator().manual_seed(31)
+    a, b = torch.rand(5000, generator=g), torch.rand(5000, generator=g) + 0.5
+    for name, fn in (("add", torch.add), ("sub", torch.sub), ("mul", torch.mul), ("div", torch.div)):
+        assert np.allclose(oracle.binary(name, a.numpy(), b.numpy()), fn(a.double(), b.double()).numpy(), rtol=1e-6)
+    x = torch.randn(1024 * 1024, generator=torch.Generator().manual_seed(42))    # test_sum.py:25-27
+    assert np.allclose(oracle.block_sum(x.numpy(), x.numel()), torch.sum(x.double()).numpy(), rtol=1e-6, atol=1e-4)
+    parts = oracle.block_sum(x.numpy(), 1000)                                    # ragged last program
+    assert parts.shape == (1049,)
+    assert np.allclose(parts, [c.double().sum().item() for c in torch.split(x, 1000)], rtol=1e-5, atol=1e-5)
+    assert np.array_equal(oracle.block_sum(np.arange(12, dtype=np.float32), 4), [6.0, 22.0, 38.0])
+
+
+def _rope_torch(x, theta):
+    """rope_reference_pytorch (test/python/triton/test_rope.py:60-95) in float64."""
+    B, L, H, D = x.shape
+    idx = torch.arange(D, dtype=torch.float64)
+    steps = torch.where(idx % 2 == 0, idx, idx - 1)
+    freqs = 1.0 / (theta ** (steps / D))
+    ang = torch.arange(L, dtype=torch.float64)[:, None] * freqs[None, :]
+    cos, sin = torch.cos(ang).reshape(1, L, 1, D), torch.sin(ang).reshape(1, L, 1, D)
+    xd = x.double()
+    fwd, bwd = torch.roll(xd, -1, 3), torch.roll(xd, 1, 3)
+    even = (torch.arange(D) % 2 == 0).view(1, 1, 1, D)
+    return torch.where(even, xd * cos - fwd * sin, bwd * sin + xd * cos)
+
+
+def test_rope_vs_reference_formula(oracle):
+    g = torch.Generator().manual_seed(32)
+    x = torch.rand(3, 8, 16, 32, generator=g)                                    # test_rope.py:20-23 shape
+    got = oracle.rope(x.numpy(), 10000.0)
+    assert np.allclose(got, _rope_torch(x, 10000.0).numpy(), rtol=1e-6, atol=1e-6)
+    assert np.array_equal(got[:, 0], x.numpy()[:, 0])                            # position 0: no rotation
+    pairs_in = x.numpy().reshape(3, 8, 16, 16, 2)
+    pairs_out = got.reshape(3, 8, 16, 16, 2)
+    assert np.allclose((pairs_out ** 2).sum(-1), (pairs_in ** 2).sum(-1), rtol=1e-5)   # rotations keep the norm
+    x2 = torch.randn(1, 300, 2, 64, generator=g)
+    assert np.allclose(oracle.rope(x2.numpy(), 500.0), _rope_torch(x2, 500.0).numpy(), rtol=1e-5, atol=1e-5)
