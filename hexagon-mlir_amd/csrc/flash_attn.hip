@@ -21,7 +21,7 @@ namespace {
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 
-constexpr int kBlockM = 128;   // query rows per workgroup
+constexpr int kWideMinS = 8192;  // sequences at least this long use 8-wave (256-row) workgroups
 constexpr int kBlockN = 64;    // keys per step
 constexpr float kRescaleLag = 8.0f;   // how far (log2) the softmax reference maximum may trail the true one
 
@@ -55,10 +55,10 @@ template <int D> __device__ __forceinline__ int swz_vtile(int row) {
 // global -> LDS copy of one [64 keys][D] tile: 64*D/8/64/4 wave-wide instructions per wave. The per-lane element
 // offsets inside a tile do not change from tile to tile, so they are computed once; only a ragged last tile
 // (keys past the end of the sequence) needs its rows clamped.
-template <typename T, int D, bool IS_V>
+template <typename T, int D, bool IS_V, int NW = 4>
 struct KvTileLoader {
   static constexpr int CPR = D / 8;                       // chunks per row
-  static constexpr int NI = kBlockN * CPR / 64 / 4;       // instructions per wave
+  static constexpr int NI = kBlockN * CPR / 64 / NW;      // instructions per wave
   int off[NI];                                            // element offset of this lane's chunk inside a tile
   int row[NI];
   int col[NI];
@@ -66,7 +66,7 @@ struct KvTileLoader {
   __device__ __forceinline__ void init(int wave, int lane) {
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
-      const int inst = j * 4 + wave;
+      const int inst = j * NW + wave;
       const int lin = inst * 64 + lane;
       row[j] = lin / CPR;
       col[j] = ((lin % CPR) ^ (IS_V ? swz_vtile<D>(row[j]) : swz_ktile<D>(row[j]))) * 8;
@@ -116,8 +116,13 @@ template <> __device__ __forceinline__ void store4o<bf16>(bf16* p, float a, floa
 // GENERAL: the number of keys (Skv) may differ from the number of queries (S) and an additive mask
 // [ZH, S, Skv] (same dtype as Q; may be null) is added to the scaled scores before the softmax, as
 // tm_tensor.attention does (qcom_hexagon_backend/lib/Transforms/LowerTmTensor.cpp:157-160); Skv % 4 == 0.
-template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false>
-__global__ __launch_bounds__(256, 2)
+// NW waves per workgroup (4 or 8), 32 query rows each: every K / V tile copied into LDS serves NW*32 query rows.
+// Eight waves halve the L2 -> LDS copy traffic (each query block streams the whole K and V of its head), worth
+// about 4 % at 16k keys; shorter sequences prefer the larger number of 128-row workgroups. (Measured on random
+// data the kernel is held back by the power limit more than by any stall: all-zero inputs run 30 % faster through
+// the same instructions and the same memory traffic, as the dense GEMM also shows.)
+template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, int NW = 4>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1)
 void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                       OutT* __restrict__ O, int ZH, int S, float scale_log2e, const T* __restrict__ Mk = nullptr,
                       int Skv_arg = 0, float mask_factor = 0.0f) {
@@ -132,6 +137,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   __shared__ __attribute__((aligned(16))) T v_lds0[kBlockN * D];
   __shared__ __attribute__((aligned(16))) T v_lds1[kBlockN * D];
 
+  constexpr int kBlockM = NW * 32;                  // query rows per workgroup
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int nqb = (S + kBlockM - 1) / kBlockM;
   // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each). Give every XCD whole heads and let it walk
@@ -175,11 +181,11 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   const int key_end = CAUSAL ? ((qb + 1) * kBlockM < S ? (qb + 1) * kBlockM : S) : Skv;
   const int n_steps = (key_end + kBlockN - 1) / kBlockN;
 
-  KvTileLoader<T, D, false> k_loader;
-  KvTileLoader<T, D, true> v_loader;
+  KvTileLoader<T, D, false, NW> k_loader;
+  KvTileLoader<T, D, true, NW> v_loader;
   k_loader.init(wave, lane);
   v_loader.init(wave, lane);
-  auto load_kv = [&](int step, T* k_dst, T* v_dst) {
+  auto load_kv = [&](int step, T* k_dst, T* v_dst) __attribute__((always_inline)) {
     k_loader.issue(k_g, step * kBlockN, Skv, k_dst);
     v_loader.issue(v_g, step * kBlockN, Skv, v_dst);
   };
@@ -190,7 +196,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   // shift invariant, so exponentials up to 2^kRescaleLag are as exact as ones below 1, and the output
   // accumulator and running sum only need rescaling when a row outgrows the lag. The decision is per row (lane);
   // the wave-uniform ballot only skips the multiplications when no row of the wave needs them.
-  auto softmax_tile = [&](int key_base, bool need_mask, f32x16& s, Frag* pf) {
+  auto softmax_tile = [&](int key_base, bool need_mask, f32x16& s, Frag* pf) __attribute__((always_inline)) {
     if (need_mask) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -227,7 +233,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   };
   // O^T += V^T P^T for one 32-key tile. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
   // which is score register hf*8 + e of this lane, so the packed probabilities are used as they are.
-  auto pv_tile = [&](const T* v_src, int jt, const Frag* pf) {
+  auto pv_tile = [&](const T* v_src, int jt, const Frag* pf) __attribute__((always_inline)) {
     const int g = lane / 16, i16 = lane % 16;
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
@@ -253,7 +259,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     if (Mk) mask_row = Mk + ((int64_t)zh * S + (qrow < S ? qrow : S - 1)) * Skv;
   }
 
-  auto process = [&](int step, const T* k_src, const T* v_src) {
+  auto process = [&](int step, const T* k_src, const T* v_src) __attribute__((always_inline)) {
     const int n0 = step * kBlockN;
     // mask values of this lane's 32 scores: four runs of four consecutive keys per 32-key tile
     typedef T MaskRun __attribute__((ext_vector_type(4)));
@@ -391,27 +397,34 @@ void flash_fwd_rowwise(const T* __restrict__ Q, const T* __restrict__ K, const T
   }
 }
 
+template <typename T, typename OutT, int D, bool CAUSAL, int NW>
+int launch_mfma_nw(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
+                   hipStream_t st) {
+  const int64_t nqb = (S + NW * 32 - 1) / (NW * 32);
+  const int64_t blocks = nqb * ZH;
+  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, CAUSAL, false, NW>), dim3((unsigned)blocks), dim3(NW * 64), 0, st,
+                     static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                     static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e);
+  return launch_status();
+}
+
 template <typename T, typename OutT, int D>
 int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
                 bool causal, hipStream_t st) {
-  const int64_t nqb = (S + kBlockM - 1) / kBlockM;
-  const int64_t blocks = nqb * ZH;
-  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
-  if (causal)
-    hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, true>), dim3((unsigned)blocks), dim3(256), 0, st,
-                       static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
-                       static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e);
-  else
-    hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, false>), dim3((unsigned)blocks), dim3(256), 0, st,
-                       static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
-                       static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e);
-  return launch_status();
+  const bool wide = S >= kWideMinS;
+  if (causal) {
+    if (wide) return launch_mfma_nw<T, OutT, D, true, 8>(Q, K, V, O, ZH, S, scale_log2e, st);
+    return launch_mfma_nw<T, OutT, D, true, 4>(Q, K, V, O, ZH, S, scale_log2e, st);
+  }
+  if (wide) return launch_mfma_nw<T, OutT, D, false, 8>(Q, K, V, O, ZH, S, scale_log2e, st);
+  return launch_mfma_nw<T, OutT, D, false, 4>(Q, K, V, O, ZH, S, scale_log2e, st);
 }
 
 template <typename T, typename OutT, int D>
 int launch_mfma_general(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
                         int64_t Skv, float scale_log2e, hipStream_t st) {
-  const int64_t nqb = (S + kBlockM - 1) / kBlockM;
+  const int64_t nqb = (S + 127) / 128;
   const int64_t blocks = nqb * ZH;
   if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
   const float mask_factor = 1.44269504088896340736f / scale_log2e;     // mask / sm_scale

@@ -220,3 +220,19 @@ def test_masked_attention_fully_masked_row_is_nan(hexmi):
     mask[0, 5, :] = float("-inf")
     got = hexmi.attention(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).cpu()
     assert torch.isnan(got[0, 5]).all() and not torch.isnan(got[0, :5]).any() and not torch.isnan(got[0, 6:]).any()
+
+
+@pytest.mark.parametrize("case", [(1, 1, 8200, 64, True), (1, 1, 8192, 128, False), (1, 2, 8192 + 130, 128, True)])
+def test_attention_long_sequences(hexmi, oracle, case):
+    # sequences of 8192 keys and more run 8-wave workgroups (256 query rows per K/V tile copy)
+    Z, H, S, D, causal = case
+    q, k, v = _qkv(Z, H, S, D, torch.float16, seed=7)
+    scale = 1.0 / math.sqrt(D)
+    got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal).cpu()
+    want = _oracle(oracle, q, k, v, scale, causal)
+    assert (got.float() - want).abs().max() <= 2e-2
+    # rows of different 256-row blocks do not interact: the first 300 rows of a causal run equal a 300-row run
+    if causal:
+        short = hexmi.flash_attention(q[:, :, :300].contiguous().cuda(), k[:, :, :300].contiguous().cuda(),
+                                      v[:, :, :300].contiguous().cuda(), scale, True).cpu()
+        assert (short.float() - got[:, :, :300].float()).abs().max() <= 2e-3
