@@ -347,7 +347,7 @@ def _time_cpu(fn, iters):
 def make_workloads():
     return {w.name: w for w in (
         Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
-        W8A16(1), W8A16(16), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
+        W8A16(1), W8A16(16), W8A16(64), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
         Elementwise("sum"),
         CopyCalibration())}
 

@@ -140,7 +140,15 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
   const int n_end = n_begin + chan_per_wg < N ? n_begin + chan_per_wg : N;
 
   for (int base = n_begin; base < n_end; base += kPTiles * 16) {
-    // weights first: all tiles of this pass, every step
+    // The scale of the output this thread will finish, requested before the weights: it comes from HBM and would
+    // otherwise be waited for after everything else. (The empty asm below is a use on every path.)
+    f16 sc;
+    {
+      const int q = (threadIdx.x / 256) % kPTiles, e = threadIdx.x % 256;
+      const int gn = base + q * 16 + (e / 64) * 4 + e % 4;
+      sc = scales[gn < n_end ? gn : n_end - 1];
+    }
+    // weights: all tiles of this pass, every step
     u32x4 wv[kPTiles][kPSteps];
 #pragma unroll
     for (int q = 0; q < kPTiles; ++q) {
@@ -183,6 +191,7 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
       }
       *reinterpret_cast<f32x4*>(red + ((q * kPWaves + wave) * 64 + lane) * 4) = acc;
     }
+    asm volatile("" : "+v"(sc));
     __syncthreads();
     if (threadIdx.x < kPTiles * 256) {
       const int q = threadIdx.x / 256, e = threadIdx.x % 256;     // e = lane*4 + element of the accumulator
@@ -192,11 +201,205 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
       const int l = e / 4;
       const int gm = l % 16;
       const int gn = base + q * 16 + (l / 16) * 4 + e % 4;
-      if (gm < M && gn < n_end) C[(int64_t)gm * N + gn] = (f16)(sum * (float)scales[gn]);
+      if (gm < M && gn < n_end) C[(int64_t)gm * N + gn] = (f16)(sum * (float)sc);
     }
     __syncthreads();
   }
 }
+
+// 16 < M <= 64 (MB = 2..4 blocks of 16 activation rows), K % 256 == 0: one persistent workgroup of 16 waves per
+// CU, each owning an equal contiguous range of at most 48 output channels, so the weights cross HBM once, in
+// contiguous 256-byte row segments. K is walked in chunks of 256. The raw int8 weight chunk [48][256] and the
+// activation chunk [MB*16][256] fp16 are copied global -> LDS (global_load_lds, no registers) by different
+// waves: waves 12..15 copy weights, four chunks ahead (five stages; this is the HBM stream, it needs the depth),
+// waves 0..3*MB-1 copy activations, two chunks ahead (three stages; L2 hits). A wave's outstanding-copy counter
+// only sees its own copies, so each role waits with its own count and the workgroup barrier publishes both.
+// Wave w < 3*MB also owns the 16 x 16 output tile (row block w/3, channel tile w%3) for the whole K loop, so
+// there is no cross-wave reduction: it reads its fragments back from LDS (16-byte chunks XOR-swizzled by row
+// through the copy's source addresses, conflict-free), converts the int8 bytes in registers and keeps one
+// accumulator. Every copying wave issues exactly three copies per chunk (repeats of real ones fill the slots and
+// rewrite the same bytes).
+constexpr int kMidKC = 256;                                 // K per chunk
+constexpr int kMidCh = 48;                                  // channels per workgroup (three tiles of 16)
+constexpr int kMidSlots = 3;                                // copies per copying wave per chunk
+constexpr int kMidAStages = 3, kMidWStages = 5;
+constexpr int kMidWWave0 = 12;                              // first of the four weight-copy waves
+
+#define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+
+template <int MB>
+__global__ __launch_bounds__(1024)
+void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
+                      f16* __restrict__ C, int M, int N, int K, int chan_per_wg) {
+  __shared__ __attribute__((aligned(16))) f16 a_s0[MB * 16 * kMidKC];
+  __shared__ __attribute__((aligned(16))) f16 a_s1[MB * 16 * kMidKC];
+  __shared__ __attribute__((aligned(16))) f16 a_s2[MB * 16 * kMidKC];
+  __shared__ __attribute__((aligned(16))) int8_t w_s0[kMidCh * kMidKC];
+  __shared__ __attribute__((aligned(16))) int8_t w_s1[kMidCh * kMidKC];
+  __shared__ __attribute__((aligned(16))) int8_t w_s2[kMidCh * kMidKC];
+  __shared__ __attribute__((aligned(16))) int8_t w_s3[kMidCh * kMidKC];
+  __shared__ __attribute__((aligned(16))) int8_t w_s4[kMidCh * kMidKC];
+
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int r16 = lane % 16, kg = lane / 16;
+  const int n_begin = blockIdx.x * chan_per_wg;
+  const int n_end = n_begin + chan_per_wg < N ? n_begin + chan_per_wg : N;
+  const int n_chunks = K / kMidKC;
+  const bool computes = wave < 3 * MB;                      // also copies activations
+  const bool copies_w = wave >= kMidWWave0;
+
+  // ---- copy slots. Activation copy i (0 .. 8*MB-1) moves rows 2i, 2i+1 (512 bytes each); weight copy t (0 .. 11)
+  //      moves rows 4t .. 4t+3 (256 bytes each). Lane positions are permuted inside a row (see the fragment side).
+  const char* slot_src[kMidSlots];                          // source of this lane for chunk 0
+  int slot_dst[kMidSlots];                                  // byte offset of the copy inside its stage
+#pragma unroll
+  for (int j = 0; j < kMidSlots; ++j) {
+    slot_src[j] = nullptr;
+    slot_dst[j] = 0;
+    if (computes) {
+      const int i = (j * 3 * MB + wave) % (8 * MB);
+      const int row = 2 * i + lane / 32;
+      const int c = lane % 32;                              // 16-byte position inside the row's 512 bytes
+      const int src_c = (c & 16) | ((c ^ row) & 15);        // the chunk that belongs at this position
+      slot_src[j] = reinterpret_cast<const char*>(A + (int64_t)(row < M ? row : M - 1) * K) + src_c * 16;
+      slot_dst[j] = i * 1024;
+    } else if (copies_w) {
+      const int t = j * 4 + (wave - kMidWWave0);
+      const int row = 4 * t + lane / 16;
+      const int c = lane % 16;
+      const int src_c = (c ^ row) & 15;
+      const int n = n_begin + row < n_end ? n_begin + row : n_end - 1;
+      slot_src[j] = reinterpret_cast<const char*>(W + (int64_t)n * K) + src_c * 16;
+      slot_dst[j] = t * 1024;
+    }
+  }
+  auto a_stage = [&](int i) __attribute__((always_inline)) { return i == 0 ? a_s0 : (i == 1 ? a_s1 : a_s2); };
+  auto w_stage = [&](int i) __attribute__((always_inline)) {
+    return i == 0 ? w_s0 : (i == 1 ? w_s1 : (i == 2 ? w_s2 : (i == 3 ? w_s3 : w_s4)));
+  };
+  // chunk indices past the end repeat the last chunk (copied, never read): every chunk issues the same copies
+  auto issue_a = [&](int chunk, f16* dst) __attribute__((always_inline)) {
+    const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
+#pragma unroll
+    for (int j = 0; j < kMidSlots; ++j)
+      __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * kMidKC * 2),
+                                       HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, 0);
+  };
+  auto issue_w = [&](int chunk, int8_t* dst) __attribute__((always_inline)) {
+    const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
+#pragma unroll
+    for (int j = 0; j < kMidSlots; ++j)
+      __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * kMidKC),
+                                       HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, 0);
+  };
+
+  // ---- fragment side: wave < 3*MB owns row block mb, channel tile nt
+  const int mb = wave / 3, nt = wave % 3;
+  int w_off[4], a_off[4][2];
+  {
+    const int wrow = nt * 16 + r16, arow = mb * 16 + r16;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      w_off[ks] = wrow * kMidKC + (((ks * 4 + kg) ^ wrow) & 15) * 16;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int c = ks * 8 + kg * 2 + h;
+        a_off[ks][h] = arow * kMidKC * 2 + ((c & 16) | ((c ^ arow) & 15)) * 16;
+      }
+    }
+  }
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  // The fragment reads are written as inline assembly: the compiler cannot tell which stage an in-flight
+  // global_load_lds writes and would make every LDS read wait for all of them (vmcnt(0)), which undoes the
+  // pipelining. The waits this kernel needs are the explicit ones around the barrier.
+  // One statement holds the reads and the wait for them, so no register of the result can be touched early.
+  auto multiply = [&](const f16* a_src, const int8_t* w_src) __attribute__((always_inline)) {
+    const unsigned a_base = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(a_src);
+    const unsigned w_base = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(w_src);
+    u32x4 raw[4], a0[4], a1[4];
+    asm volatile(
+        "ds_read_b128 %0, %12\n\tds_read_b128 %1, %13\n\tds_read_b128 %2, %14\n\tds_read_b128 %3, %15\n\t"
+        "ds_read_b128 %4, %16\n\tds_read_b128 %5, %17\n\tds_read_b128 %6, %18\n\tds_read_b128 %7, %19\n\t"
+        "ds_read_b128 %8, %20\n\tds_read_b128 %9, %21\n\tds_read_b128 %10, %22\n\tds_read_b128 %11, %23\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(raw[0]), "=&v"(raw[1]), "=&v"(raw[2]), "=&v"(raw[3]), "=&v"(a0[0]), "=&v"(a0[1]), "=&v"(a0[2]),
+          "=&v"(a0[3]), "=&v"(a1[0]), "=&v"(a1[1]), "=&v"(a1[2]), "=&v"(a1[3])
+        : "v"(w_base + w_off[0]), "v"(w_base + w_off[1]), "v"(w_base + w_off[2]), "v"(w_base + w_off[3]),
+          "v"(a_base + a_off[0][0]), "v"(a_base + a_off[1][0]), "v"(a_base + a_off[2][0]), "v"(a_base + a_off[3][0]),
+          "v"(a_base + a_off[0][1]), "v"(a_base + a_off[1][1]), "v"(a_base + a_off[2][1]), "v"(a_base + a_off[3][1])
+        : "memory");
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      f16x8 w0, w1;
+      cvt16(raw[ks], w0, w1);
+      // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, __builtin_bit_cast(f16x8, a0[ks]), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, __builtin_bit_cast(f16x8, a1[ks]), acc, 0, 0, 0);
+    }
+  };
+  // s_waitcnt immediates (gfx9 encoding), LDS counter untouched: copies of the newer chunks may stay in flight
+  constexpr int kNewerA = (kMidAStages - 2) * kMidSlots, kNewerW = (kMidWStages - 2) * kMidSlots;
+  constexpr int kWaitA = (kNewerA & 0xF) | ((kNewerA >> 4) << 14) | (0x7 << 4) | (0xF << 8);
+  constexpr int kWaitW = (kNewerW & 0xF) | ((kNewerW >> 4) << 14) | (0x7 << 4) | (0xF << 8);
+
+  // Channel scales of this lane's four outputs, requested before anything else: they come from HBM and would
+  // otherwise be waited for at the very end. The empty asm statements are uses on every path, which keeps the
+  // loads here instead of next to the stores.
+  f16 sc[4] = {(f16)0, (f16)0, (f16)0, (f16)0};
+  if (computes) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int gn = n_begin + nt * 16 + kg * 4 + e;
+      sc[e] = scales[gn < n_end ? gn : n_end - 1];
+    }
+  }
+  // prologue: activations of chunks 0, 1; weights of chunks 0 .. 3
+  if (computes) {
+    issue_a(0, a_s0);
+    issue_a(1, a_s1);
+  } else if (copies_w) {
+    issue_w(0, w_s0);
+    issue_w(1, w_s1);
+    issue_w(2, w_s2);
+    issue_w(3, w_s3);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) asm volatile("" : "+v"(sc[e]));
+  constexpr int kPeriod = kMidAStages * kMidWStages;        // stage assignment repeats every 15 chunks
+  for (int base = 0; base < n_chunks; base += kPeriod) {
+#pragma unroll
+    for (int u = 0; u < kPeriod; ++u) {
+      if (base + u < n_chunks) {
+        const int chunk = base + u;
+        if (computes) __builtin_amdgcn_s_waitcnt(kWaitA);
+        else if (copies_w) __builtin_amdgcn_s_waitcnt(kWaitW);
+        // chunk landed for every wave; the stages of chunk-1 are free. A bare s_barrier: __syncthreads() would add
+        // a wait for every outstanding copy and undo the pipelining.
+        __builtin_amdgcn_s_barrier();
+        if (computes) {
+          issue_a(chunk + 2, a_stage((u + 2) % kMidAStages));
+          multiply(a_stage(u % kMidAStages), w_stage(u % kMidWStages));
+        } else if (copies_w) {
+          issue_w(chunk + 4, w_stage((u + 4) % kMidWStages));
+        }
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // trailing copies land before the LDS is released
+
+  if (computes) {
+    const int gm = mb * 16 + r16;
+    const int gn = n_begin + nt * 16 + kg * 4;
+    if (gm < M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (gn + e < n_end) C[(int64_t)gm * N + gn + e] = (f16)(acc[e] * (float)sc[e]);
+    }
+  }
+}
+#undef HEXMI_LDS
+#undef HEXMI_GLB
 
 // One or two activation rows (decode): no matrix cores. A wave owns RPW consecutive output channels and reads
 // each 4 KiB-aligned weight row with fully contiguous 16-byte loads (lane i takes bytes [1024*j + 16*i, +16) of
@@ -312,6 +515,19 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     const int grid = (int)((N + chan_per_wg - 1) / chan_per_wg);
     hipLaunchKernelGGL(w8a16_persist_kernel, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K,
                        chan_per_wg);
+    return launch_status();
+  }
+  if (M <= 64 && K % kMidKC == 0 && N <= 0x7fffffff) {
+    const int cus = hexmi_num_cus();
+    if (cus <= 0) return HEXMI_ELAUNCH;
+    int chan_per_wg = (int)((N + cus - 1) / cus);
+    if (chan_per_wg < 16) chan_per_wg = 16;
+    if (chan_per_wg > kMidCh) chan_per_wg = kMidCh;         // more workgroups than CUs beyond 48 channels per CU
+    const int grid = (int)((N + chan_per_wg - 1) / chan_per_wg);
+#define HEXMI_MID(MB) \
+  hipLaunchKernelGGL(w8a16_mid_kernel<MB>, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg)
+    if (M <= 16) HEXMI_MID(1); else if (M <= 32) HEXMI_MID(2); else if (M <= 48) HEXMI_MID(3); else HEXMI_MID(4);
+#undef HEXMI_MID
     return launch_status();
   }
   if (M > 64 && K % 32 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8))

@@ -78,7 +78,7 @@ def test_w8a16_parity(hexmi, oracle, M, N, K):
     assert (got.float() - want.float()).abs().max() / math.sqrt(K) <= 2e-2
 
 
-@pytest.mark.parametrize("M", [1, 16, 256])
+@pytest.mark.parametrize("M", [1, 16, 32, 64, 256])
 def test_w8a16_config_sizes(hexmi, oracle, M):
     # measured configuration: N=11008, K=4096; the oracle covers every 43rd output channel, all M rows
     from hexmi.workloads import w8a16_inputs
