@@ -203,6 +203,25 @@ class W8A16(Workload):
                 "full size, dequantise + fp32 matmul on CPU")
 
 
+class W8A16Packed(W8A16):
+    """The same product on weights pre-packed once into fragment-major order (not part of the timed step)."""
+
+    def __init__(self, M):
+        super().__init__(M)
+        self.name = "w8a16_packed_m%d" % M
+        self.desc += ", weights pre-packed by hexmi_pack_w8"
+
+    def setup(self, torch, hexmi):
+        super().setup(torch, hexmi)
+        for s in self.sets:
+            s["wp"] = hexmi.pack_w8(s["w"])
+            del s["w"]
+
+    def step(self, i):
+        s = self.sets[i % len(self.sets)]
+        self.hexmi.w8a16_matmul_packed(s["a"], s["wp"], s["scales"], out=s["out"])
+
+
 class Attention(Workload):
     bound, dtype, kernel = "mfma", "f16", "flash_fwd_kernel"
 
@@ -347,7 +366,7 @@ def _time_cpu(fn, iters):
 def make_workloads():
     return {w.name: w for w in (
         Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
-        W8A16(1), W8A16(16), W8A16(64), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
+        W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
         Elementwise("sum"),
         CopyCalibration())}
 

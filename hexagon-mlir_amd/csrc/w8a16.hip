@@ -127,6 +127,9 @@ void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const
 constexpr int kPWaves = 16;
 constexpr int kPTiles = 3;                                  // tiles per workgroup per pass
 constexpr int kPSteps = 4;                                  // 64-wide steps per wave: K <= 16 * 4 * 64
+// PACKED: W is the fragment-major layout written by pack_w8_kernel (chan_per_wg is then a multiple of 16): the
+// 16 rows x 64 k of a tile step are one contiguous KiB in lane order, so a wave's loads are fully contiguous.
+template <bool PACKED>
 __global__ __launch_bounds__(1024)
 void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
                           f16* __restrict__ C, int M, int N, int K, int chan_per_wg) {
@@ -152,13 +155,25 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
     u32x4 wv[kPTiles][kPSteps];
 #pragma unroll
     for (int q = 0; q < kPTiles; ++q) {
-      int n = base + q * 16 + r16;
-      n = n < n_end ? n : n_end - 1;                        // past the range: re-read its last row, unused
-      const int8_t* wrow = W + (int64_t)n * K + (int64_t)wave * ksl + kg * 16;
+      if constexpr (PACKED) {
+        int tile = base / 16 + q;
+        const int last = (N + 15) / 16 - 1;
+        tile = tile <= last ? tile : last;                  // past the end: re-read the last tile, unused
+        const int8_t* blk = W + ((int64_t)tile * (K / 64) + (int64_t)wave * steps) * 1024 + lane * 16;
 #pragma unroll
-      for (int u = 0; u < kPSteps; ++u) {
-        const int st = u < steps ? u : steps - 1;
-        wv[q][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + st * 64));
+        for (int u = 0; u < kPSteps; ++u) {
+          const int st = u < steps ? u : steps - 1;
+          wv[q][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(blk + st * 1024));
+        }
+      } else {
+        int n = base + q * 16 + r16;
+        n = n < n_end ? n : n_end - 1;                      // past the range: re-read its last row, unused
+        const int8_t* wrow = W + (int64_t)n * K + (int64_t)wave * ksl + kg * 16;
+#pragma unroll
+        for (int u = 0; u < kPSteps; ++u) {
+          const int st = u < steps ? u : steps - 1;
+          wv[q][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + st * 64));
+        }
       }
     }
     // this wave's activation slice: rows r16, k in [wave*ksl + u*64 + kg*16, +16)
@@ -462,6 +477,25 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
   }
 }
 
+// One-time re-layout of int8 weights [N, K] into fragment-major order for the small-M kernels (the analogue of
+// the reference's constant-weight block linearisation, qcom_hexagon_backend/lib/Transforms/
+// PreprocessWeightsForHMXPass.cpp:39-117): tiles of 16 channels x 64 k, tile (t, s) at byte
+// ((t * K/64) + s) * 1024, inside it lane l = g*16 + r holds the 16 bytes W[16t + r][64s + 16g .. +16).
+// Channels past N (the last tile) are zero. One thread per 16-byte chunk of the output.
+__global__ __launch_bounds__(256)
+void pack_w8_kernel(const int8_t* __restrict__ W, int8_t* __restrict__ Wp, int64_t N, int64_t K, int64_t chunks) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= chunks) return;
+  const int lane = (int)(o % 64);
+  const int64_t blk = o / 64;                                // t * K/64 + s
+  const int64_t t = blk / (K / 64), sidx = blk % (K / 64);
+  const int64_t row = t * 16 + lane % 16;
+  const int64_t k = sidx * 64 + (lane / 16) * 16;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (row < N) v = *reinterpret_cast<const u32x4*>(W + row * K + k);
+  *reinterpret_cast<u32x4*>(Wp + o * 16) = v;
+}
+
 __global__ __launch_bounds__(256)
 void dequant_kernel(const int8_t* __restrict__ W, const f16* __restrict__ scales, float* __restrict__ out,
                     int64_t N, int64_t K) {
@@ -513,7 +547,7 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     int chan_per_wg = (int)((N + cus - 1) / cus);
     if (chan_per_wg < 16) chan_per_wg = 16;                 // one full tile at least
     const int grid = (int)((N + chan_per_wg - 1) / chan_per_wg);
-    hipLaunchKernelGGL(w8a16_persist_kernel, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K,
+    hipLaunchKernelGGL(w8a16_persist_kernel<false>, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K,
                        chan_per_wg);
     return launch_status();
   }
@@ -538,6 +572,46 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     if (left > 32) rc = launch_pass<4>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
     else if (left > 16) rc = launch_pass<2>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
     else rc = launch_pass<1>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
+  }
+  return rc;
+}
+
+extern "C" int hexmi_pack_w8(int64_t N, int64_t K, const int8_t* W, int8_t* Wp, hexmi_stream_t stream) {
+  if (N < 0 || K < 0) return HEXMI_EINVAL;
+  if (N == 0 || K == 0) return HEXMI_OK;
+  if (!W || !Wp) return HEXMI_EINVAL;
+  if (K % 64 != 0) return HEXMI_ENOTSUP;
+  if (!aligned_to(W, 16) || !aligned_to(Wp, 16)) return HEXMI_EINVAL;
+  const int64_t chunks = ((N + 15) / 16) * 16 * (K / 16);   // 16-byte chunks of the packed buffer
+  const int64_t blocks = (chunks + 255) / 256;
+  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  hipLaunchKernelGGL(pack_w8_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), W, Wp, N, K, chunks);
+  return launch_status();
+}
+
+extern "C" int hexmi_gemm_w8a16_packed(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* Wp,
+                                       const void* scales, void* C, hexmi_stream_t stream) {
+  if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
+  if (M == 0 || N == 0) return HEXMI_OK;
+  if (!A || !Wp || !scales || !C) return HEXMI_EINVAL;
+  // the K slices of the 16 waves are whole 64-wide steps, at most four each
+  if (K == 0 || K % (kPWaves * 64) != 0 || K / (kPWaves * 64) > kPSteps) return HEXMI_ENOTSUP;
+  if (!aligned_to(A, 16) || !aligned_to(Wp, 16)) return HEXMI_EINVAL;
+  if (M > 0x7fffffff || N > 0x7fffffff - 16) return HEXMI_ENOTSUP;
+  const int cus = hexmi_num_cus();
+  if (cus <= 0) return HEXMI_ELAUNCH;
+  hipStream_t st = as_stream(stream);
+  const int64_t tiles = (N + 15) / 16;
+  const int tiles_per_wg = (int)((tiles + cus - 1) / cus);
+  const int chan_per_wg = tiles_per_wg * 16;
+  const int grid = (int)((tiles + tiles_per_wg - 1) / tiles_per_wg);
+  // sixteen activation rows per launch: more rows walk the packed weights again (they then come from the caches)
+  int rc = HEXMI_OK;
+  for (int64_t m = 0; m < M && rc == HEXMI_OK; m += 16) {
+    const int rows = (int)(M - m < 16 ? M - m : 16);
+    hipLaunchKernelGGL(w8a16_persist_kernel<true>, dim3(grid), dim3(1024), 0, st, static_cast<const f16*>(A) + m * K, Wp,
+                       static_cast<const f16*>(scales), static_cast<f16*>(C) + m * N, rows, (int)N, (int)K, chan_per_wg);
+    rc = launch_status();
   }
   return rc;
 }

@@ -34,6 +34,8 @@ SIGNATURES = {
     "hexmi_matmul_f16f16_f32": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_gemm": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _int, _int, _ptr]),
     "hexmi_gemm_w8a16": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "hexmi_pack_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr]),
+    "hexmi_gemm_w8a16_packed": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_dequant_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_flash_attn_fwd": (_int, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _ptr]),
     "hexmi_unary": (_int, [_int, _ptr, _ptr, _i64, _int, _ptr]),

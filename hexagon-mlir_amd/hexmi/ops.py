@@ -46,6 +46,8 @@ _LIBDEF.define("layer_norm(Tensor x, Tensor? weight, Tensor? bias, float eps, Te
 _LIBDEF.define("matmul(Tensor a, Tensor b, bool trans_b, Tensor(a!) out) -> ()")
 _LIBDEF.define("w8a16_matmul(Tensor a, Tensor w, Tensor scales, Tensor(a!) out) -> ()")
 _LIBDEF.define("dequant_w8(Tensor w, Tensor scales, Tensor(a!) out) -> ()")
+_LIBDEF.define("pack_w8(Tensor w, Tensor(a!) out) -> ()")
+_LIBDEF.define("w8a16_matmul_packed(Tensor a, Tensor wp, Tensor scales, Tensor(a!) out) -> ()")
 _LIBDEF.define("flash_attention(Tensor q, Tensor k, Tensor v, float sm_scale, bool causal, Tensor(a!) out) -> ()")
 _LIBDEF.define("unary(int op, Tensor x, Tensor(a!) out) -> ()")
 _LIBDEF.define("binary(int op, Tensor a, Tensor b, Tensor(a!) out) -> ()")
@@ -89,6 +91,20 @@ def _w8a16_impl(a, w, scales, out):
     with torch.cuda.device(a.device):
         _lib.check(_lib.lib().hexmi_gemm_w8a16(M, N, K, _p(a), _p(w), _p(scales), _p(out), _stream()),
                    "hexmi_gemm_w8a16")
+
+
+def _pack_impl(w, out):
+    N, K = w.shape
+    with torch.cuda.device(w.device):
+        _lib.check(_lib.lib().hexmi_pack_w8(N, K, _p(w), _p(out), _stream()), "hexmi_pack_w8")
+
+
+def _w8a16_packed_impl(a, wp, scales, out):
+    M, K = a.shape
+    N = scales.shape[0]
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().hexmi_gemm_w8a16_packed(M, N, K, _p(a), _p(wp), _p(scales), _p(out), _stream()),
+                   "hexmi_gemm_w8a16_packed")
 
 
 def _dequant_impl(w, scales, out):
@@ -135,7 +151,8 @@ def _rope_impl(x, theta, out):
 
 
 for _name, _fn in (("softmax", _softmax_impl), ("rms_norm", _rms_norm_impl), ("layer_norm", _layer_norm_impl),
-                   ("matmul", _matmul_impl), ("w8a16_matmul", _w8a16_impl), ("dequant_w8", _dequant_impl),
+                   ("matmul", _matmul_impl), ("w8a16_matmul", _w8a16_impl), ("dequant_w8", _dequant_impl), ("pack_w8", _pack_impl),
+                   ("w8a16_matmul_packed", _w8a16_packed_impl),
                    ("flash_attention", _flash_impl), ("attention", _attention_impl),
                    ("unary", _unary_impl), ("binary", _binary_impl), ("block_sum", _block_sum_impl),
                    ("rope", _rope_impl)):
@@ -266,6 +283,39 @@ def w8a16_matmul(a, w_int8, scales, out=None):
     ad, wd, sd = _stage(a, dev), _stage(w_int8, dev), _stage(scales, dev)
     od = _out_like(out, (a.shape[0], w_int8.shape[0]), torch.float16, dev)
     torch.ops.hexmi.w8a16_matmul(ad, wd, sd, od)
+    return _finish(od, out)
+
+
+def pack_w8(w_int8):
+    """One-time re-layout of int8 weights [N,K] (K % 64 == 0) into the fragment-major order `w8a16_matmul_packed`
+    reads (flat int8 tensor of ceil(N/16)*16*K bytes); the analogue of the reference's constant-weight
+    pre-processing (qcom_hexagon_backend/lib/Transforms/PreprocessWeightsForHMXPass.cpp:39-117)."""
+    if w_int8.dtype != torch.int8 or w_int8.dim() != 2:
+        raise TypeError("hexmi.pack_w8: expected an int8 [N,K] tensor")
+    N, K = w_int8.shape
+    if K % 64 != 0:
+        raise ValueError("hexmi.pack_w8: K must be a multiple of 64")
+    dev = _device() if w_int8.device.type != "cuda" else w_int8.device
+    wd = _stage(w_int8, dev)
+    out = torch.empty(((N + 15) // 16) * 16 * K, dtype=torch.int8, device=dev)
+    torch.ops.hexmi.pack_w8(wd, out)
+    return out
+
+
+def w8a16_matmul_packed(a, w_packed, scales, out=None):
+    """`w8a16_matmul` on weights packed by `pack_w8` (N = len(scales)); same result, bit for bit."""
+    if a.dtype != torch.float16 or w_packed.dtype != torch.int8 or scales.dtype != torch.float16:
+        raise TypeError("hexmi.w8a16_matmul_packed: expected fp16 activations, packed int8 weights, fp16 scales")
+    if a.dim() != 2 or scales.dim() != 1:
+        raise ValueError("hexmi.w8a16_matmul_packed: shapes A[M,K], scales[N] required")
+    M, K = a.shape
+    N = scales.shape[0]
+    if w_packed.numel() != ((N + 15) // 16) * 16 * K:
+        raise ValueError("hexmi.w8a16_matmul_packed: packed weights do not match N=%d, K=%d" % (N, K))
+    dev = _device() if a.device.type != "cuda" else a.device
+    ad, wd, sd = _stage(a, dev), _stage(w_packed, dev), _stage(scales, dev)
+    od = _out_like(out, (M, N), torch.float16, dev)
+    torch.ops.hexmi.w8a16_matmul_packed(ad, wd, sd, od)
     return _finish(od, out)
 
 

@@ -122,6 +122,25 @@ int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void *A,
 int hexmi_dequant_w8(int64_t N, int64_t K, const int8_t *W, const void *scales,
                      float *out, hexmi_stream_t stream);
 
+/* One-time weight pre-pack for the small-M path: the analogue of the
+ * reference's compile-time re-layout of constant matmul weights into the
+ * matrix unit's own order (RM -> WH block linearisation,
+ * qcom_hexagon_backend/lib/Transforms/PreprocessWeightsForHMXPass.cpp:39-117).
+ * Wp holds ceil(N/16)*16*K bytes: tiles of 16 channels x 64 k, tile (t, s) at
+ * byte ((t * K/64) + s) * 1024; inside a tile lane l = g*16 + r (0 <= l < 64)
+ * holds the 16 bytes W[16t + r][64s + 16g .. 64s + 16g + 16); channels past N
+ * are zero. K % 64 == 0. A pure permutation of bytes: bit-exact. */
+int hexmi_pack_w8(int64_t N, int64_t K, const int8_t *W, int8_t *Wp,
+                  hexmi_stream_t stream);
+
+/* hexmi_gemm_w8a16 on weights packed by hexmi_pack_w8: every weight load of a
+ * wave is a contiguous KiB already in MFMA fragment order. K % 1024 == 0 and
+ * K <= 4096. Meant for M <= 16 (decode batches); larger M runs 16 rows per
+ * launch. Same results as hexmi_gemm_w8a16, bit for bit. */
+int hexmi_gemm_w8a16_packed(int64_t M, int64_t N, int64_t K, const void *A,
+                            const int8_t *Wp, const void *scales, void *C,
+                            hexmi_stream_t stream);
+
 /* Attention -------------------------------------------------------------- */
 
 /* O = softmax(sm_scale * Q K^T [+ causal mask]) V per (z, h), online softmax

@@ -20,7 +20,7 @@ def test_header_declares_expected_entry_points():
     names = _declared()
     for must in ("hexmi_softmax", "hexmi_rms_norm", "hexmi_layer_norm", "hexmi_matmul_f16f16_f32", "hexmi_gemm",
                  "hexmi_gemm_w8a16", "hexmi_dequant_w8", "hexmi_flash_attn_fwd", "hexmi_attention", "hexmi_unary",
-                 "hexmi_binary", "hexmi_block_sum", "hexmi_rope"):
+                 "hexmi_binary", "hexmi_block_sum", "hexmi_rope", "hexmi_pack_w8", "hexmi_gemm_w8a16_packed"):
         assert must in names
 
 

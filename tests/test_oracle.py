@@ -378,3 +378,17 @@ def test_rope_vs_reference_formula(oracle):
     assert np.allclose((pairs_out ** 2).sum(-1), (pairs_in ** 2).sum(-1), rtol=1e-5)   # rotations keep the norm
     x2 = torch.randn(1, 300, 2, 64, generator=g)
     assert np.allclose(oracle.rope(x2.numpy(), 500.0), _rope_torch(x2, 500.0).numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_pack_w8_is_the_documented_permutation(oracle):
+    # independent statement with reshape / transpose: [T,16,S,4,16] -> [T,S,4,16,16]
+    g = torch.Generator().manual_seed(33)
+    w = torch.randint(-128, 128, (40, 192), generator=g, dtype=torch.int8).numpy()
+    got = oracle.pack_w8(w)
+    padded = np.zeros((48, 192), np.int8)
+    padded[:40] = w
+    want = padded.reshape(3, 16, 3, 4, 16).transpose(0, 2, 3, 1, 4).reshape(-1)
+    assert np.array_equal(got, want)
+    # every input byte appears exactly once (pure permutation plus zero padding)
+    ids = (np.arange(48 * 192, dtype=np.int64) % 251).astype(np.int8).reshape(48, 192)
+    assert sorted(oracle.pack_w8(ids).tolist()) == sorted(ids.reshape(-1).tolist())

@@ -104,3 +104,33 @@ def test_w8a16_errors(hexmi):
     with pytest.raises(hexmi.HexmiError):                     # K not a multiple of 64
         hexmi.w8a16_matmul(torch.zeros(2, 40, dtype=torch.float16).cuda(), torch.zeros(4, 40, dtype=torch.int8).cuda(),
                            torch.zeros(4, dtype=torch.float16).cuda())
+
+
+@pytest.mark.parametrize("N,K", [(48, 1024), (1000, 2048), (11008, 4096), (17, 1024)])
+def test_pack_w8_bit_exact(hexmi, oracle, N, K):
+    w = torch.randint(-128, 128, (N, K), generator=_gen(5), dtype=torch.int8)
+    got = hexmi.pack_w8(w.cuda()).cpu().numpy()
+    if N * K <= 2 ** 21:
+        assert np.array_equal(got, oracle.pack_w8(w.numpy()))
+    T = (N + 15) // 16
+    padded = torch.zeros(T * 16, K, dtype=torch.int8)
+    padded[:N] = w
+    want = padded.view(T, 16, K // 64, 4, 16).permute(0, 2, 3, 1, 4).reshape(-1)
+    assert np.array_equal(got, want.numpy())
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 40])
+@pytest.mark.parametrize("N,K", [(96, 1024), (1000, 2048), (11008, 4096), (11, 4096)])
+def test_w8a16_packed_equals_unpacked(hexmi, oracle, M, N, K):
+    a, w, s = _inputs(M, N, K, seed=6)
+    wp = hexmi.pack_w8(w.cuda())
+    got = hexmi.w8a16_matmul_packed(a.cuda(), wp, s.cuda()).cpu()
+    if N <= 1000:
+        want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w.numpy(), s.numpy()))
+        assert close16(got, want, max_ulp=1, atol=2e-4)
+    ref = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
+    assert close16(got, ref, max_ulp=1, atol=2e-4)            # other kernels sum in another order
+    if 2 < M <= 16:
+        assert torch.equal(got, ref)                          # same kernel, same arithmetic: bit for bit
+    with pytest.raises(ValueError):
+        hexmi.w8a16_matmul_packed(a.cuda(), wp[:-16], s.cuda())
