@@ -443,6 +443,81 @@ void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT*
   }
 }
 
+// fp32 inputs (the reference's torch-mlir graphs multiply fp32 matrices, e.g.
+// test/python/torch-mlir/test_add_matmul_softmax.py:25-29): 64x64 tile, K in steps of 16 through LDS, every thread a
+// 4x4 block of fp32 FMAs. Any shape; not a matrix-core path (no fp16 rounding of the operands).
+template <bool TRANS_B>
+__global__ __launch_bounds__(256)
+void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C, int M, int N,
+                     int K, int64_t lda, int64_t ldb, int64_t ldc) {
+  constexpr int TB = 64, TK = 16;
+  __shared__ float a_s[TK][TB + 4];                  // [k][m]
+  __shared__ float b_s[TK][TB + 4];                  // [k][n]
+  const int m0 = blockIdx.y * TB, n0 = blockIdx.x * TB;
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;   // thread owns rows ty*4.., columns tx*4..
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+  for (int k0 = 0; k0 < K; k0 += TK) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < TB * TK; e += 256) {
+      {
+        const int r = e / TK, k = e % TK;            // A: consecutive threads walk k (contiguous in memory)
+        const int gm = m0 + r, gk = k0 + k;
+        a_s[k][r] = (gm < M && gk < K) ? A[(int64_t)gm * lda + gk] : 0.0f;
+      }
+      if (TRANS_B) {
+        const int r = e / TK, k = e % TK;            // B[n][k]
+        const int gn = n0 + r, gk = k0 + k;
+        b_s[k][r] = (gn < N && gk < K) ? B[(int64_t)gn * ldb + gk] : 0.0f;
+      } else {
+        const int k = e / TB, c = e % TB;            // B[k][n]: consecutive threads walk n
+        const int gn = n0 + c, gk = k0 + k;
+        b_s[k][c] = (gn < N && gk < K) ? B[(int64_t)gk * ldb + gn] : 0.0f;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < TK; ++k) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = a_s[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bv[j] = b_s[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gm = m0 + ty * 4 + i;
+    if (gm >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gn = n0 + tx * 4 + j;
+      if (gn < N) C[(int64_t)gm * ldc + gn] = acc[i][j];
+    }
+  }
+}
+
+int launch_f32(bool trans_b, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+               int64_t ldb, int64_t ldc, hipStream_t s) {
+  dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+  if (grid.y > 65535) return HEXMI_ENOTSUP;
+  const float* a = static_cast<const float*>(A);
+  const float* b = static_cast<const float*>(B);
+  float* c = static_cast<float*>(C);
+  if (trans_b)
+    hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, s, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc);
+  else
+    hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, s, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc);
+  return launch_status();
+}
+
 template <typename T, typename OutT, int WM, int WN, bool TRANS_B>
 int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                  int64_t ldc, hipStream_t s) {
@@ -524,6 +599,7 @@ extern "C" int hexmi_gemm(int64_t M, int64_t N, int64_t K, const void* A, int64_
   if (K == 0) return HEXMI_ENOTSUP;
   hipStream_t s = as_stream(stream);
   const bool tb = trans_b != 0;
+  if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) return launch_f32(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
   if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F16) return dispatch_trans<f16, f16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
   if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F32) return dispatch_trans<f16, float>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
   if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_BF16) return dispatch_trans<bf16, bf16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);

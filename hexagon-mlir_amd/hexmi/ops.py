@@ -253,13 +253,15 @@ def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=No
 
 
 def matmul(a, b, out=None, out_dtype=None, trans_b=False):
-    """C = A @ B (or A @ B.T when trans_b), fp16/bf16 inputs, fp32 accumulation.
-    out_dtype: the input dtype (default) or torch.float32
+    """C = A @ B (or A @ B.T when trans_b), fp16/bf16 inputs with fp32 accumulation on the matrix cores, or fp32
+    inputs with fp32 FMAs. out_dtype: the input dtype (default) or torch.float32
     (test/python/triton/test_matmul.py:35-91; docs/tutorials/triton/matmul_hexkl.md:61-111)."""
     if a.dim() != 2 or b.dim() != 2:
         raise ValueError("hexmi.matmul takes 2-D tensors")
-    if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16):
-        raise TypeError("hexmi.matmul: A and B must both be float16 or both bfloat16")
+    if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise TypeError("hexmi.matmul: A and B must both be float16, both bfloat16 or both float32")
+    if a.dtype == torch.float32 and (out_dtype or (out.dtype if out is not None else torch.float32)) != torch.float32:
+        raise TypeError("hexmi.matmul: float32 operands give a float32 result")
     M, K = a.shape
     N = b.shape[0] if trans_b else b.shape[1]
     if (b.shape[1] if trans_b else b.shape[0]) != K:
@@ -437,3 +439,16 @@ def rope(x, theta=10000.0, out=None):
     od = _out_like(out, x.shape, x.dtype, dev)
     torch.ops.hexmi.rope(xd, float(theta), od)
     return _finish(od, out)
+
+
+def add_matmul_softmax(x, y, z, out=None):
+    """softmax((x + y) @ z, dim=-1): the graph of test/python/torch-mlir/test_add_matmul_softmax.py:19-29, which the
+    reference compiles into one fused kernel; here the three kernels run back to back on one stream."""
+    if x.shape != y.shape or x.dim() != 2 or z.dim() != 2 or x.shape[1] != z.shape[0]:
+        raise ValueError("hexmi.add_matmul_softmax: x, y [M,K] and z [K,N] required")
+    if not (x.dtype == y.dtype == z.dtype):
+        raise TypeError("hexmi.add_matmul_softmax: operand dtypes differ")
+    dev = _device() if x.device.type != "cuda" else x.device
+    total = binary("add", _stage(x, dev), _stage(y, dev))
+    product = matmul(total, _stage(z, dev))
+    return softmax(product, out=out)

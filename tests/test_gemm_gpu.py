@@ -165,8 +165,38 @@ def test_gemm_argument_errors(hexmi):
     a = torch.zeros(8, 8, device="cuda", dtype=torch.float16)
     lib = _lib.lib()
     assert lib.hexmi_gemm(8, 8, 8, a.data_ptr(), 4, a.data_ptr(), 8, a.data_ptr(), 8, _lib.F16, _lib.F16, 0, None) == _lib.EINVAL
-    assert lib.hexmi_gemm(8, 8, 8, a.data_ptr(), 8, a.data_ptr(), 8, a.data_ptr(), 8, _lib.F32, _lib.F32, 0, None) == _lib.ENOTSUP
+    assert lib.hexmi_gemm(8, 8, 8, a.data_ptr(), 8, a.data_ptr(), 8, a.data_ptr(), 8, _lib.F32, _lib.F16, 0, None) == _lib.ENOTSUP
+    assert lib.hexmi_gemm(8, 8, 8, a.data_ptr(), 8, a.data_ptr(), 8, a.data_ptr(), 8, _lib.F16, _lib.BF16, 0, None) == _lib.ENOTSUP
     with pytest.raises(TypeError):
-        hexmi.matmul(torch.zeros(4, 4, device="cuda"), torch.zeros(4, 4, device="cuda"))
+        hexmi.matmul(torch.zeros(4, 4, device="cuda", dtype=torch.float64), torch.zeros(4, 4, device="cuda", dtype=torch.float64))
     with pytest.raises(ValueError):
         hexmi.matmul(a, torch.zeros(4, 4, device="cuda", dtype=torch.float16))
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("shape", [(32, 32, 32), (1, 1, 1), (65, 130, 17), (200, 77, 300), (512, 512, 512)])
+def test_matmul_fp32(hexmi, oracle, shape, trans_b):
+    M, N, K = shape
+    g = torch.Generator().manual_seed(40)
+    a = torch.randn(M, K, generator=g)
+    b = torch.randn(N, K, generator=g) if trans_b else torch.randn(K, N, generator=g)
+    got = hexmi.matmul(a.cuda(), b.cuda(), trans_b=trans_b).cpu()
+    want = a.double() @ (b.double().t() if trans_b else b.double())
+    assert got.dtype == torch.float32
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5 * (K ** 0.5))
+    with pytest.raises(TypeError):
+        hexmi.matmul(a.cuda(), b.cuda(), trans_b=trans_b, out_dtype=torch.float16)
+
+
+def test_add_matmul_softmax_reference_graph(hexmi):
+    # test/python/torch-mlir/test_add_matmul_softmax.py:32-60: three 32x32 fp32 randn, rtol 1e-5, atol 1e-6
+    g = torch.Generator().manual_seed(41)
+    x, y, z = (torch.randn(32, 32, generator=g) for _ in range(3))
+    got = hexmi.add_matmul_softmax(x, y, z)
+    want = torch.nn.functional.softmax(torch.matmul(x + y, z), dim=-1)
+    assert got.device.type == "cuda"
+    assert torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-6)
+    # fp16 operands run the matrix-core GEMM
+    got16 = hexmi.add_matmul_softmax(x.half(), y.half(), z.half()).cpu()
+    want16 = torch.nn.functional.softmax(torch.matmul((x.half() + y.half()).float(), z.half().float()), dim=-1)
+    assert torch.allclose(got16.float(), want16, atol=2e-2)
