@@ -28,11 +28,15 @@ __device__ __forceinline__ float unary(float x) {
     // 0.5*x*(1 + tanh(u)), u = 0.797885*x + 0.035677*x^3, tanh(u) = (1 - e^-2u) / (1 + e^-2u)
     // (test/python/triton/test_gelu.py:26-30,54). 0.5*(1 + tanh(u)) = 1 / (1 + e^-2u): the same function without
     // the cancellation in 1 + tanh(u) for negative u, and e^-2u = inf gives 0 instead of inf/inf.
-    // v_exp_f32 and v_rcp_f32 (1 ulp each) keep the kernel bound by HBM rather than by the vector ALUs
-    const float u = 0.797885f * x + 0.035677f * x * x * x;
-    return x * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
+    // v_exp_f32 and v_rcp_f32 (1 ulp each) and the constants folded into the exp2 argument,
+    // e^-2u = 2^(x * (a + b x^2)), a = -2 log2(e) * 0.797885, b = -2 log2(e) * 0.035677, keep the kernel bound
+    // by HBM rather than by the vector ALUs (eight fp16 elements per 16-byte access).
+    constexpr float a = -2.0f * 1.44269504088896340736f * 0.797885f;
+    constexpr float b = -2.0f * 1.44269504088896340736f * 0.035677f;
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * fmaf(b, x * x, a)));
   } else if constexpr (OP == HEXMI_SILU) {
-    return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x));   // x / (1 + e^-x), test/python/triton/test_silu.py:50
+    // x / (1 + e^-x), test/python/triton/test_silu.py:50
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896340736f));
   } else if constexpr (OP == HEXMI_RSQRT) {
     return 1.0f / sqrtf(x);                          // test/python/triton/test_rsqrt.py:20-24
   } else if constexpr (OP == HEXMI_SIN) {
@@ -129,9 +133,9 @@ void binary_scalar_kernel(const T* __restrict__ a, const T* __restrict__ b, T* _
 // out[p] = sum(x[p*block .. (p+1)*block)), one workgroup per program of the reference's launch grid
 // (test/python/triton/test_sum.py:30-36: `tl.store(output_ptr + pid, tl.sum(x))`). fp32 accumulation in a fixed
 // order (per-thread strided partials, wave butterfly, waves in order): the result does not depend on timing.
-constexpr int kSumThreads = 1024;
-
-template <typename T>
+// kSumThreads threads per program: 1024 for large blocks (a single program must pull its block through one CU),
+// 256 for blocks up to 64 KiB (several 16-byte loads in flight per thread, a cheaper final exchange).
+template <typename T, int kSumThreads>
 __global__ __launch_bounds__(kSumThreads)
 void block_sum_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t block, int64_t n) {
   constexpr int N = Chunk<T>::N;
@@ -301,8 +305,12 @@ template <typename T>
 int launch_block_sum(const void* x, void* out, int64_t n, int64_t block, hipStream_t s) {
   const int64_t programs = (n + block - 1) / block;
   if (programs > 0x7fffffff) return HEXMI_ENOTSUP;
-  hipLaunchKernelGGL((block_sum_kernel<T>), dim3((unsigned)programs), dim3(kSumThreads), 0, s,
-                     static_cast<const T*>(x), static_cast<T*>(out), block, n);
+  if (block * (int64_t)sizeof(T) <= 65536)
+    hipLaunchKernelGGL((block_sum_kernel<T, 256>), dim3((unsigned)programs), dim3(256), 0, s,
+                       static_cast<const T*>(x), static_cast<T*>(out), block, n);
+  else
+    hipLaunchKernelGGL((block_sum_kernel<T, 1024>), dim3((unsigned)programs), dim3(1024), 0, s,
+                       static_cast<const T*>(x), static_cast<T*>(out), block, n);
   return launch_status();
 }
 
