@@ -90,13 +90,17 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
   const float inv_n = 1.0f / (float)cols;
 
   Vec16<T> wv[CHUNKS], bv[CHUNKS];
+  float wf[PIPE ? CHUNKS : 1][N], bf[PIPE ? CHUNKS : 1][N];   // PIPE: weight and bias resident as fp32
   if constexpr (PIPE && OP != kSoftmax) {
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
       const int col = (c * THREADS + t) * N;
-      if (col < cols) {
-        if (w) wv[c] = load16(w + col);
-        if (OP == kLayerNorm && b) bv[c] = load16(b + col);
+      if (w) wv[c] = load16(w + col);
+      if (OP == kLayerNorm && b) bv[c] = load16(b + col);
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        wf[c][i] = w ? to_f32<T>(wv[c].v[i]) : 1.0f;
+        bf[c][i] = (OP == kLayerNorm && b) ? to_f32<T>(bv[c].v[i]) : 0.0f;
       }
     }
   }
@@ -206,18 +210,29 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
         const int col = (c * THREADS + t) * N;
         if (FULL || (col < cols && row_valid)) {
           Vec16<T> o;
-          if (w) {
-            if constexpr (!PIPE) wv[c] = load16(w + col);
+          if constexpr (PIPE) {
+            // (x - mean) * rstd * w + b with the last two steps fused; w = 1 / b = 0 stand in for absent operands
+            if (OP == kLayerNorm && b) {
 #pragma unroll
-            for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd * to_f32<T>(wv[c].v[i]);
+              for (int i = 0; i < N; ++i) v[c][i] = fmaf(v[c][i] * rstd, wf[c][i], bf[c][i]);
+            } else {
+#pragma unroll
+              for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd * wf[c][i];
+            }
           } else {
+            if (w) {
+              wv[c] = load16(w + col);
 #pragma unroll
-            for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd;
-          }
-          if (OP == kLayerNorm && b) {
-            if constexpr (!PIPE) bv[c] = load16(b + col);
+              for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd * to_f32<T>(wv[c].v[i]);
+            } else {
 #pragma unroll
-            for (int i = 0; i < N; ++i) v[c][i] += to_f32<T>(bv[c].v[i]);
+              for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd;
+            }
+            if (OP == kLayerNorm && b) {
+              bv[c] = load16(b + col);
+#pragma unroll
+              for (int i = 0; i < N; ++i) v[c][i] += to_f32<T>(bv[c].v[i]);
+            }
           }
 #pragma unroll
           for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i]);
