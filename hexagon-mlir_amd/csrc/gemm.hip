@@ -54,15 +54,15 @@ constexpr int waitcnt_imm(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | (7 <
 
 // global -> LDS copy of a [ROWS x 32] K-contiguous slab: ROWS/64 wave-wide instructions per wave, 16 rows each.
 // Rows past row_max are clamped (their products are never stored).
-template <typename T, int ROWS>
+template <typename T, int ROWS, int NW = 4>
 struct KMajorLoader {
-  static constexpr int NI = ROWS / 64;
+  static constexpr int NI = ROWS / (16 * NW);
   const T* ptr[NI];
   int lds_off[NI];
   __device__ __forceinline__ void init(const T* g, int64_t ld, int row0, int row_max, int wave, int lane) {
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
-      const int inst = j * 4 + wave;
+      const int inst = j * NW + wave;
       const int row = inst * 16 + lane / 4;
       const int c = (lane % 4) ^ swz_k(row);
       int grow = row0 + row;
@@ -77,9 +77,9 @@ struct KMajorLoader {
 };
 
 // global -> LDS copy of a [32 x COLS] N-contiguous slab; column chunks past col_max are clamped.
-template <typename T, int COLS>
+template <typename T, int COLS, int NW = 4>
 struct NMajorLoader {
-  static constexpr int NI = COLS / 64;
+  static constexpr int NI = COLS / (16 * NW);
   static constexpr int CPR = COLS / kChunk;         // chunks per row
   const T* ptr[NI];
   int lds_off[NI];
@@ -88,7 +88,7 @@ struct NMajorLoader {
     ld = ld_;
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
-      const int inst = j * 4 + wave;
+      const int inst = j * NW + wave;
       const int lin = inst * 64 + lane;
       const int k = lin / CPR;
       const int c = (lin % CPR) ^ swz_n(k);
@@ -212,14 +212,19 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
 // K % 32 == 0. TAIL: the slab count is not a multiple of 4, so the last pass over the four stages guards its MFMAs.
 // B_I8: B is int8 [N,K] (weight-only quantisation, needs TRANS_B and T = fp16); its slabs are copied raw into
 // LDS, converted to fp16 LDS -> LDS one slab later, and the result is multiplied by scales[column].
-template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false>
-__global__ __launch_bounds__(256)
+// NWN: waves along N (2: four waves, one per SIMD, each WM x WN tiles of 32x32; 4: eight waves, two per SIMD).
+// The eight-wave 256x256 form (WM = 4, WN = 2) measured the same as four waves with 4x4 tiles on both benchmark
+// shapes: on random data the kernel is held back by the power limit, not by issue stalls a second wave could fill.
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false, int NWN = 2>
+__global__ __launch_bounds__(NWN * 128)
 void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __restrict__ C, int M, int N, int K,
                  int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
                  const f16* __restrict__ scales = nullptr) {
   const T* B = static_cast<const T*>(Bv);
   typedef typename Mfma<T>::Frag Frag;
-  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  constexpr int NW = 2 * NWN;                       // waves per workgroup
+  constexpr int BM = 2 * WM * 32, BN = NWN * WN * 32;
+  static_assert(!B_I8 || NWN == 2, "the int8 loader is written for four waves");
   __shared__ __attribute__((aligned(16))) T a_s0[BM * BK];
   __shared__ __attribute__((aligned(16))) T a_s1[BM * BK];
   __shared__ __attribute__((aligned(16))) T a_s2[BM * BK];
@@ -235,7 +240,7 @@ void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __r
   __shared__ __attribute__((aligned(16))) int8_t r_s3[B_I8 ? BN * BK : 16];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int wm = wave / 2, wn = wave % 2;
+  const int wm = wave / NWN, wn = wave % NWN;
   int tm, tn;
   tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
@@ -248,16 +253,16 @@ void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __r
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  KMajorLoader<T, BM> load_a;
+  KMajorLoader<T, BM, NW> load_a;
   load_a.init(A, lda, m0, M - 1, wave, lane);
-  KMajorLoader<T, BN> load_bk;
-  NMajorLoader<T, BN> load_bn;
+  KMajorLoader<T, BN, NW> load_bk;
+  NMajorLoader<T, BN, NW> load_bn;
   I8Loader<BN> load_b8;
   if constexpr (B_I8) load_b8.init(static_cast<const int8_t*>(Bv), ldb, n0, N - 1, wave, lane, threadIdx.x);
   else if constexpr (TRANS_B) load_bk.init(B, ldb, n0, N - 1, wave, lane);
   else load_bn.init(B, ldb, n0, N - kChunk, wave, lane);
-  constexpr int NLA = BM / 64;                      // copy instructions per wave per slab (A)
-  constexpr int NLB = B_I8 ? I8Loader<BN>::NI : BN / 64;   // B copies per wave per slab
+  constexpr int NLA = BM / (16 * NW);               // copy instructions per wave per slab (A)
+  constexpr int NLB = B_I8 ? I8Loader<BN>::NI : BN / (16 * NW);   // B copies per wave per slab
 
   // part 0 = the A copies of slab kt, part 1 = its B copies
   auto issue_part = [&](int kt, T* a_dst, T* b_dst, auto part) {
@@ -518,17 +523,17 @@ int launch_f32(bool trans_b, const void* A, const void* B, void* C, int64_t M, i
   return launch_status();
 }
 
-template <typename T, typename OutT, int WM, int WN, bool TRANS_B>
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B, int NWN = 2>
 int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                  int64_t ldc, hipStream_t s) {
-  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  constexpr int BM = 2 * WM * 32, BN = NWN * WN * 32;
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   if ((K / BK) % 4 == 0)
-    hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, false>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A, B,
-                       C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, false, false, NWN>), dim3(tiles_m * tiles_n),
+                       dim3(NWN * 128), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
   else
-    hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, true>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A, B,
-                       C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, true, false, NWN>), dim3(tiles_m * tiles_n),
+                       dim3(NWN * 128), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
   return launch_status();
 }
 
