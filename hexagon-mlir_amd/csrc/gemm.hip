@@ -408,6 +408,300 @@ void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __r
   }
 }
 
+// ---- K % 64 == 0: paired slabs ------------------------------------------------------------------------------
+// A K-contiguous operand fetched 32 elements of K at a time touches half of a 128-byte line per row; the other
+// half is fetched one slab later, by which time the line has left the vector L1, so every line crosses
+// L2 -> L1 twice. Here a stage holds 64 elements of K: each row of a copy is one whole line (8 lanes x 16 bytes),
+// the L2 request count halves, and one barrier serves 64 elements of K instead of 32.
+constexpr int BK2 = 64;
+__device__ __forceinline__ int swz_k2(int row) { return (row >> 1) & 7; }      // row pitch 128 B: 16 rows, 16 slots
+// N-contiguous tiles: 32 lanes of a transposing read touch 8 rows (k%4, k/8%2) x 32 bytes of one column block;
+// the XOR spreads them over the eight 32-byte slots of 256 bytes of banks. A row's chunks stay whole 128-byte lines.
+__device__ __forceinline__ int swz_n2(int k) { return ((k & 3) | (((k >> 3) & 1) << 2)) << 1; }
+
+// Copies are buffer loads into LDS: the address is a uniform base (a buffer descriptor in scalar registers, rebuilt
+// per slab by scalar adds) plus a per-lane 32-bit byte offset that never changes, and the LDS destination is a
+// scalar, so a copy costs no vector arithmetic. Offsets stay below 2^31 (checked by the launcher); rows and column
+// chunks outside the matrix are clamped by the loaders, the descriptor's own range check is left wide open.
+template <typename T>
+__device__ __forceinline__ void copy_to_lds(const char* base, int voff, T* lds) {
+#if defined(__HIP_DEVICE_COMPILE__)        // the descriptor type exists in the device pass only
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, 0x7fffffff, 0x00020000);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, HEXMI_LDS(lds), 16, voff, 0, 0, 0);
+#endif
+}
+
+template <typename T, int ROWS>
+struct KMajorLoader2 {
+  static constexpr int NI = ROWS / 32;              // 8 rows per wave-wide copy, four waves
+  int voff[NI];
+  int lds_off[NI];
+  // row0 + row is clamped to row_max; offsets are relative to row row0 of g
+  __device__ __forceinline__ void init(int64_t ld, int row0, int row_max, int wave, int lane) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int inst = j * 4 + wave;
+      const int row = inst * 8 + lane / 8;
+      const int c = (lane % 8) ^ swz_k2(row);
+      int grow = row0 + row;
+      grow = grow < row_max ? grow : row_max;
+      voff[j] = (int)(((int64_t)(grow - row0) * ld + c * kChunk) * (int64_t)sizeof(T));
+      lds_off[j] = inst * 8 * BK2;
+    }
+  }
+  __device__ __forceinline__ void issue(int j, T* lds, const char* base) const {   // j: an unrolled constant
+    if (j < NI) copy_to_lds(base, voff[j], lds + lds_off[j]);
+  }
+};
+
+template <typename T, int COLS>
+struct NMajorLoader2 {
+  static constexpr int NI = COLS / 32;              // [64 x COLS] elements, 512 per copy, four waves
+  static constexpr int CPR = COLS / kChunk;
+  int voff[NI];
+  int lds_off[NI];
+  // column chunks past col_max are clamped; offsets are relative to column col0 of row 0 of g
+  __device__ __forceinline__ void init(int64_t ld, int col0, int col_max, int wave, int lane) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int inst = j * 4 + wave;
+      const int lin = inst * 64 + lane;
+      const int k = lin / CPR;
+      const int c = (lin % CPR) ^ swz_n2(k);
+      int gcol = col0 + c * kChunk;
+      gcol = gcol < col_max ? gcol : col_max;
+      voff[j] = (int)(((int64_t)k * ld + (gcol - col0)) * (int64_t)sizeof(T));
+      lds_off[j] = inst * 64 * kChunk;
+    }
+  }
+  __device__ __forceinline__ void issue(int j, T* lds, const char* base) const {   // j: an unrolled constant
+    if (j < NI) copy_to_lds(base, voff[j], lds + lds_off[j]);
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::Frag read_kmajor2(const T* lds, int row, int chunk) {
+  typedef typename Mfma<T>::Frag Frag;
+  return *reinterpret_cast<const Frag*>(lds + row * BK2 + ((chunk ^ swz_k2(row)) * kChunk));
+}
+
+// ds_read_tr16_b64: 16 lanes hand in the addresses of a [4 k x 16 columns] block (lane i: row i/4, columns
+// 4*(i%4)..+3) and lane i receives column i's four k values; two of them give a lane 8 consecutive k.
+template <typename T, int COLS>
+__device__ __forceinline__ typename Mfma<T>::Frag read_nmajor2(const T* lds, int col_tile, int ks, int lane) {
+  typedef typename Mfma<T>::Frag Frag;
+  constexpr int CPR = COLS / kChunk;
+  const int g = lane / 16, i = lane % 16;
+  const int n = col_tile + (i & 3) * 4;
+  const int kb = ks * 32 + g * 8 + (i >> 2);
+  union { i16x4 h[2]; Frag f; } u;
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int k = kb + p * 4;
+    const int c = (n / kChunk) ^ swz_n2(k);
+    const T* addr = lds + (k * CPR + c) * kChunk + (n % kChunk);
+    u.h[p] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
+  }
+  return u.f;
+}
+
+// The accumulator is tied to the destination in inline assembly: left to the compiler, the 16x16x32 builtin gets
+// a destination register of its own and a copy back per instruction. Each accumulator is touched once per 64
+// MFMAs, far beyond the instruction's latency, and the epilogue reads them after the copy drain and its address
+// arithmetic, so no wait states are missing around the assembly.
+template <typename T> struct Mfma16;
+template <> struct Mfma16<f16> {
+  static __device__ __forceinline__ void run(const f16x8& a, const f16x8& b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+template <> struct Mfma16<bf16> {
+  static __device__ __forceinline__ void run(const bf16x8& a, const bf16x8& b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+
+// Two stages of [tile x 64], MFMA 16x16x32 (on random data the chip runs at its power limit, and this shape
+// sustains about 12 % more than 32x32x16 there: it updates a quarter of the accumulators per instruction for half
+// the products). A wave owns TM x TN tiles of 16x16 and runs, per paired slab j, two steps of 32 elements of K;
+// each step is two phases of TM/2 * TN MFMAs. Fragments of the next step are read while the current one
+// multiplies. The copies of slab j+1 are issued in phase 3 of slab j-1 (A) and phase 0 of slab j (B), into the
+// stage slab j-1 was read from; the one barrier, between phases 2 and 3, comes after every wave's last read of
+// slab j and after all of slab j+1 has landed. TAIL: the slab count is odd.
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL>
+__global__ __launch_bounds__(256)
+void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __restrict__ C, int M, int N, int K,
+                     int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n) {
+  typedef typename Mfma<T>::Frag Frag;
+  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  constexpr int TM = 2 * WM, TN = 2 * WN;           // 16x16 tiles per wave
+  __shared__ __attribute__((aligned(16))) T a_p0[BM * BK2];
+  __shared__ __attribute__((aligned(16))) T a_p1[BM * BK2];
+  __shared__ __attribute__((aligned(16))) T b_p0[BN * BK2];
+  __shared__ __attribute__((aligned(16))) T b_p1[BN * BK2];
+
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // scalar: LDS destinations stay scalar
+  const int wm = wave / 2, wn = wave % 2;
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  f32x4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+
+  KMajorLoader2<T, BM> load_a;
+  load_a.init(lda, m0, M - 1, wave, lane);
+  KMajorLoader2<T, BN> load_bk;
+  NMajorLoader2<T, BN> load_bn;
+  if constexpr (TRANS_B) load_bk.init(ldb, n0, N - 1, wave, lane);
+  else load_bn.init(ldb, n0, N - kChunk, wave, lane);     // N % 8 == 0, so n0 <= N - 8
+  // uniform bases of this tile's operand panels; slab j adds j * (bytes per 64 elements of K)
+  const char* a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda);
+  const char* b_base = reinterpret_cast<const char*>(TRANS_B ? B + (int64_t)n0 * ldb : B + n0);
+  const int64_t a_step = BK2 * (int64_t)sizeof(T);
+  const int64_t b_step = (TRANS_B ? BK2 : BK2 * ldb) * (int64_t)sizeof(T);
+  constexpr int NLA = BM / 32, NLB = BN / 32;
+
+  static_assert(TM == TN && TN >= 4, "a round carries two fragment reads: 2*TM rounds read TM+TN fragments twice");
+  auto copy_a = [&](int i, const char* base, T* dst) __attribute__((always_inline)) {
+    load_a.issue(i, dst, base);
+  };
+  auto copy_b = [&](int i, const char* base, T* dst) __attribute__((always_inline)) {
+    if constexpr (TRANS_B) load_bk.issue(i, dst, base);
+    else load_bn.issue(i, dst, base);
+  };
+  // fragments of step ks (32 elements of K): lane holds row/column lane%16 of a tile, K group lane/16 (8 elements)
+  auto read_a = [&](const T* src, int ks, int i) __attribute__((always_inline)) {
+    return read_kmajor2<T>(src, (wm * TM + i) * 16 + lane % 16, ks * 4 + lane / 16);
+  };
+  auto read_b = [&](const T* src, int ks, int j) __attribute__((always_inline)) {
+    if constexpr (TRANS_B) return read_kmajor2<T>(src, (wn * TN + j) * 16 + lane % 16, ks * 4 + lane / 16);
+    else return read_nmajor2<T, BN>(src, (wn * TN + j) * 16, ks, lane);
+  };
+  auto mfma_row = [&](const Frag* af, const Frag* bf, int i) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) Mfma16<T>::run(bf[j], af[i], acc[i][j]);
+  };
+  const int KT = K / BK2;
+  auto clampj = [&](int j) { return j < KT ? j : KT - 1; };      // past the end: reload the last slab (never used)
+
+  // Copy n of a slab: the NLA copies of A, then the NLB of B.
+  constexpr int NL = NLA + NLB;
+  auto copy_n = [&](int n, int slab, T* a_dst, T* b_dst) __attribute__((always_inline)) {
+    if constexpr (TRANS_B) {
+      if (n < NLA) copy_a(n, a_base + slab * a_step, a_dst);
+      else copy_b(n - NLA, b_base + slab * b_step, b_dst);
+    } else {
+      if (n < NLB) copy_b(n, b_base + slab * b_step, b_dst);
+      else copy_a(n - NLB, a_base + slab * a_step, a_dst);
+    }
+  };
+  // Fragment n of a step: the TN of B (every MFMA row needs all of them), then the TM of A in row order.
+  auto read_n = [&](int n, const T* a_src, const T* b_src, int ks, Frag* af_dst, Frag* bf_dst) __attribute__((always_inline)) {
+    if (n < TN) bf_dst[n] = read_b(b_src, ks, n);
+    else af_dst[n - TN] = read_a(a_src, ks, n - TN);
+  };
+
+  Frag af[2][TM], bf[2][TN];
+  // A slab's copies are issued in the window between the barrier that frees their stage and the next barrier:
+  // copies_before(w) of them before round w of the window (2*TM rounds). LATE of them fall after the slab boundary,
+  // so the prologue leaves slab 1's last LATE copies to slab 0.
+  // K-contiguous B: two copies in each of the TM rounds after the barrier (longest lead); N-contiguous B: two in
+  // each of the first TM/2 rounds, then one per round, the last TM/2 of them after the slab boundary. Measured on
+  // 8192^3 bf16 against five other placements.
+  auto copies_before = [](int w) constexpr {
+    int sum = 0;
+    for (int r = 0; r < w; ++r) {
+      if (TRANS_B) sum += r < TM ? 2 : 0;
+      else sum += r < TM / 2 ? 2 : (r < TM + TM / 2 ? 1 : 0);
+    }
+    return sum;
+  };
+  constexpr int LATE = NL - copies_before(TM);
+  static_assert(copies_before(2 * TM) == NL, "the window carries all of a slab's copies");
+#pragma unroll
+  for (int n = 0; n < NL; ++n) copy_n(n, 0, a_p0, b_p0);
+#pragma unroll
+  for (int n = 0; n < NL - LATE; ++n) copy_n(n, clampj(1), a_p1, b_p1);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(NL - LATE));             // slab 0 landed
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int n = 0; n < TM + TN; ++n) read_n(n, a_p0, b_p0, 0, af[0], bf[0]);
+
+  // The MFMAs are inline assembly, which the scheduler's group directives do not see, so the issue order is the
+  // source order, pinned by full scheduling fences. A slab is 2*TM rounds of TN MFMAs (one row of tiles); a round
+  // carries two fragment reads and up to two copies, one after every other MFMA. The barrier sits in the middle:
+  // by then every wave has read both steps of this slab, and all of the next slab has landed.
+#define HEXMI_FENCE __builtin_amdgcn_sched_barrier(0)
+  auto slab = [&](T* acur, T* bcur, T* anxt, T* bnxt, int j) __attribute__((always_inline)) {
+    const bool live = !TAIL || j < KT;
+    const int j1 = clampj(j + 1), j2 = clampj(j + 2);
+#pragma unroll
+    for (int q = 0; q < 2 * TM; ++q) {
+      const int ks = q / TM, row = q % TM;
+      if (q == TM) {
+        HEXMI_FENCE;
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+        __builtin_amdgcn_s_barrier();
+        HEXMI_FENCE;
+      }
+#pragma unroll
+      for (int jj = 0; jj < TN / 2; ++jj) {
+        if (live) {
+          Mfma16<T>::run(bf[ks][2 * jj], af[ks][row], acc[row][2 * jj]);
+          Mfma16<T>::run(bf[ks][2 * jj + 1], af[ks][row], acc[row][2 * jj + 1]);
+        }
+        HEXMI_FENCE;
+        // side instructions of slot jj of round q
+        if (jj < 2) {
+          // fragment reads: first half of the slab reads step 1 of this slab, second half step 0 of the next
+          const int n = row * 2 + jj;
+          if (ks == 0) read_n(n, acur, bcur, 1, af[1], bf[1]);
+          else read_n(n, anxt, bnxt, 0, af[0], bf[0]);
+        }
+        constexpr int CSLOT = (TN >= 8 && !TRANS_B) ? 2 : 0;   // first of the two copy slots of a round
+        if (jj >= CSLOT && jj < CSLOT + 2) {
+          // copies of the window that opened at this slab's barrier (rounds TM..2TM-1, slab j+2 into this slab's
+          // stage) and of the window that opened at the previous one (rounds 0.., slab j+1 into the other stage)
+          const int c = jj - CSLOT;
+          const int w = (q + TM) % (2 * TM);               // round index within its window
+          const int lo = copies_before(w), hi = copies_before(w + 1);
+          if (lo + c < hi) {
+            if (ks == 1) copy_n(lo + c, j2, acur, bcur);
+            else copy_n(lo + c, j1, anxt, bnxt);
+          }
+        }
+        HEXMI_FENCE;
+      }
+    }
+  };
+  for (int j = 0; j < KT; j += 2) {
+    slab(a_p0, b_p0, a_p1, b_p1, j);
+    slab(a_p1, b_p1, a_p0, b_p0, j + 1);
+  }
+#undef HEXMI_FENCE
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));       // drain the trailing copies before the workgroup's LDS goes away
+
+  // acc[i][j][r]: row lane%16 of tile row i, column 4*(lane/16) + r of tile column j
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int row = m0 + (wm * TM + i) * 16 + lane % 16;
+    if (row >= M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + (wn * TN + j) * 16 + 4 * (lane / 16);
+      if (col < N)
+        store4<OutT>(C + (int64_t)row * ldc + col, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+    }
+  }
+}
+
 // Any shape, any alignment: 64x64 tile, scalar guarded loads through LDS, MFMA 32x32x16 with zero padding.
 template <typename T, typename OutT, bool TRANS_B>
 __global__ __launch_bounds__(256)
@@ -528,6 +822,17 @@ int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t 
                  int64_t ldc, hipStream_t s) {
   constexpr int BM = 2 * WM * 32, BN = NWN * WN * 32;
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+  // K % 64 == 0: the paired-slab kernel; its per-lane copy offsets (up to 256 rows, or 64 rows of K) must stay
+  // below 2^31 bytes
+  if (NWN == 2 && K % BK2 == 0 && lda < (1 << 21) && ldb < (1 << 21)) {
+    if ((K / BK2) % 2 == 0)
+      hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, false>), dim3(tiles_m * tiles_n), dim3(256), 0, s,
+                         A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+    else
+      hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, true>), dim3(tiles_m * tiles_n), dim3(256), 0, s,
+                         A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+    return launch_status();
+  }
   if ((K / BK) % 4 == 0)
     hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, false, false, NWN>), dim3(tiles_m * tiles_n),
                        dim3(NWN * 128), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
