@@ -76,17 +76,17 @@ struct KvTileLoader {
   }
   __device__ __forceinline__ void issue(const T* __restrict__ g, int key0, int S, T* lds) const {
     if (key0 + kBlockN <= S) {
-      const T* base = g + (int64_t)key0 * D;
+      const char* base = reinterpret_cast<const char*>(g + (int64_t)key0 * D);
 #pragma unroll
-      for (int j = 0; j < NI; ++j)
-        __builtin_amdgcn_global_load_lds(HEXMI_GLB(base + off[j]), HEXMI_LDS(lds + lds_off[j]), 16, 0, 0);
+      for (int j = 0; j < NI; ++j) copy_to_lds(base, off[j] * (int)sizeof(T), lds + lds_off[j]);
     } else {
+      // ragged last tile: rows clamped to the last key, offsets from the head's first key (S*D*sizeof(T) < 2^31)
+      const char* base = reinterpret_cast<const char*>(g);
 #pragma unroll
       for (int j = 0; j < NI; ++j) {
         int key = key0 + row[j];
         key = key < S ? key : S - 1;
-        __builtin_amdgcn_global_load_lds(HEXMI_GLB(g + (int64_t)key * D + col[j]), HEXMI_LDS(lds + lds_off[j]), 16, 0,
-                                         0);
+        copy_to_lds(base, (key * D + col[j]) * (int)sizeof(T), lds + lds_off[j]);
       }
     }
   }
@@ -452,7 +452,9 @@ int launch_rowwise(const void* Q, const void* K, const void* V, const void* mask
 template <typename T, typename OutT>
 int dispatch_half(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
                   int64_t Skv, int64_t D, float scale_log2e, bool causal, hipStream_t st) {
-  const bool ok = aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16);
+  // the matrix-core kernels address a head's keys with 32-bit byte offsets
+  const bool ok = aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16) &&
+                  Skv * D * (int64_t)sizeof(T) < 0x7fffffff;
   const bool plain = !mask && Skv == S;
   if (ok && plain && D == 128) return launch_mfma<T, OutT, 128>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
   if (ok && plain && D == 64) return launch_mfma<T, OutT, 64>(Q, K, V, O, ZH, S, scale_log2e, causal, st);

@@ -419,17 +419,8 @@ __device__ __forceinline__ int swz_k2(int row) { return (row >> 1) & 7; }      /
 // the XOR spreads them over the eight 32-byte slots of 256 bytes of banks. A row's chunks stay whole 128-byte lines.
 __device__ __forceinline__ int swz_n2(int k) { return ((k & 3) | (((k >> 3) & 1) << 2)) << 1; }
 
-// Copies are buffer loads into LDS: the address is a uniform base (a buffer descriptor in scalar registers, rebuilt
-// per slab by scalar adds) plus a per-lane 32-bit byte offset that never changes, and the LDS destination is a
-// scalar, so a copy costs no vector arithmetic. Offsets stay below 2^31 (checked by the launcher); rows and column
-// chunks outside the matrix are clamped by the loaders, the descriptor's own range check is left wide open.
-template <typename T>
-__device__ __forceinline__ void copy_to_lds(const char* base, int voff, T* lds) {
-#if defined(__HIP_DEVICE_COMPILE__)        // the descriptor type exists in the device pass only
-  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, 0x7fffffff, 0x00020000);
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, HEXMI_LDS(lds), 16, voff, 0, 0, 0);
-#endif
-}
+// Copies are copy_to_lds() buffer loads: rows and column chunks outside the matrix are clamped by the loaders,
+// per-lane offsets stay below 2^31 (checked by the launcher).
 
 template <typename T, int ROWS>
 struct KMajorLoader2 {

@@ -115,6 +115,19 @@ inline int launch_status() {
   return hipGetLastError() == hipSuccess ? HEXMI_OK : HEXMI_ELAUNCH;
 }
 
+// 16 bytes per lane, global -> LDS, as a buffer load: the address is a uniform base (a buffer descriptor in scalar
+// registers, built by scalar arithmetic) plus a per-lane 32-bit byte offset, and the LDS destination (lds + lane*16
+// bytes) is a scalar, so a copy costs no vector arithmetic. voff must stay below 2^31; the descriptor's own range
+// check is left wide open, callers clamp what must not be read.
+template <typename T>
+__device__ __forceinline__ void copy_to_lds(const char* base, int voff, T* lds) {
+#if defined(__HIP_DEVICE_COMPILE__)        // the descriptor type exists in the device pass only
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, 0x7fffffff, 0x00020000);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(lds), 16, voff, 0, 0, 0);
+#endif
+}
+
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 inline int dtype_size(int dtype) {
