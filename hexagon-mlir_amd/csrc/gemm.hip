@@ -680,6 +680,39 @@ void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __r
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));       // drain the trailing copies before the workgroup's LDS goes away
 
   // acc[i][j][r]: row lane%16 of tile row i, column 4*(lane/16) + r of tile column j
+  if constexpr (sizeof(OutT) == 2) {
+    if (ldc % 8 == 0) {
+      // 16-bit results go through LDS so that a store instruction writes whole rows of the wave's tile (TN*32
+      // contiguous bytes per row) instead of 8-byte pieces of 16 rows. Each wave stages its tile in one of the four
+      // operand stages (same size or larger); chunks are XOR-swizzled so both the 8-byte writes and the 16-byte
+      // reads spread over the banks.
+      __syncthreads();                                // every wave has finished reading fragments
+      OutT* cs = reinterpret_cast<OutT*>(wave == 0 ? a_p0 : wave == 1 ? a_p1 : wave == 2 ? b_p0 : b_p1);
+      constexpr int CP = TN * 2;                      // 16-byte chunks per row of the wave's tile
+      constexpr int PITCH = TN * 16;                  // elements
+      static_assert(TM * 16 * PITCH <= BM * BK2 && TM * 16 * PITCH <= BN * BK2, "a wave's tile fits one stage");
+      auto swz = [](int row) { return CP == 16 ? (row & 15) : ((row >> 1) & 7); };
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row = i * 16 + lane % 16;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int col = j * 16 + 4 * (lane / 16);
+          store4<OutT>(cs + row * PITCH + (((col / kChunk) ^ swz(row)) * kChunk) + col % kChunk, acc[i][j][0],
+                       acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+        }
+      }
+      constexpr int RPI = 64 / CP;                    // rows per store instruction
+#pragma unroll
+      for (int r0 = 0; r0 < TM * 16; r0 += RPI) {
+        const int row = r0 + lane / CP, c = lane % CP;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(cs + row * PITCH + ((c ^ swz(row)) * kChunk));
+        const int grow = m0 + wm * TM * 16 + row, gcol = n0 + wn * TN * 16 + c * kChunk;
+        if (grow < M && gcol < N) *reinterpret_cast<u32x4*>(C + (int64_t)grow * ldc + gcol) = v;
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int row = m0 + (wm * TM + i) * 16 + lane % 16;
