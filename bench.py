@@ -147,7 +147,7 @@ class LayerNorm(Norms):
 
 
 class Gemm(Workload):
-    bound, kernel = "mfma", "gemm_kernel"
+    bound, kernel = "mfma", "gemm_kernel_k64"
 
     def __init__(self, size, dtype_name):
         self.size, self.dtype = size, dtype_name

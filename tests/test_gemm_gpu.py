@@ -43,6 +43,8 @@ SHAPES = [
     (1024, 512, 64),      # test_matmul.py:26-28
     (256, 256, 64), (512, 768, 128), (256, 512, 192),
     (100, 72, 64), (300, 264, 128),          # ragged M / N on the tiled path
+    (256, 256, 96), (300, 264, 160),         # K % 64 == 32: the four-stage 32-wide-slab kernel
+    (384, 256, 320),                         # odd number of 64-wide slabs
     (33, 17, 40), (1, 8, 8), (65, 130, 24), (7, 5, 3),   # generic path
 ]
 
@@ -82,6 +84,42 @@ def test_gemm_closed_forms(hexmi):
     c1 = hexmi.matmul(a.cuda(), b.cuda(), out_dtype=torch.float32).cpu()
     c2 = hexmi.matmul(a.cuda(), b.t().contiguous().cuda(), out_dtype=torch.float32, trans_b=True).cpu()
     assert torch.equal(c1, c2)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gemm_large_ragged_tiles(hexmi, dtype, trans_b):
+    # enough 256x256 tiles for the large-tile kernel, ragged in M and N, odd slab count; checked on sampled rows
+    # against a float64 product of the same rounded inputs
+    M, N, K = 2900, 2904, 192
+    a, b = _inputs(M, N, K, dtype, trans_b, seed=11)
+    got = hexmi.matmul(a.cuda(), b.cuda(), out_dtype=torch.float32, trans_b=trans_b).cpu()
+    rows = torch.cat([torch.arange(0, M, 37), torch.arange(M - 50, M)])
+    bb = b.double().t() if trans_b else b.double()
+    want = a[rows].double() @ bb
+    mag = a[rows].double().abs() @ bb.abs()
+    assert ((got[rows].double() - want).abs() <= 1e-5 * mag + 1e-30).all()
+    got16 = hexmi.matmul(a.cuda(), b.cuda(), trans_b=trans_b).cpu()
+    assert torch.equal(got16, got.to(dtype))          # the 16-bit result is the rounded fp32 result, staged or not
+
+
+def test_gemm_strided_operands(hexmi):
+    # leading dimensions larger than the rows (C ABI only): same arithmetic as the dense call, bit for bit; ldc % 8 != 0
+    # takes the direct (unstaged) 16-bit stores
+    from hexmi import _lib
+    L = _lib.lib()
+    M, N, K = 300, 264, 128
+    lda, ldb, ldc = K + 8, N + 16, N + 4
+    g = _gen(12)
+    a_big = (2 * torch.rand(M, lda, generator=g) - 1).half().cuda()
+    b_big = (2 * torch.rand(K, ldb, generator=g) - 1).half().cuda()
+    c_big = torch.full((M, ldc), 7.0, dtype=torch.float16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    rc = L.hexmi_gemm(M, N, K, a_big.data_ptr(), lda, b_big.data_ptr(), ldb, c_big.data_ptr(), ldc, 1, 1, 0, st)
+    assert rc == 0
+    dense = hexmi.matmul(a_big[:, :K].contiguous(), b_big[:, :N].contiguous())
+    assert torch.equal(c_big[:, :N], dense)
+    assert (c_big[:, N:] == 7.0).all()                # nothing written past the N columns
 
 
 def test_hexkl_entry_point(hexmi, oracle):
