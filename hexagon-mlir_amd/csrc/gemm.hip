@@ -496,6 +496,46 @@ __device__ __forceinline__ typename Mfma<T>::Frag read_nmajor2(const T* lds, int
   return u.f;
 }
 
+// Weight-only quantised B: int8 [N,K] rows, 64 bytes per row and slab (four 16-byte chunks, 16 rows per copy),
+// kept as int8 in LDS and widened to fp16 in registers, one fragment (8 values of one row) at a time.
+__device__ __forceinline__ int swz_k8(int row) { return (row >> 2) & 3; }      // row pitch 64 B
+template <int ROWS>
+struct I8RowLoader2 {
+  static constexpr int NI = ROWS / 64;              // 16 rows per wave-wide copy, four waves
+  int voff[NI];
+  int lds_off[NI];
+  __device__ __forceinline__ void init(int64_t ld, int row0, int row_max, int wave, int lane) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int inst = j * 4 + wave;
+      const int row = inst * 16 + lane / 4;
+      const int c = (lane % 4) ^ swz_k8(row);
+      int grow = row0 + row;
+      grow = grow < row_max ? grow : row_max;
+      voff[j] = (int)((int64_t)(grow - row0) * ld + c * 16);
+      lds_off[j] = inst * 16 * (BK2 / 4);           // 32-bit words
+    }
+  }
+  // The LDS stage is declared as 32-bit words, not bytes: accesses through a character type may alias anything, and
+  // the compiler then holds every fragment read until all copies in flight have landed.
+  __device__ __forceinline__ void issue(int j, uint32_t* lds, const char* base) const {   // j: an unrolled constant
+    if (j < NI) copy_to_lds(base, voff[j], lds + lds_off[j]);
+  }
+};
+// One 16-byte read per lane and slab: lane (row lane%16, K group g = lane/16) takes bytes [16g, 16g+16) of its row,
+// the first 8 for step 0 and the last 8 for step 1; the K slots of an MFMA may be assigned freely as long as A
+// uses the same assignment (k = 16g + 8*step + 0..7). (An 8-byte read per step would do, but the compiler then
+// holds every such read until all copies in flight have landed.)
+__device__ __forceinline__ u32x4 read_i8row(const uint32_t* lds, int row, int kgroup) {
+  return *reinterpret_cast<const u32x4*>(lds + row * (BK2 / 4) + ((kgroup ^ swz_k8(row)) * 4));
+}
+__device__ __forceinline__ f16x8 widen_i8(u32x2 raw) {
+  union { uint32_t u[4]; f16x8 f; } r;
+  cvt4(raw[0], r.u[0], r.u[1]);
+  cvt4(raw[1], r.u[2], r.u[3]);
+  return r.f;
+}
+
 // The accumulator is tied to the destination in inline assembly: left to the compiler, the 16x16x32 builtin gets
 // a destination register of its own and a copy back per instruction. Each accumulator is touched once per 64
 // MFMAs, far beyond the instruction's latency, and the epilogue reads them after the copy drain and its address
@@ -518,18 +558,31 @@ template <> struct Mfma16<bf16> {
 // each step is two phases of TM/2 * TN MFMAs. Fragments of the next step are read while the current one
 // multiplies. The copies of slab j+1 are issued in phase 3 of slab j-1 (A) and phase 0 of slab j (B), into the
 // stage slab j-1 was read from; the one barrier, between phases 2 and 3, comes after every wave's last read of
-// slab j and after all of slab j+1 has landed. TAIL: the slab count is odd.
-template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL>
+// slab j and after all of slab j+1 has landed. NS = 4 stages (small tiles, whose slabs are too short to cover the
+// memory latency with one slab of lead) fill the stage of slab j with slab j+4 instead. TAIL: the slab count is not
+// a multiple of NS.
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false, int NS = 2>
 __global__ __launch_bounds__(256)
-void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __restrict__ C, int M, int N, int K,
-                     int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n) {
+void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __restrict__ C, int M, int N, int K,
+                     int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
+                     const f16* __restrict__ scales = nullptr) {
+  static_assert(!B_I8 || (TRANS_B && sizeof(T) == 2), "int8 B is [N,K] and multiplies fp16 A");
+  const T* B = static_cast<const T*>(Bv);
   typedef typename Mfma<T>::Frag Frag;
   constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
   constexpr int TM = 2 * WM, TN = 2 * WN;           // 16x16 tiles per wave
+  static_assert(NS == 2 || NS == 4, "two stages, or four for small tiles");
   __shared__ __attribute__((aligned(16))) T a_p0[BM * BK2];
   __shared__ __attribute__((aligned(16))) T a_p1[BM * BK2];
-  __shared__ __attribute__((aligned(16))) T b_p0[BN * BK2];
-  __shared__ __attribute__((aligned(16))) T b_p1[BN * BK2];
+  __shared__ __attribute__((aligned(16))) T a_p2[NS == 4 ? BM * BK2 : 8];
+  __shared__ __attribute__((aligned(16))) T a_p3[NS == 4 ? BM * BK2 : 8];
+  // int8 B keeps its own element type end to end (copies and reads must name the same LDS objects for the
+  // compiler to tell the stage being filled from the stage being read); same bytes, so a wave's result tile fits
+  typedef typename std::conditional<B_I8, uint32_t, T>::type BT;
+  __shared__ __attribute__((aligned(16))) BT b_p0[BN * BK2 / (B_I8 ? 2 : 1)];
+  __shared__ __attribute__((aligned(16))) BT b_p1[BN * BK2 / (B_I8 ? 2 : 1)];
+  __shared__ __attribute__((aligned(16))) BT b_p2[NS == 4 ? BN * BK2 / (B_I8 ? 2 : 1) : 8];
+  __shared__ __attribute__((aligned(16))) BT b_p3[NS == 4 ? BN * BK2 / (B_I8 ? 2 : 1) : 8];
 
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // scalar: LDS destinations stay scalar
@@ -550,30 +603,40 @@ void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __r
   load_a.init(lda, m0, M - 1, wave, lane);
   KMajorLoader2<T, BN> load_bk;
   NMajorLoader2<T, BN> load_bn;
-  if constexpr (TRANS_B) load_bk.init(ldb, n0, N - 1, wave, lane);
+  I8RowLoader2<BN> load_b8;
+  if constexpr (B_I8) load_b8.init(ldb, n0, N - 1, wave, lane);
+  else if constexpr (TRANS_B) load_bk.init(ldb, n0, N - 1, wave, lane);
   else load_bn.init(ldb, n0, N - kChunk, wave, lane);     // N % 8 == 0, so n0 <= N - 8
   // uniform bases of this tile's operand panels; slab j adds j * (bytes per 64 elements of K)
   const char* a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda);
-  const char* b_base = reinterpret_cast<const char*>(TRANS_B ? B + (int64_t)n0 * ldb : B + n0);
+  const char* b_base = B_I8 ? static_cast<const char*>(Bv) + (int64_t)n0 * ldb
+                            : reinterpret_cast<const char*>(TRANS_B ? B + (int64_t)n0 * ldb : B + n0);
   const int64_t a_step = BK2 * (int64_t)sizeof(T);
-  const int64_t b_step = (TRANS_B ? BK2 : BK2 * ldb) * (int64_t)sizeof(T);
-  constexpr int NLA = BM / 32, NLB = BN / 32;
+  const int64_t b_step = B_I8 ? BK2 : (TRANS_B ? BK2 : BK2 * ldb) * (int64_t)sizeof(T);
+  constexpr int NLA = BM / 32, NLB = B_I8 ? BN / 64 : BN / 32;
 
   static_assert(TM == TN && TN >= 4, "a round carries two fragment reads: 2*TM rounds read TM+TN fragments twice");
   auto copy_a = [&](int i, const char* base, T* dst) __attribute__((always_inline)) {
     load_a.issue(i, dst, base);
   };
-  auto copy_b = [&](int i, const char* base, T* dst) __attribute__((always_inline)) {
-    if constexpr (TRANS_B) load_bk.issue(i, dst, base);
+  auto copy_b = [&](int i, const char* base, BT* dst) __attribute__((always_inline)) {
+    if constexpr (B_I8) load_b8.issue(i, dst, base);
+    else if constexpr (TRANS_B) load_bk.issue(i, dst, base);
     else load_bn.issue(i, dst, base);
   };
   // fragments of step ks (32 elements of K): lane holds row/column lane%16 of a tile, K group lane/16 (8 elements)
   auto read_a = [&](const T* src, int ks, int i) __attribute__((always_inline)) {
-    return read_kmajor2<T>(src, (wm * TM + i) * 16 + lane % 16, ks * 4 + lane / 16);
+    // int8 B fixes the K slots of a step as k = 16*(lane/16) + 8*step + 0..7 (see read_i8row)
+    return read_kmajor2<T>(src, (wm * TM + i) * 16 + lane % 16, B_I8 ? 2 * (lane / 16) + ks : ks * 4 + lane / 16);
   };
-  auto read_b = [&](const T* src, int ks, int j) __attribute__((always_inline)) {
-    if constexpr (TRANS_B) return read_kmajor2<T>(src, (wn * TN + j) * 16 + lane % 16, ks * 4 + lane / 16);
+  auto read_b = [&](const BT* src, int ks, int j) __attribute__((always_inline)) {
+    if constexpr (B_I8) return Frag{};              // int8 B is read raw (read_b8) and widened later
+    else if constexpr (TRANS_B) return read_kmajor2<T>(src, (wn * TN + j) * 16 + lane % 16, ks * 4 + lane / 16);
     else return read_nmajor2<T, BN>(src, (wn * TN + j) * 16, ks, lane);
+  };
+  auto read_b8 = [&](const BT* src, int j) __attribute__((always_inline)) {
+    if constexpr (B_I8) return read_i8row(src, (wn * TN + j) * 16 + lane % 16, lane / 16);
+    else return u32x4{};
   };
   auto mfma_row = [&](const Frag* af, const Frag* bf, int i) __attribute__((always_inline)) {
 #pragma unroll
@@ -584,7 +647,7 @@ void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __r
 
   // Copy n of a slab: the NLA copies of A, then the NLB of B.
   constexpr int NL = NLA + NLB;
-  auto copy_n = [&](int n, int slab, T* a_dst, T* b_dst) __attribute__((always_inline)) {
+  auto copy_n = [&](int n, int slab, T* a_dst, BT* b_dst) __attribute__((always_inline)) {
     if constexpr (TRANS_B) {
       if (n < NLA) copy_a(n, a_base + slab * a_step, a_dst);
       else copy_b(n - NLA, b_base + slab * b_step, b_dst);
@@ -594,9 +657,20 @@ void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __r
     }
   };
   // Fragment n of a step: the TN of B (every MFMA row needs all of them), then the TM of A in row order.
-  auto read_n = [&](int n, const T* a_src, const T* b_src, int ks, Frag* af_dst, Frag* bf_dst) __attribute__((always_inline)) {
-    if (n < TN) bf_dst[n] = read_b(b_src, ks, n);
-    else af_dst[n - TN] = read_a(a_src, ks, n - TN);
+  u32x4 braw[TN];                                   // int8 B: both steps of a slab as read, before widening
+  auto widen_b = [&](int ks, int j, Frag* bf_dst) __attribute__((always_inline)) {
+    if constexpr (B_I8) bf_dst[j] = widen_i8(u32x2{braw[j][2 * ks], braw[j][2 * ks + 1]});
+  };
+  auto read_n = [&](int n, const T* a_src, const BT* b_src, int ks, Frag* af_dst, Frag* bf_dst) __attribute__((always_inline)) {
+    if (n < TN) {
+      if constexpr (B_I8) {
+        if (ks == 0) braw[n] = read_b8(b_src, n);   // once per slab, with the reads of its step 0
+      } else {
+        bf_dst[n] = read_b(b_src, ks, n);
+      }
+    } else {
+      af_dst[n - TN] = read_a(a_src, ks, n - TN);
+    }
   };
 
   Frag af[2][TM], bf[2][TN];
@@ -609,7 +683,7 @@ void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __r
   auto copies_before = [](int w) constexpr {
     int sum = 0;
     for (int r = 0; r < w; ++r) {
-      if (TRANS_B) sum += r < TM ? 2 : 0;
+      if (TRANS_B) sum += 2 * r + 2 <= NL ? 2 : (2 * r < NL ? 1 : 0);
       else sum += r < TM / 2 ? 2 : (r < TM + TM / 2 ? 1 : 0);
     }
     return sum;
@@ -618,27 +692,39 @@ void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __r
   static_assert(copies_before(2 * TM) == NL, "the window carries all of a slab's copies");
 #pragma unroll
   for (int n = 0; n < NL; ++n) copy_n(n, 0, a_p0, b_p0);
+  if constexpr (NS == 4) {
 #pragma unroll
-  for (int n = 0; n < NL - LATE; ++n) copy_n(n, clampj(1), a_p1, b_p1);
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm(NL - LATE));             // slab 0 landed
+    for (int n = 0; n < NL; ++n) copy_n(n, clampj(1), a_p1, b_p1);
+#pragma unroll
+    for (int n = 0; n < NL; ++n) copy_n(n, clampj(2), a_p2, b_p2);
+#pragma unroll
+    for (int n = 0; n < NL - LATE; ++n) copy_n(n, clampj(3), a_p3, b_p3);
+  } else {
+#pragma unroll
+    for (int n = 0; n < NL - LATE; ++n) copy_n(n, clampj(1), a_p1, b_p1);
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 1) * NL - LATE));  // slab 0 landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int n = 0; n < TM + TN; ++n) read_n(n, a_p0, b_p0, 0, af[0], bf[0]);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) widen_b(0, j, bf[0]);
 
   // The MFMAs are inline assembly, which the scheduler's group directives do not see, so the issue order is the
   // source order, pinned by full scheduling fences. A slab is 2*TM rounds of TN MFMAs (one row of tiles); a round
   // carries two fragment reads and up to two copies, one after every other MFMA. The barrier sits in the middle:
   // by then every wave has read both steps of this slab, and all of the next slab has landed.
 #define HEXMI_FENCE __builtin_amdgcn_sched_barrier(0)
-  auto slab = [&](T* acur, T* bcur, T* anxt, T* bnxt, int j) __attribute__((always_inline)) {
+  // cur / nxt / prv: the stages of slabs j, j+1 and j-1 (= j+NS-1; with two stages prv is nxt).
+  auto slab = [&](T* acur, BT* bcur, T* anxt, BT* bnxt, T* aprv, BT* bprv, int j) __attribute__((always_inline)) {
     const bool live = !TAIL || j < KT;
-    const int j1 = clampj(j + 1), j2 = clampj(j + 2);
+    const int j1 = clampj(j + NS - 1), j2 = clampj(j + NS);
 #pragma unroll
     for (int q = 0; q < 2 * TM; ++q) {
       const int ks = q / TM, row = q % TM;
       if (q == TM) {
         HEXMI_FENCE;
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * NL));    // all but slabs j+2 .. j+NS-1 have landed
         __builtin_amdgcn_s_barrier();
         HEXMI_FENCE;
       }
@@ -655,31 +741,58 @@ void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __r
           const int n = row * 2 + jj;
           if (ks == 0) read_n(n, acur, bcur, 1, af[1], bf[1]);
           else read_n(n, anxt, bnxt, 0, af[0], bf[0]);
+          if constexpr (B_I8) {
+            // widen two B fragments per round: step 1 of this slab during its first half (read long ago), step 0
+            // of the next slab during the second half, one (small tile) or two rounds after its read
+            constexpr int FIRST = TN >= 8 ? 2 : 1;
+            const int m = ks == 0 ? 2 * row + jj : 2 * (row - FIRST) + jj;
+            if (m >= 0 && m < TN) widen_b(1 - ks, m, bf[1 - ks]);
+          }
         }
         constexpr int CSLOT = (TN >= 8 && !TRANS_B) ? 2 : 0;   // first of the two copy slots of a round
         if (jj >= CSLOT && jj < CSLOT + 2) {
-          // copies of the window that opened at this slab's barrier (rounds TM..2TM-1, slab j+2 into this slab's
-          // stage) and of the window that opened at the previous one (rounds 0.., slab j+1 into the other stage)
+          // copies of the window that opened at this slab's barrier (rounds TM..2TM-1, slab j+NS into this slab's
+          // stage) and of the window that opened at the previous one (rounds 0.., slab j+NS-1 into the stage of j-1)
           const int c = jj - CSLOT;
           const int w = (q + TM) % (2 * TM);               // round index within its window
           const int lo = copies_before(w), hi = copies_before(w + 1);
           if (lo + c < hi) {
             if (ks == 1) copy_n(lo + c, j2, acur, bcur);
-            else copy_n(lo + c, j1, anxt, bnxt);
+            else copy_n(lo + c, j1, aprv, bprv);
           }
         }
         HEXMI_FENCE;
       }
     }
   };
-  for (int j = 0; j < KT; j += 2) {
-    slab(a_p0, b_p0, a_p1, b_p1, j);
-    slab(a_p1, b_p1, a_p0, b_p0, j + 1);
+  for (int j = 0; j < KT; j += NS) {
+    if constexpr (NS == 2) {
+      slab(a_p0, b_p0, a_p1, b_p1, a_p1, b_p1, j);
+      slab(a_p1, b_p1, a_p0, b_p0, a_p0, b_p0, j + 1);
+    } else {
+      slab(a_p0, b_p0, a_p1, b_p1, a_p3, b_p3, j);
+      slab(a_p1, b_p1, a_p2, b_p2, a_p0, b_p0, j + 1);
+      slab(a_p2, b_p2, a_p3, b_p3, a_p1, b_p1, j + 2);
+      slab(a_p3, b_p3, a_p0, b_p0, a_p2, b_p2, j + 3);
+    }
   }
 #undef HEXMI_FENCE
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));       // drain the trailing copies before the workgroup's LDS goes away
 
   // acc[i][j][r]: row lane%16 of tile row i, column 4*(lane/16) + r of tile column j
+  if constexpr (B_I8) {
+    // per-output-channel scales multiply the finished sums
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int col = n0 + (wn * TN + j) * 16 + 4 * (lane / 16);
+      col = col < N - 4 ? col : N - 4;              // past the edge: any valid run, those columns are not stored
+      const f16x4 sc = *reinterpret_cast<const f16x4*>(scales + col);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[i][j][r] *= (float)sc[r];
+    }
+  }
   if constexpr (sizeof(OutT) == 2) {
     if (ldc % 8 == 0) {
       // 16-bit results go through LDS so that a store instruction writes whole rows of the wave's tile (TN*32
@@ -687,7 +800,8 @@ void gemm_kernel_k64(const T* __restrict__ A, const T* __restrict__ B, OutT* __r
       // operand stages (same size or larger); chunks are XOR-swizzled so both the 8-byte writes and the 16-byte
       // reads spread over the banks.
       __syncthreads();                                // every wave has finished reading fragments
-      OutT* cs = reinterpret_cast<OutT*>(wave == 0 ? a_p0 : wave == 1 ? a_p1 : wave == 2 ? b_p0 : b_p1);
+      OutT* cs = wave == 0 ? reinterpret_cast<OutT*>(a_p0) : wave == 1 ? reinterpret_cast<OutT*>(a_p1)
+                 : wave == 2 ? reinterpret_cast<OutT*>(b_p0) : reinterpret_cast<OutT*>(b_p1);
       constexpr int CP = TN * 2;                      // 16-byte chunks per row of the wave's tile
       constexpr int PITCH = TN * 16;                  // elements
       static_assert(TM * 16 * PITCH <= BM * BK2 && TM * 16 * PITCH <= BN * BK2, "a wave's tile fits one stage");
@@ -849,12 +963,13 @@ int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t 
   // K % 64 == 0: the paired-slab kernel; its per-lane copy offsets (up to 256 rows, or 64 rows of K) must stay
   // below 2^31 bytes
   if (NWN == 2 && K % BK2 == 0 && lda < (1 << 21) && ldb < (1 << 21)) {
-    if ((K / BK2) % 2 == 0)
-      hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, false>), dim3(tiles_m * tiles_n), dim3(256), 0, s,
-                         A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+    constexpr int NS = WM <= 2 ? 4 : 2;            // small tiles: four stages (their slabs are short)
+    if ((K / BK2) % NS == 0)
+      hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, false, false, NS>), dim3(tiles_m * tiles_n),
+                         dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n, nullptr);
     else
-      hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, true>), dim3(tiles_m * tiles_n), dim3(256), 0, s,
-                         A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
+      hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, true, false, NS>), dim3(tiles_m * tiles_n),
+                         dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n, nullptr);
     return launch_status();
   }
   if ((K / BK) % 4 == 0)
@@ -900,6 +1015,18 @@ int launch_w8a16(const f16* A, const int8_t* W, const f16* scales, f16* C, int64
                  hipStream_t s) {
   constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+  if (K % BK2 == 0 && K < (1 << 21)) {
+    constexpr int NS = WM <= 2 ? 4 : 2;
+    if ((K / BK2) % NS == 0)
+      hipLaunchKernelGGL((gemm_kernel_k64<f16, f16, WM, WN, true, false, true, NS>), dim3(tiles_m * tiles_n),
+                         dim3(256), 0, s, A, static_cast<const void*>(W), C, (int)M, (int)N, (int)K, K, K, N, tiles_m,
+                         tiles_n, scales);
+    else
+      hipLaunchKernelGGL((gemm_kernel_k64<f16, f16, WM, WN, true, true, true, NS>), dim3(tiles_m * tiles_n),
+                         dim3(256), 0, s, A, static_cast<const void*>(W), C, (int)M, (int)N, (int)K, K, K, N, tiles_m,
+                         tiles_n, scales);
+    return launch_status();
+  }
   if ((K / BK) % 4 == 0)
     hipLaunchKernelGGL((gemm_kernel<f16, f16, WM, WN, true, false, true>), dim3(tiles_m * tiles_n), dim3(256), 0, s, A,
                        static_cast<const void*>(W), C, (int)M, (int)N, (int)K, K, K, N, tiles_m, tiles_n, scales);
