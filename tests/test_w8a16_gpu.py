@@ -95,6 +95,18 @@ def test_w8a16_config_sizes(hexmi, oracle, M):
     assert torch.equal(got_p, got[:, perm])
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 520, 192), (130, 264, 320), (2900, 2904, 128), (2100, 4104, 192)])
+def test_w8a16_many_rows(hexmi, M, N, K):
+    # the tiled kernels (128x128 tiles with four stages, 256x256 with two; odd and even slab counts, ragged edges),
+    # checked on sampled rows against a float64 product of the exactly dequantised weights
+    a, w, s = _inputs(M, N, K, seed=8)
+    got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
+    rows = torch.cat([torch.arange(0, M, 41), torch.arange(M - 20, M)])
+    want = (a[rows].double() @ w.double().t()) * s.double()[None, :]
+    assert close16(got[rows], want.half(), max_ulp=1, atol=2e-4)
+    assert (got[rows].double() - want).abs().max() / math.sqrt(K) <= 2e-2
+
+
 def test_w8a16_errors(hexmi):
     a = torch.zeros(2, 64, dtype=torch.float16)
     with pytest.raises(TypeError):
