@@ -1,7 +1,7 @@
 // Flash-attention forward: O = softmax(scale * Q K^T [+ causal mask]) V, [Z,H,S,D] contiguous.
 //
 // Matrix-core kernel (fp16 / bf16, D = 64 or 128): a workgroup of 4 waves owns 128 query rows (32 per wave) and
-// walks the keys in blocks of 64. K and V blocks are copied global -> LDS with global_load_lds_dwordx4, double
+// walks the keys in blocks of 64. K and V blocks are copied global -> LDS with buffer loads (copy_to_lds), double
 // buffered. Per key block and wave:
 //   S^T = K Q^T  with v_mfma_f32_32x32x16 (K fragment first): a lane then holds 32 scores of ONE query row
 //                (row = lane%32), so row max / row sum are in-lane reductions plus one exchange with lane^32;
