@@ -146,3 +146,15 @@ def test_w8a16_packed_equals_unpacked(hexmi, oracle, M, N, K):
         assert torch.equal(got, ref)                          # same kernel, same arithmetic: bit for bit
     with pytest.raises(ValueError):
         hexmi.w8a16_matmul_packed(a.cuda(), wp[:-16], s.cuda())
+
+
+def test_packed_weights_through_a_tensor_file(hexmi, tmp_path):
+    # pre-packed weights kept in the reference's raw tensor format (test/utils/dsp/include/tensor.h:235-260)
+    a, w, s = _inputs(8, 1000, 2048, seed=7)
+    wp = hexmi.pack_w8(w.cuda())
+    path = str(tmp_path / "wp.bin")
+    hexmi.save_tensor(path, wp)
+    back = hexmi.load_tensor(path)
+    assert back.dtype == torch.int8 and torch.equal(back, wp.cpu())
+    got = hexmi.w8a16_matmul_packed(a.cuda(), back.cuda(), s.cuda()).cpu()
+    assert torch.equal(got, hexmi.w8a16_matmul_packed(a.cuda(), wp, s.cuda()).cpu())
