@@ -429,6 +429,10 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
   const int n0 = (blockIdx.x * 4 + wave) * RPW;
   if (n0 >= N) return;
 
+  // the channel scales first: they come from HBM and would otherwise be waited for after everything else
+  f16 sc[RPW];
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) sc[r] = scales[n0 + r < N ? n0 + r : N - 1];
   u32x4 wv[RPW][KJ];
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
@@ -472,7 +476,7 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
       const float tot = wave_sum(acc[m]);
-      if (lane == 0 && n < N && m < M) C[(int64_t)m * N + n] = (f16)(tot * (float)scales[n]);
+      if (lane == 0 && n < N && m < M) C[(int64_t)m * N + n] = (f16)(tot * (float)sc[r]);
     }
   }
 }
