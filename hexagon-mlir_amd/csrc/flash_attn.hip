@@ -261,6 +261,9 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
 
   auto process = [&](int step, const T* k_src, const T* v_src) __attribute__((always_inline)) {
     const int n0 = step * kBlockN;
+    // causal: a key block wholly past this wave's 32 rows contributes nothing (wave-uniform; the workgroup's
+    // barriers and copies are outside)
+    if (CAUSAL && n0 > q0 + 31) return;
     // mask values of this lane's 32 scores: four runs of four consecutive keys per 32-key tile
     typedef T MaskRun __attribute__((ext_vector_type(4)));
     MaskRun mk[2][4];
