@@ -140,209 +140,221 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   constexpr int kBlockM = NW * 32;                  // query rows per workgroup
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int nqb = (S + kBlockM - 1) / kBlockM;
-  // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each). Give every XCD whole heads and let it walk
-  // them one after the other, longest query blocks first, so the K/V of the head in progress stays in its L2.
-  int zh, qb;
-  if (ZH % 8 == 0) {
-    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
-    zh = xcd + 8 * (slot / nqb);
-    qb = nqb - 1 - slot % nqb;
-  } else {
-    zh = blockIdx.x % ZH;
-    qb = nqb - 1 - blockIdx.x / ZH;
-  }
-  const int64_t base = (int64_t)zh * S * D;
-  const int64_t kv_base = (int64_t)zh * Skv * D;
-  const T* q_g = Q + base;
-  const T* k_g = K + kv_base;
-  const T* v_g = V + kv_base;
-
-  const int q0 = qb * kBlockM + wave * 32;           // first query row of this wave
-  const int qrow = q0 + lane % 32;                    // the query row this lane's scores belong to
-  const int half = lane / 32;
-
-  // Q fragments stay in registers: lane = (row lane%32, d = ds*16 + half*8 .. +8)
-  Frag qf[DS];
-  {
-    const int qr = qrow < S ? qrow : S - 1;
-#pragma unroll
-    for (int ds = 0; ds < DS; ++ds)
-      qf[ds] = *reinterpret_cast<const Frag*>(q_g + (int64_t)qr * D + ds * 16 + half * 8);
-  }
-
-  f32x16 o_acc[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.0f;
-  float m_i = -INFINITY;                              // running max (already multiplied by scale*log2e)
-  float l_i = 0.0f;                                   // this lane's share of the running sum
-
-  const int key_end = CAUSAL ? ((qb + 1) * kBlockM < S ? (qb + 1) * kBlockM : S) : Skv;
-  const int n_steps = (key_end + kBlockN - 1) / kBlockN;
-
-  KvTileLoader<T, D, false, NW> k_loader;
-  KvTileLoader<T, D, true, NW> v_loader;
-  k_loader.init(wave, lane);
-  v_loader.init(wave, lane);
-  auto load_kv = [&](int step, T* k_dst, T* v_dst) __attribute__((always_inline)) {
-    k_loader.issue(k_g, step * kBlockN, Skv, k_dst);
-    v_loader.issue(v_g, step * kBlockN, Skv, v_dst);
-  };
-
-  // One 32-key tile of the online softmax: mask, row max, (rare) rescale, exponentials, row sum; leaves the
-  // probabilities as the two MFMA operands pf[0], pf[1] (score registers 0..7 and 8..15 of this lane).
-  // The reference maximum m_i may lag the true running maximum by up to kRescaleLag (log2 units): softmax is
-  // shift invariant, so exponentials up to 2^kRescaleLag are as exact as ones below 1, and the output
-  // accumulator and running sum only need rescaling when a row outgrows the lag. The decision is per row (lane);
-  // the wave-uniform ballot only skips the multiplications when no row of the wave needs them.
-  auto softmax_tile = [&](int key_base, bool need_mask, f32x16& s, Frag* pf) __attribute__((always_inline)) {
-    if (need_mask) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = key_base + 8 * (r / 4) + 4 * half + r % 4;
-        if ((CAUSAL && key > qrow) || key >= Skv) s[r] = -INFINITY;
-      }
+  // Persistent workgroups: the grid is at most what the chip holds at once, and a workgroup walks several (head,
+  // query block) units, which takes the per-unit launch cost and the idle tail out of short causal units.
+  // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): every XCD gets a list of whole heads, longest
+  // query blocks first, and its workgroups take the list in snake order (unit it*P + u, then it*P + P-1-u, ...),
+  // so a workgroup's long and short units alternate and the head in progress stays in the XCD's L2.
+  const int total = ZH * nqb;
+  const bool by_xcd = ZH % 8 == 0 && gridDim.x % 8 == 0;
+  const int P = by_xcd ? gridDim.x / 8 : gridDim.x;             // workgroups sharing one list
+  const int u = by_xcd ? blockIdx.x / 8 : blockIdx.x;
+  const int list_len = by_xcd ? total / 8 : total;
+  for (int it = 0; it * P < list_len; ++it) {
+    const int unit = it * P + ((it & 1) ? P - 1 - u : u);
+    if (unit >= list_len) continue;                             // workgroup-uniform
+    int zh, qb;
+    if (by_xcd) {
+      zh = blockIdx.x % 8 + 8 * (unit / nqb);
+      qb = nqb - 1 - unit % nqb;
+    } else {
+      zh = unit % ZH;
+      qb = nqb - 1 - unit / ZH;
     }
-    float mx = -INFINITY;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
-    mx = fmaxf(mx, other_half(mx));
-    const float m_blk = mx * scale_log2e;
-    const bool grow = m_blk > m_i + kRescaleLag;
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-      const float m_new = grow ? m_blk : m_i;
-      const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_new) : 1.0f;
-      l_i *= alpha;
-      m_i = m_new;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
-    }
-    float p[16];
-    float sum = 0.0f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, -m_i));
-      sum += p[r];
-    }
-    l_i += sum;
-    pf[0] = MfmaT<T>::pack(&p[0]);
-    pf[1] = MfmaT<T>::pack(&p[8]);
-  };
-  // O^T += V^T P^T for one 32-key tile. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
-  // which is score register hf*8 + e of this lane, so the packed probabilities are used as they are.
-  auto pv_tile = [&](const T* v_src, int jt, const Frag* pf) __attribute__((always_inline)) {
-    const int g = lane / 16, i16 = lane % 16;
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        union { i16x4 h[2]; Frag f; } vf;
-#pragma unroll
-        for (int pp = 0; pp < 2; ++pp) {
-          const int row = jt * 32 + hf * 16 + 8 * pp + 4 * (g >> 1) + (i16 >> 2);
-          const int col = dt * 32 + (g & 1) * 16 + (i16 & 3) * 4;
-          const int c = (col / 8) ^ swz_vtile<D>(row);
-          const T* addr = v_src + (row * CPR + c) * 8 + (col % 8);
-          vf.h[pp] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
-        }
-        o_acc[dt] = MfmaT<T>::run(vf.f, pf[hf], o_acc[dt]);
-      }
-    }
-  };
+    const int64_t base = (int64_t)zh * S * D;
+    const int64_t kv_base = (int64_t)zh * Skv * D;
+    const T* q_g = Q + base;
+    const T* k_g = K + kv_base;
+    const T* v_g = V + kv_base;
 
-  // mask row of this lane's query (GENERAL with a mask only)
-  const T* mask_row = nullptr;
-  if constexpr (GENERAL) {
-    if (Mk) mask_row = Mk + ((int64_t)zh * S + (qrow < S ? qrow : S - 1)) * Skv;
-  }
+    const int q0 = qb * kBlockM + wave * 32;           // first query row of this wave
+    const int qrow = q0 + lane % 32;                    // the query row this lane's scores belong to
+    const int half = lane / 32;
 
-  auto process = [&](int step, const T* k_src, const T* v_src) __attribute__((always_inline)) {
-    const int n0 = step * kBlockN;
-    // causal: a key block wholly past this wave's 32 rows contributes nothing (wave-uniform; the workgroup's
-    // barriers and copies are outside)
-    if (CAUSAL && n0 > q0 + 31) return;
-    // mask values of this lane's 32 scores: four runs of four consecutive keys per 32-key tile
-    typedef T MaskRun __attribute__((ext_vector_type(4)));
-    MaskRun mk[2][4];
-    if constexpr (GENERAL) {
-      if (mask_row) {
+    // Q fragments stay in registers: lane = (row lane%32, d = ds*16 + half*8 .. +8)
+    Frag qf[DS];
+    {
+      const int qr = qrow < S ? qrow : S - 1;
 #pragma unroll
-        for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-          for (int g4 = 0; g4 < 4; ++g4) {
-            int key = n0 + jt * 32 + 8 * g4 + 4 * half;
-            key = key + 4 <= Skv ? key : Skv - 4;          // past the end: any valid run, those scores are dropped
-            mk[jt][g4] = *reinterpret_cast<const MaskRun*>(mask_row + key);
-          }
-      }
+      for (int ds = 0; ds < DS; ++ds)
+        qf[ds] = *reinterpret_cast<const Frag*>(q_g + (int64_t)qr * D + ds * 16 + half * 8);
     }
-    // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4], one MFMA chain per 32-key tile
-    f32x16 s[2];
-#pragma unroll
-    for (int jt = 0; jt < 2; ++jt) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[jt][r] = 0.0f;
-      const int krow = jt * 32 + lane % 32;
-#pragma unroll
-      for (int ds = 0; ds < DS; ++ds) {
-        const int c = (ds * 2 + half) ^ swz_ktile<D>(krow);
-        Frag kf = *reinterpret_cast<const Frag*>(k_src + (krow * CPR + c) * 8);
-        s[jt] = MfmaT<T>::run(kf, qf[ds], s[jt]);
-      }
-    }
-    // The softmax of tile 0 runs on the vector ALUs while the matrix cores finish the scores of tile 1, and the
-    // softmax of tile 1 while they accumulate P V of tile 0.
-    if constexpr (GENERAL) {
-      if (mask_row) {
-        // softmax(scale*s + mask) = softmax(scale * (s + mask/scale)): fold the mask into the raw scores
-#pragma unroll
-        for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[jt][r] = fmaf(to_f32<T>(mk[jt][r / 4][r % 4]), mask_factor, s[jt][r]);
-      }
-    }
-    const bool need_mask = (CAUSAL && n0 + kBlockN - 1 > q0) || (n0 + kBlockN > Skv);
-    Frag pf[4];
-    softmax_tile(n0, need_mask, s[0], &pf[0]);
-    pv_tile(v_src, 0, &pf[0]);
-    softmax_tile(n0 + 32, need_mask, s[1], &pf[2]);
-    pv_tile(v_src, 1, &pf[2]);
-  };
 
-  load_kv(0, k_lds0, v_lds0);
-  int step = 0;
-  for (; step + 1 < n_steps; step += 2) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    load_kv(step + 1, k_lds1, v_lds1);
-    process(step, k_lds0, v_lds0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (step + 2 < n_steps) load_kv(step + 2, k_lds0, v_lds0);
-    process(step + 1, k_lds1, v_lds1);
-  }
-  if (step < n_steps) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    process(step, k_lds0, v_lds0);
-  }
-
-  // ---- epilogue: o_acc[dt][r] is O[qrow][dt*32 + 8*(r/4) + 4*half + r%4] * l
-  const float l_tot = l_i + other_half(l_i);
-  const float inv_l = 1.0f / l_tot;
-  if (qrow < S) {
-    OutT* o_row = O + base + (int64_t)qrow * D;
+    f32x16 o_acc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int d = dt * 32 + 8 * q4 + 4 * half;
-        store4o<OutT>(o_row + d, o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l,
-                      o_acc[dt][q4 * 4 + 2] * inv_l, o_acc[dt][q4 * 4 + 3] * inv_l);
+      for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.0f;
+    float m_i = -INFINITY;                              // running max (already multiplied by scale*log2e)
+    float l_i = 0.0f;                                   // this lane's share of the running sum
+
+    const int key_end = CAUSAL ? ((qb + 1) * kBlockM < S ? (qb + 1) * kBlockM : S) : Skv;
+    const int n_steps = (key_end + kBlockN - 1) / kBlockN;
+
+    KvTileLoader<T, D, false, NW> k_loader;
+    KvTileLoader<T, D, true, NW> v_loader;
+    k_loader.init(wave, lane);
+    v_loader.init(wave, lane);
+    auto load_kv = [&](int step, T* k_dst, T* v_dst) __attribute__((always_inline)) {
+      k_loader.issue(k_g, step * kBlockN, Skv, k_dst);
+      v_loader.issue(v_g, step * kBlockN, Skv, v_dst);
+    };
+
+    // One 32-key tile of the online softmax: mask, row max, (rare) rescale, exponentials, row sum; leaves the
+    // probabilities as the two MFMA operands pf[0], pf[1] (score registers 0..7 and 8..15 of this lane).
+    // The reference maximum m_i may lag the true running maximum by up to kRescaleLag (log2 units): softmax is
+    // shift invariant, so exponentials up to 2^kRescaleLag are as exact as ones below 1, and the output
+    // accumulator and running sum only need rescaling when a row outgrows the lag. The decision is per row (lane);
+    // the wave-uniform ballot only skips the multiplications when no row of the wave needs them.
+    auto softmax_tile = [&](int key_base, bool need_mask, f32x16& s, Frag* pf) __attribute__((always_inline)) {
+      if (need_mask) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key_base + 8 * (r / 4) + 4 * half + r % 4;
+          if ((CAUSAL && key > qrow) || key >= Skv) s[r] = -INFINITY;
+        }
       }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
+      mx = fmaxf(mx, other_half(mx));
+      const float m_blk = mx * scale_log2e;
+      const bool grow = m_blk > m_i + kRescaleLag;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        const float m_new = grow ? m_blk : m_i;
+        const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_new) : 1.0f;
+        l_i *= alpha;
+        m_i = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+      }
+      float p[16];
+      float sum = 0.0f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, -m_i));
+        sum += p[r];
+      }
+      l_i += sum;
+      pf[0] = MfmaT<T>::pack(&p[0]);
+      pf[1] = MfmaT<T>::pack(&p[8]);
+    };
+    // O^T += V^T P^T for one 32-key tile. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
+    // which is score register hf*8 + e of this lane, so the packed probabilities are used as they are.
+    auto pv_tile = [&](const T* v_src, int jt, const Frag* pf) __attribute__((always_inline)) {
+      const int g = lane / 16, i16 = lane % 16;
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          union { i16x4 h[2]; Frag f; } vf;
+#pragma unroll
+          for (int pp = 0; pp < 2; ++pp) {
+            const int row = jt * 32 + hf * 16 + 8 * pp + 4 * (g >> 1) + (i16 >> 2);
+            const int col = dt * 32 + (g & 1) * 16 + (i16 & 3) * 4;
+            const int c = (col / 8) ^ swz_vtile<D>(row);
+            const T* addr = v_src + (row * CPR + c) * 8 + (col % 8);
+            vf.h[pp] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
+          }
+          o_acc[dt] = MfmaT<T>::run(vf.f, pf[hf], o_acc[dt]);
+        }
+      }
+    };
+
+    // mask row of this lane's query (GENERAL with a mask only)
+    const T* mask_row = nullptr;
+    if constexpr (GENERAL) {
+      if (Mk) mask_row = Mk + ((int64_t)zh * S + (qrow < S ? qrow : S - 1)) * Skv;
+    }
+
+    auto process = [&](int step, const T* k_src, const T* v_src) __attribute__((always_inline)) {
+      const int n0 = step * kBlockN;
+      // causal: a key block wholly past this wave's 32 rows contributes nothing (wave-uniform; the workgroup's
+      // barriers and copies are outside)
+      if (CAUSAL && n0 > q0 + 31) return;
+      // mask values of this lane's 32 scores: four runs of four consecutive keys per 32-key tile
+      typedef T MaskRun __attribute__((ext_vector_type(4)));
+      MaskRun mk[2][4];
+      if constexpr (GENERAL) {
+        if (mask_row) {
+#pragma unroll
+          for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+              int key = n0 + jt * 32 + 8 * g4 + 4 * half;
+              key = key + 4 <= Skv ? key : Skv - 4;          // past the end: any valid run, those scores are dropped
+              mk[jt][g4] = *reinterpret_cast<const MaskRun*>(mask_row + key);
+            }
+        }
+      }
+      // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4], one MFMA chain per 32-key tile
+      f32x16 s[2];
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[jt][r] = 0.0f;
+        const int krow = jt * 32 + lane % 32;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+          const int c = (ds * 2 + half) ^ swz_ktile<D>(krow);
+          Frag kf = *reinterpret_cast<const Frag*>(k_src + (krow * CPR + c) * 8);
+          s[jt] = MfmaT<T>::run(kf, qf[ds], s[jt]);
+        }
+      }
+      // The softmax of tile 0 runs on the vector ALUs while the matrix cores finish the scores of tile 1, and the
+      // softmax of tile 1 while they accumulate P V of tile 0.
+      if constexpr (GENERAL) {
+        if (mask_row) {
+          // softmax(scale*s + mask) = softmax(scale * (s + mask/scale)): fold the mask into the raw scores
+#pragma unroll
+          for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[jt][r] = fmaf(to_f32<T>(mk[jt][r / 4][r % 4]), mask_factor, s[jt][r]);
+        }
+      }
+      const bool need_mask = (CAUSAL && n0 + kBlockN - 1 > q0) || (n0 + kBlockN > Skv);
+      Frag pf[4];
+      softmax_tile(n0, need_mask, s[0], &pf[0]);
+      pv_tile(v_src, 0, &pf[0]);
+      softmax_tile(n0 + 32, need_mask, s[1], &pf[2]);
+      pv_tile(v_src, 1, &pf[2]);
+    };
+
+    load_kv(0, k_lds0, v_lds0);
+    int step = 0;
+    for (; step + 1 < n_steps; step += 2) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      load_kv(step + 1, k_lds1, v_lds1);
+      process(step, k_lds0, v_lds0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (step + 2 < n_steps) load_kv(step + 2, k_lds0, v_lds0);
+      process(step + 1, k_lds1, v_lds1);
+    }
+    if (step < n_steps) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      process(step, k_lds0, v_lds0);
+    }
+
+    // ---- epilogue: o_acc[dt][r] is O[qrow][dt*32 + 8*(r/4) + 4*half + r%4] * l
+    const float l_tot = l_i + other_half(l_i);
+    const float inv_l = 1.0f / l_tot;
+    if (qrow < S) {
+      OutT* o_row = O + base + (int64_t)qrow * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int d = dt * 32 + 8 * q4 + 4 * half;
+          store4o<OutT>(o_row + d, o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l,
+                        o_acc[dt][q4 * 4 + 2] * inv_l, o_acc[dt][q4 * 4 + 3] * inv_l);
+        }
+    }
+    __syncthreads();                                            // the next unit's copies reuse both stages
   }
 }
 
@@ -400,12 +412,23 @@ void flash_fwd_rowwise(const T* __restrict__ Q, const T* __restrict__ K, const T
   }
 }
 
+// Grid of the persistent kernel: what the chip holds at once (a multiple of 8 so every XCD gets the same number
+// of workgroups), or one workgroup per unit when there are fewer units than that.
+inline int64_t resident_grid(int64_t units, int per_cu) {
+  const int cus = hexmi_num_cus();
+  if (cus <= 0) return -1;
+  const int64_t resident = (int64_t)cus * per_cu / 8 * 8;
+  return units < resident || resident == 0 ? units : resident;
+}
+
 template <typename T, typename OutT, int D, bool CAUSAL, int NW>
 int launch_mfma_nw(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
                    hipStream_t st) {
   const int64_t nqb = (S + NW * 32 - 1) / (NW * 32);
-  const int64_t blocks = nqb * ZH;
-  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  const int64_t units = nqb * ZH;
+  if (units > 0x7fffffff) return HEXMI_ENOTSUP;
+  const int64_t blocks = resident_grid(units, NW == 4 ? 2 : 1);
+  if (blocks <= 0) return HEXMI_ELAUNCH;
   hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, CAUSAL, false, NW>), dim3((unsigned)blocks), dim3(NW * 64), 0, st,
                      static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
                      static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e);
@@ -428,8 +451,10 @@ template <typename T, typename OutT, int D>
 int launch_mfma_general(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
                         int64_t Skv, float scale_log2e, hipStream_t st) {
   const int64_t nqb = (S + 127) / 128;
-  const int64_t blocks = nqb * ZH;
-  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  const int64_t units = nqb * ZH;
+  if (units > 0x7fffffff) return HEXMI_ENOTSUP;
+  const int64_t blocks = resident_grid(units, 2);
+  if (blocks <= 0) return HEXMI_ELAUNCH;
   const float mask_factor = 1.44269504088896340736f / scale_log2e;     // mask / sm_scale
   hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, false, true>), dim3((unsigned)blocks), dim3(256), 0, st,
                      static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
