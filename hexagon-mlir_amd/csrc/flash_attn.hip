@@ -34,6 +34,13 @@ template <> struct MfmaT<f16> {
   static __device__ __forceinline__ Frag pack(const float* p) {
     return Frag{(f16)p[0], (f16)p[1], (f16)p[2], (f16)p[3], (f16)p[4], (f16)p[5], (f16)p[6], (f16)p[7]};
   }
+  // acc + the eight packed values, two per instruction
+  static __device__ __forceinline__ float sum8(Frag f, float acc) {
+    const f16x2 one = {(f16)1.0f, (f16)1.0f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2(f16x2{f[2 * e], f[2 * e + 1]}, one, acc, false);
+    return acc;
+  }
 };
 template <> struct MfmaT<bf16> {
   typedef bf16x8 Frag;
@@ -42,6 +49,13 @@ template <> struct MfmaT<bf16> {
   }
   static __device__ __forceinline__ Frag pack(const float* p) {
     return Frag{(bf16)p[0], (bf16)p[1], (bf16)p[2], (bf16)p[3], (bf16)p[4], (bf16)p[5], (bf16)p[6], (bf16)p[7]};
+  }
+  static __device__ __forceinline__ float sum8(Frag f, float acc) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const bf16x2_t one = {(bf16)1.0f, (bf16)1.0f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2_t{f[2 * e], f[2 * e + 1]}, one, acc, false);
+    return acc;
   }
 };
 
@@ -231,15 +245,13 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
           for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
       }
       float p[16];
-      float sum = 0.0f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, -m_i));
-        sum += p[r];
-      }
-      l_i += sum;
+      for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, -m_i));
       pf[0] = MfmaT<T>::pack(&p[0]);
       pf[1] = MfmaT<T>::pack(&p[8]);
+      // the running sum takes the probabilities as rounded for the matrix cores (what P V actually multiplies),
+      // two per instruction
+      l_i = MfmaT<T>::sum8(pf[1], MfmaT<T>::sum8(pf[0], l_i));
     };
     // O^T += V^T P^T for one 32-key tile. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
     // which is score register hf*8 + e of this lane, so the packed probabilities are used as they are.
