@@ -236,3 +236,18 @@ def test_attention_long_sequences(hexmi, oracle, case):
         short = hexmi.flash_attention(q[:, :, :300].contiguous().cuda(), k[:, :, :300].contiguous().cuda(),
                                       v[:, :, :300].contiguous().cuda(), scale, True).cpu()
         assert (short.float() - got[:, :, :300].float()).abs().max() <= 2e-3
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("case", [(2, 36, 1280, 64), (1, 72, 1024, 128), (5, 13, 777, 128)])
+def test_attention_more_units_than_resident_workgroups(hexmi, case, causal):
+    # more (head, query block) units than the persistent grid holds, head counts that are and are not multiples of
+    # the 8 XCDs, ragged lengths: every unit must be visited exactly once. Oracle: the PyTorch CPU call the
+    # reference's test uses (test/python/triton/test_flash_attention.py:212).
+    Z, H, S, D = case
+    q, k, v = _qkv(Z, H, S, D, torch.float16, seed=5)
+    scale = 1.0 / math.sqrt(D)
+    got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal, out_dtype=torch.float32).cpu()
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal,
+                                                            scale=scale)
+    assert (got - want).abs().max() <= 5e-3
