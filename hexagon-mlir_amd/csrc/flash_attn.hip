@@ -214,23 +214,30 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       v_loader.issue(v_g, step * kBlockN, Skv, v_dst);
     };
 
-    // One 32-key tile of the online softmax: mask, row max, (rare) rescale, exponentials, row sum; leaves the
-    // probabilities as the two MFMA operands pf[0], pf[1] (score registers 0..7 and 8..15 of this lane).
-    // The reference maximum m_i may lag the true running maximum by up to kRescaleLag (log2 units): softmax is
-    // shift invariant, so exponentials up to 2^kRescaleLag are as exact as ones below 1, and the output
-    // accumulator and running sum only need rescaling when a row outgrows the lag. The decision is per row (lane);
-    // the wave-uniform ballot only skips the multiplications when no row of the wave needs them.
-    auto softmax_tile = [&](int key_base, bool need_mask, f32x16& s, Frag* pf) __attribute__((always_inline)) {
+    // Online softmax of one 64-key block (two 32-key score tiles): mask, row max, (rare) rescale; the exponentials
+    // follow per tile (exp_tile). The reference maximum m_i may lag the true running maximum by up to kRescaleLag
+    // (log2 units): softmax is shift invariant, so exponentials up to 2^kRescaleLag are as exact as ones below 1,
+    // and the output accumulator and running sum only need rescaling when a row outgrows the lag. The decision is
+    // per row (lane); the wave-uniform ballot only skips the multiplications when no row of the wave needs them.
+    // One decision per block (not per tile) leaves one branch between the score MFMAs and everything after them,
+    // so the exponentials of the second tile can be scheduled under the P V MFMAs of the first.
+    float neg_m = 0.0f;                                 // -(reference maximum) as the exponentials use it
+    auto block_max = [&](int n0, bool need_mask, f32x16* s) __attribute__((always_inline)) {
       if (need_mask) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = key_base + 8 * (r / 4) + 4 * half + r % 4;
-          if ((CAUSAL && key > qrow) || key >= Skv) s[r] = -INFINITY;
-        }
-      }
-      float mx = -INFINITY;
+        for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
+          for (int r = 0; r < 16; ++r) {
+            const int key = n0 + jt * 32 + 8 * (r / 4) + 4 * half + r % 4;
+            if ((CAUSAL && key > qrow) || key >= Skv) s[jt][r] = -INFINITY;
+          }
+      }
+      float mx = -INFINITY, mx1 = -INFINITY;            // one chain per tile: three-operand maxima, no NaN quieting
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[0][r]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx1 = fmaxf(mx1, s[1][r]);
+      mx = fmaxf(mx, mx1);
       mx = fmaxf(mx, other_half(mx));
       const float m_blk = mx * scale_log2e;
       const bool grow = m_blk > m_i + kRescaleLag;
@@ -243,10 +250,17 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+        // a row with every key masked so far keeps m_i = -inf and neg_m = 0: its scores are all -inf and give
+        // exp2(-inf) = 0, not exp2(-inf + inf)
+        neg_m = m_i == -INFINITY ? 0.0f : -m_i;
       }
+    };
+    // probabilities of one 32-key tile as the two MFMA operands pf[0], pf[1] (score registers 0..7 and 8..15 of
+    // this lane), and their sum into l_i
+    auto exp_tile = [&](const f32x16& s, Frag* pf) __attribute__((always_inline)) {
       float p[16];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, -m_i));
+      for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, neg_m));
       pf[0] = MfmaT<T>::pack(&p[0]);
       pf[1] = MfmaT<T>::pack(&p[8]);
       // the running sum takes the probabilities as rounded for the matrix cores (what P V actually multiplies),
@@ -254,25 +268,34 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       l_i = MfmaT<T>::sum8(pf[1], MfmaT<T>::sum8(pf[0], l_i));
     };
     // O^T += V^T P^T for one 32-key tile. MFMA k-slot (half h, e) <-> key jt*32 + hf*16 + 8*(e/4) + 4*h + e%4,
-    // which is score register hf*8 + e of this lane, so the packed probabilities are used as they are.
-    auto pv_tile = [&](const T* v_src, int jt, const Frag* pf) __attribute__((always_inline)) {
+    // which is score register hf*8 + e of this lane, so the packed probabilities are used as they are. The V
+    // fragments of a tile (read_v) do not depend on the scores: the first tile's are read before the softmax so
+    // their LDS latency is spent under it.
+    struct VFrags { Frag f[2][DT]; };
+    auto read_v = [&](const T* v_src, int jt, VFrags& vf) __attribute__((always_inline)) {
       const int g = lane / 16, i16 = lane % 16;
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          union { i16x4 h[2]; Frag f; } vf;
+          union { i16x4 h[2]; Frag f; } u;
 #pragma unroll
           for (int pp = 0; pp < 2; ++pp) {
             const int row = jt * 32 + hf * 16 + 8 * pp + 4 * (g >> 1) + (i16 >> 2);
             const int col = dt * 32 + (g & 1) * 16 + (i16 & 3) * 4;
             const int c = (col / 8) ^ swz_vtile<D>(row);
             const T* addr = v_src + (row * CPR + c) * 8 + (col % 8);
-            vf.h[pp] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
+            u.h[pp] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(addr));
           }
-          o_acc[dt] = MfmaT<T>::run(vf.f, pf[hf], o_acc[dt]);
+          vf.f[hf][dt] = u.f;
         }
       }
+    };
+    auto pv_tile = [&](const VFrags& vf, const Frag* pf) __attribute__((always_inline)) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o_acc[dt] = MfmaT<T>::run(vf.f[hf][dt], pf[hf], o_acc[dt]);
     };
 
     // mask row of this lane's query (GENERAL with a mask only)
@@ -301,22 +324,45 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
             }
         }
       }
-      // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4], one MFMA chain per 32-key tile
+      // ---- scores: s[jt][r] = Q[qrow] . K[n0 + jt*32 + 8*(r/4) + 4*half + r%4]. The MFMA chains of the two 32-key
+      // tiles are interleaved (a chain alone waits for its own previous result) and their K fragments are read
+      // kAhead steps ahead of use, so the LDS latency is paid once per block and not once per step.
       f32x16 s[2];
 #pragma unroll
-      for (int jt = 0; jt < 2; ++jt) {
+      for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[jt][r] = 0.0f;
-        const int krow = jt * 32 + lane % 32;
+      {
+        constexpr int kAhead = GENERAL ? 2 : 3;      // the masked kernel holds its mask values too
+        const int krow = lane % 32;
+        auto read_k = [&](int jt, int ds) __attribute__((always_inline)) {
+          const int row = jt * 32 + krow;
+          const int c = (ds * 2 + half) ^ swz_ktile<D>(row);
+          return *reinterpret_cast<const Frag*>(k_src + (row * CPR + c) * 8);
+        };
+        Frag kf[2][DS];
+#pragma unroll
+        for (int ds = 0; ds < kAhead && ds < DS; ++ds) {
+          kf[0][ds] = read_k(0, ds);
+          kf[1][ds] = read_k(1, ds);
+        }
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
-          const int c = (ds * 2 + half) ^ swz_ktile<D>(krow);
-          Frag kf = *reinterpret_cast<const Frag*>(k_src + (krow * CPR + c) * 8);
-          s[jt] = MfmaT<T>::run(kf, qf[ds], s[jt]);
+          if (ds + kAhead < DS) {
+            kf[0][ds + kAhead] = read_k(0, ds + kAhead);
+            kf[1][ds + kAhead] = read_k(1, ds + kAhead);
+          }
+          s[0] = MfmaT<T>::run(kf[0][ds], qf[ds], s[0]);
+          s[1] = MfmaT<T>::run(kf[1][ds], qf[ds], s[1]);
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
-      // The softmax of tile 0 runs on the vector ALUs while the matrix cores finish the scores of tile 1, and the
-      // softmax of tile 1 while they accumulate P V of tile 0.
+      VFrags vf0, vf1;
+      constexpr bool kEarlyV = !GENERAL;                // the masked kernel has no registers to spare for it
+      if constexpr (kEarlyV) {
+        read_v(v_src, 0, vf0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if constexpr (GENERAL) {
         if (mask_row) {
           // softmax(scale*s + mask) = softmax(scale * (s + mask/scale)): fold the mask into the raw scores
@@ -327,11 +373,15 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
         }
       }
       const bool need_mask = (CAUSAL && n0 + kBlockN - 1 > q0) || (n0 + kBlockN > Skv);
+      block_max(n0, need_mask, s);
+      // The exponentials of tile 1 run on the vector ALUs while the matrix cores accumulate P V of tile 0.
       Frag pf[4];
-      softmax_tile(n0, need_mask, s[0], &pf[0]);
-      pv_tile(v_src, 0, &pf[0]);
-      softmax_tile(n0 + 32, need_mask, s[1], &pf[2]);
-      pv_tile(v_src, 1, &pf[2]);
+      if constexpr (!kEarlyV) read_v(v_src, 0, vf0);
+      read_v(v_src, 1, vf1);
+      exp_tile(s[0], &pf[0]);
+      pv_tile(vf0, &pf[0]);
+      exp_tile(s[1], &pf[2]);
+      pv_tile(vf1, &pf[2]);
     };
 
     load_kv(0, k_lds0, v_lds0);

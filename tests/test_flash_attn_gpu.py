@@ -222,6 +222,25 @@ def test_masked_attention_fully_masked_row_is_nan(hexmi):
     assert torch.isnan(got[0, 5]).all() and not torch.isnan(got[0, :5]).any() and not torch.isnan(got[0, 6:]).any()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", [(2, 200, 320, 128, 40), (1, 130, 260, 64, 70)])
+def test_masked_attention_window_mask(hexmi, oracle, case, dtype):
+    # a band mask (-inf outside a window that ends past the row index): most rows have every key of their first
+    # 64-key blocks masked out, so the running maximum is still -inf when the first finite score arrives
+    B, Sq, Skv, D, width = case
+    g = _gen(31)
+    q = torch.randn(B, Sq, D, generator=g).to(dtype)
+    k, v = torch.randn(B, Skv, D, generator=g).to(dtype), torch.randn(B, Skv, D, generator=g).to(dtype)
+    rows, cols = torch.arange(Sq)[:, None], torch.arange(Skv)[None, :]
+    keep = (cols > rows + 60 - width) & (cols <= rows + 60)
+    mask = torch.zeros(Sq, Skv).masked_fill(~keep, float("-inf")).to(dtype).expand(B, Sq, Skv).contiguous()
+    scale = 1.0 / math.sqrt(D)
+    got = hexmi.attention(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).cpu()
+    want = _oracle_masked(oracle, q, k, v, mask, scale)
+    assert not torch.isnan(got).any()
+    assert (got.float() - want).abs().max() <= (2e-2 if dtype == torch.float16 else 4e-2)
+
+
 @pytest.mark.parametrize("case", [(1, 1, 8200, 64, True), (1, 1, 8192, 128, False), (1, 2, 8192 + 130, 128, True)])
 def test_attention_long_sequences(hexmi, oracle, case):
     # sequences of 8192 keys and more run 8-wave workgroups (256 query rows per K/V tile copy)
