@@ -21,7 +21,7 @@ namespace {
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 
-constexpr int kWideMinS = 8192;  // sequences at least this long use 8-wave (256-row) workgroups
+constexpr int kWideMinS = 2048;  // sequences at least this long may use 8-wave (256-row) workgroups
 constexpr int kBlockN = 64;    // keys per step
 constexpr float kRescaleLag = 8.0f;   // how far (log2) the softmax reference maximum may trail the true one
 
@@ -132,7 +132,7 @@ template <> __device__ __forceinline__ void store4o<bf16>(bf16* p, float a, floa
 // tm_tensor.attention does (qcom_hexagon_backend/lib/Transforms/LowerTmTensor.cpp:157-160); Skv % 4 == 0.
 // NW waves per workgroup (4 or 8), 32 query rows each: every K / V tile copied into LDS serves NW*32 query rows.
 // Eight waves halve the L2 -> LDS copy traffic (each query block streams the whole K and V of its head), worth
-// about 4 % at 16k keys; shorter sequences prefer the larger number of 128-row workgroups. (Measured on random
+// 1-9 % from 2048 keys on; short sequences and small grids prefer the larger number of 128-row workgroups. (Measured on random
 // data the kernel is held back by the power limit more than by any stall: all-zero inputs run 30 % faster through
 // the same instructions and the same memory traffic, as the dense GEMM also shows.)
 template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, int NW = 4>
@@ -500,7 +500,9 @@ int launch_mfma_nw(const void* Q, const void* K, const void* V, void* O, int64_t
 template <typename T, typename OutT, int D>
 int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
                 bool causal, hipStream_t st) {
-  const bool wide = S >= kWideMinS;
+  // 256-row workgroups halve the L2 -> LDS copy traffic (1-9 % faster from 2048 keys on), if there are enough of
+  // them to fill the chip; smaller problems keep the larger number of 128-row workgroups
+  const bool wide = S >= kWideMinS && ZH * ((S + 255) / 256) >= hexmi_num_cus();
   if (causal) {
     if (wide) return launch_mfma_nw<T, OutT, D, true, 8>(Q, K, V, O, ZH, S, scale_log2e, st);
     return launch_mfma_nw<T, OutT, D, true, 4>(Q, K, V, O, ZH, S, scale_log2e, st);

@@ -243,7 +243,7 @@ def test_masked_attention_window_mask(hexmi, oracle, case, dtype):
 
 @pytest.mark.parametrize("case", [(1, 1, 8200, 64, True), (1, 1, 8192, 128, False), (1, 2, 8192 + 130, 128, True)])
 def test_attention_long_sequences(hexmi, oracle, case):
-    # sequences of 8192 keys and more run 8-wave workgroups (256 query rows per K/V tile copy)
+    # long sequences, few heads (too few 256-row workgroups to fill the chip: 128-row workgroups)
     Z, H, S, D, causal = case
     q, k, v = _qkv(Z, H, S, D, torch.float16, seed=7)
     scale = 1.0 / math.sqrt(D)
@@ -255,6 +255,22 @@ def test_attention_long_sequences(hexmi, oracle, case):
         short = hexmi.flash_attention(q[:, :, :300].contiguous().cuda(), k[:, :, :300].contiguous().cuda(),
                                       v[:, :, :300].contiguous().cuda(), scale, True).cpu()
         assert (short.float() - got[:, :, :300].float()).abs().max() <= 2e-3
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("case", [(2, 16, 2048 + 70, 128, torch.float16), (1, 40, 2048, 64, torch.float16),
+                                  (4, 8, 2304, 128, torch.bfloat16), (1, 8, 8192 + 130, 128, torch.float16)])
+def test_attention_256_row_workgroups(hexmi, case, causal):
+    # from 2048 keys on, grids with at least one 256-row block per CU run 8-wave workgroups (256 query rows per
+    # K/V tile copy): ragged lengths, head counts off the XCD multiple, both dtypes. Oracle: the PyTorch CPU call
+    # the reference's test uses (test/python/triton/test_flash_attention.py:212).
+    Z, H, S, D, dtype = case
+    q, k, v = _qkv(Z, H, S, D, dtype, seed=9)
+    scale = 1.0 / math.sqrt(D)
+    got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal, out_dtype=torch.float32).cpu()
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal,
+                                                            scale=scale)
+    assert (got - want).abs().max() <= (5e-3 if dtype == torch.float16 else 3e-2)
 
 
 @pytest.mark.parametrize("causal", [False, True])
