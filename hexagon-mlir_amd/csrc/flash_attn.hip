@@ -106,6 +106,36 @@ struct KvTileLoader {
   }
 };
 
+// global -> LDS copy of the additive-mask tile of one wave: [32 query rows][64 keys], 128 bytes per row, four
+// wave-wide instructions of 8 rows each. A lane later reads 8-byte runs of its own row (lane%32), so the 16-byte
+// chunks of a row are XOR swizzled by row/2: the 32 rows of a read then cover every bank twice, the minimum for
+// 512 bytes. Keys past the end of the sequence are clamped to the last chunk (their scores are dropped anyway),
+// rows past the last query to the last query.
+template <typename T>
+struct MaskTileLoader {
+  int rowoff[4];                                            // element offset of this lane's row from the first row
+  int col0;                                                 // first key of this lane's chunk inside the tile, j = 0
+  __device__ __forceinline__ void init(int wave, int lane, int rows_left, int Skv) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int r = wave * 32 + j * 8 + lane / 8;                 // row j*8 + lane/8 of the tile
+      r = r < rows_left ? r : rows_left - 1;
+      rowoff[j] = r * Skv;
+    }
+    col0 = ((lane % 8) ^ ((lane / 16) & 7)) * 8;            // swizzle (row/2)%8 = (lane/16 + 4*(j%2)) % 8
+  }
+  // mask_wg: the mask row of the workgroup's first query; lds: this wave's [32][64] tile of the stage
+  __device__ __forceinline__ void issue(const T* __restrict__ mask_wg, int key0, int Skv, T* lds) const {
+    const char* base = reinterpret_cast<const char*>(mask_wg);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int key = key0 + (col0 ^ ((j & 1) * 32));
+      key = key + 8 <= Skv ? key : Skv - 8;
+      copy_to_lds(base, (rowoff[j] + key) * (int)sizeof(T), lds + j * 512);
+    }
+  }
+};
+
 // Value held by lane ^ 32 (v_permlane32_swap exchanges the upper half of one register with the lower half of
 // another; no LDS round trip).
 __device__ __forceinline__ float other_half(float v) {
@@ -135,12 +165,16 @@ template <> __device__ __forceinline__ void store4o<bf16>(bf16* p, float a, floa
 // 1-9 % from 2048 keys on; short sequences and small grids prefer the larger number of 128-row workgroups. (Measured on random
 // data the kernel is held back by the power limit more than by any stall: all-zero inputs run 30 % faster through
 // the same instructions and the same memory traffic, as the dense GEMM also shows.)
-template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, int NW = 4>
+// MASK_LDS (GENERAL, 8 waves, a mask with Skv % 8 == 0): the mask tiles are copied global -> LDS one key block ahead
+// like K and V (no registers, whole 128-byte rows), instead of being loaded into registers in 8-byte runs at the
+// top of the block that uses them.
+template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, int NW = 4, bool MASK_LDS = false>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1)
 void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                       OutT* __restrict__ O, int ZH, int S, float scale_log2e, const T* __restrict__ Mk = nullptr,
                       int Skv_arg = 0, float mask_factor = 0.0f) {
   static_assert(!(CAUSAL && GENERAL), "the causal kernel has as many keys as queries and no mask");
+  static_assert(!MASK_LDS || (GENERAL && NW == 8), "staged mask tiles: general kernel, 8 waves");
   const int Skv = GENERAL ? Skv_arg : S;
   typedef typename MfmaT<T>::Frag Frag;
   constexpr int DS = D / 16;                        // 16-wide steps over the head dimension
@@ -150,6 +184,8 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   __shared__ __attribute__((aligned(16))) T k_lds1[kBlockN * D];
   __shared__ __attribute__((aligned(16))) T v_lds0[kBlockN * D];
   __shared__ __attribute__((aligned(16))) T v_lds1[kBlockN * D];
+  __shared__ __attribute__((aligned(16))) T m_lds0[MASK_LDS ? NW * 32 * kBlockN : 8];
+  __shared__ __attribute__((aligned(16))) T m_lds1[MASK_LDS ? NW * 32 * kBlockN : 8];
 
   constexpr int kBlockM = NW * 32;                  // query rows per workgroup
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -209,9 +245,16 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     KvTileLoader<T, D, true, NW> v_loader;
     k_loader.init(wave, lane);
     v_loader.init(wave, lane);
-    auto load_kv = [&](int step, T* k_dst, T* v_dst) __attribute__((always_inline)) {
+    MaskTileLoader<T> m_loader;
+    const T* mask_wg = nullptr;
+    if constexpr (MASK_LDS) {
+      mask_wg = Mk + ((int64_t)zh * S + qb * kBlockM) * Skv;
+      m_loader.init(wave, lane, S - qb * kBlockM, Skv);
+    }
+    auto load_kv = [&](int step, T* k_dst, T* v_dst, T* m_dst) __attribute__((always_inline)) {
       k_loader.issue(k_g, step * kBlockN, Skv, k_dst);
       v_loader.issue(v_g, step * kBlockN, Skv, v_dst);
+      if constexpr (MASK_LDS) m_loader.issue(mask_wg, step * kBlockN, Skv, m_dst + wave * (32 * kBlockN));
     };
 
     // Online softmax of one 64-key block (two 32-key score tiles): mask, row max, (rare) rescale; the exponentials
@@ -300,11 +343,11 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
 
     // mask row of this lane's query (GENERAL with a mask only)
     const T* mask_row = nullptr;
-    if constexpr (GENERAL) {
+    if constexpr (GENERAL && !MASK_LDS) {
       if (Mk) mask_row = Mk + ((int64_t)zh * S + (qrow < S ? qrow : S - 1)) * Skv;
     }
 
-    auto process = [&](int step, const T* k_src, const T* v_src) __attribute__((always_inline)) {
+    auto process = [&](int step, const T* k_src, const T* v_src, const T* m_src) __attribute__((always_inline)) {
       const int n0 = step * kBlockN;
       // causal: a key block wholly past this wave's 32 rows contributes nothing (wave-uniform; the workgroup's
       // barriers and copies are outside)
@@ -312,7 +355,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       // mask values of this lane's 32 scores: four runs of four consecutive keys per 32-key tile
       typedef T MaskRun __attribute__((ext_vector_type(4)));
       MaskRun mk[2][4];
-      if constexpr (GENERAL) {
+      if constexpr (GENERAL && !MASK_LDS) {
         if (mask_row) {
 #pragma unroll
           for (int jt = 0; jt < 2; ++jt)
@@ -363,8 +406,17 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
         read_v(v_src, 0, vf0);
         __builtin_amdgcn_sched_barrier(0);
       }
+      if constexpr (MASK_LDS) {                         // staged mask tile: read after the score MFMAs are issued
+        const int row = lane % 32;
+        const T* m_row = m_src + wave * (32 * kBlockN) + row * kBlockN + half * 4;
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4)
+            mk[jt][g4] = *reinterpret_cast<const MaskRun*>(m_row + ((jt * 4 + g4) ^ ((row >> 1) & 7)) * 8);
+      }
       if constexpr (GENERAL) {
-        if (mask_row) {
+        if (MASK_LDS || mask_row) {
           // softmax(scale*s + mask) = softmax(scale * (s + mask/scale)): fold the mask into the raw scores
 #pragma unroll
           for (int jt = 0; jt < 2; ++jt)
@@ -384,22 +436,22 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       pv_tile(vf1, &pf[2]);
     };
 
-    load_kv(0, k_lds0, v_lds0);
+    load_kv(0, k_lds0, v_lds0, m_lds0);
     int step = 0;
     for (; step + 1 < n_steps; step += 2) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      load_kv(step + 1, k_lds1, v_lds1);
-      process(step, k_lds0, v_lds0);
+      load_kv(step + 1, k_lds1, v_lds1, m_lds1);
+      process(step, k_lds0, v_lds0, m_lds0);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (step + 2 < n_steps) load_kv(step + 2, k_lds0, v_lds0);
-      process(step + 1, k_lds1, v_lds1);
+      if (step + 2 < n_steps) load_kv(step + 2, k_lds0, v_lds0, m_lds0);
+      process(step + 1, k_lds1, v_lds1, m_lds1);
     }
     if (step < n_steps) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      process(step, k_lds0, v_lds0);
+      process(step, k_lds0, v_lds0, m_lds0);
     }
 
     // ---- epilogue: o_acc[dt][r] is O[qrow][dt*32 + 8*(r/4) + 4*half + r%4] * l
@@ -514,12 +566,25 @@ int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH
 template <typename T, typename OutT, int D>
 int launch_mfma_general(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
                         int64_t Skv, float scale_log2e, hipStream_t st) {
+  const float mask_factor = 1.44269504088896340736f / scale_log2e;     // mask / sm_scale
+  // a mask whose rows are whole 16-byte chunks is staged through LDS by 256-row workgroups (one per CU); the
+  // copies address a workgroup's 256 mask rows with 32-bit byte offsets
+  if (mask != nullptr && Skv % 8 == 0 && aligned_to(mask, 16) && S > 128 && Skv <= (1 << 21)) {
+    const int64_t units8 = (S + 255) / 256 * ZH;
+    if (units8 > 0x7fffffff) return HEXMI_ENOTSUP;
+    const int64_t blocks8 = resident_grid(units8, 1);
+    if (blocks8 <= 0) return HEXMI_ELAUNCH;
+    hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, false, true, 8, true>), dim3((unsigned)blocks8), dim3(512), 0,
+                       st, static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                       static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e, static_cast<const T*>(mask), (int)Skv,
+                       mask_factor);
+    return launch_status();
+  }
   const int64_t nqb = (S + 127) / 128;
   const int64_t units = nqb * ZH;
   if (units > 0x7fffffff) return HEXMI_ENOTSUP;
   const int64_t blocks = resident_grid(units, 2);
   if (blocks <= 0) return HEXMI_ELAUNCH;
-  const float mask_factor = 1.44269504088896340736f / scale_log2e;     // mask / sm_scale
   hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, false, true>), dim3((unsigned)blocks), dim3(256), 0, st,
                      static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
                      static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e, static_cast<const T*>(mask), (int)Skv,

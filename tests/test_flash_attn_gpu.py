@@ -158,7 +158,10 @@ def _mask(B, Sq, Skv, dtype, seed, drop=0.3):
 
 
 MASKED_CASES = [(2, 128, 128, 128), (3, 200, 72, 64), (1, 1, 64, 128), (2, 77, 516, 128), (1, 300, 4, 64),
-                (1, 130, 1024, 128), (2, 65, 66, 64), (1, 40, 100, 80)]   # the last two: Skv % 4 != 0 / other D
+                (1, 130, 1024, 128), (2, 65, 66, 64), (1, 40, 100, 80),   # the last two: Skv % 4 != 0 / other D
+                # more than 128 queries and Skv % 8 == 0: mask tiles staged through LDS by 256-row workgroups
+                # (ragged last row block, ragged last key block, several row blocks, many batch entries)
+                (3, 300, 520, 128), (2, 513, 72, 64), (1, 257, 2048 + 8, 128), (40, 129, 136, 64)]
 
 
 @pytest.mark.parametrize("with_mask", [True, False])
