@@ -14,8 +14,14 @@ extern "C" const char* hexmi_strerror(int status) {
 }
 
 extern "C" int hexmi_num_cus(void) {
+  // launchers ask on every call: the attribute is looked up once per device (a racing first call stores the same
+  // value twice)
+  constexpr int kMaxDevices = 64;
+  static int cached[kMaxDevices];
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < kMaxDevices && cached[dev] > 0) return cached[dev];
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < kMaxDevices) cached[dev] = cus;
   return cus;
 }
