@@ -27,6 +27,7 @@ for _p in (ROOT, os.path.join(ROOT, "hexagon-mlir_amd")):
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 / bf16 matrix, published
+MFMA_F32_PEAK_TFLOPS = 157.3   # MI355X fp32 matrix, published
 ROTATE_BYTES = 640 << 20       # rotate HBM-bound workloads over more than 2x the 256 MB Infinity Cache
 
 
@@ -157,7 +158,9 @@ class Gemm(Workload):
 
     def setup(self, torch, hexmi):
         from hexmi.workloads import gemm_inputs, gemm_flops
-        dt = torch.float16 if self.dtype == "f16" else torch.bfloat16
+        dt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[self.dtype]
+        if self.dtype == "f32":
+            self.kernel, self.peak = "gemm_f32_mfma_kernel", MFMA_F32_PEAK_TFLOPS
         self.hexmi, self.host = hexmi, gemm_inputs(self.size, self.size, self.size, dt)
         self.work = gemm_flops(self.size, self.size, self.size)
         self.sets = _sets(torch, self.host, 0, rotate=False)
@@ -365,14 +368,14 @@ def _time_cpu(fn, iters):
 
 def make_workloads():
     return {w.name: w for w in (
-        Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
+        Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"), Gemm(4096, "f32"),
         W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
         Elementwise("sum"),
         CopyCalibration())}
 
 
 ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "gemm": "gemm_f16_4096",
-           "gemm_bf16": "gemm_bf16_8192", "attn": "attn_causal_f16_4x32x4096x128",
+           "gemm_bf16": "gemm_bf16_8192", "gemm_f32": "gemm_f32_4096", "attn": "attn_causal_f16_4x32x4096x128",
            "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
            "rope": "rope_f16_4x4096x32x128", "sum": "block_sum_f32_8192x4096", "rms_norm": "rms_norm_f16_8192x4096",
            "layer_norm": "layer_norm_f16_8192x4096"}
@@ -415,7 +418,7 @@ def measure(torch, wl, steps, warmup, use_graph=True):
 
 
 PROFILE_KEYS = {"norms_f16_8192x4096": "norms", "softmax_f32_4096x1024": "softmax", "gemm_f16_4096": "gemm",
-                "gemm_bf16_8192": "gemm_bf16", "w8a16_m1": "w8a16_m1", "w8a16_m16": "w8a16_m16",
+                "gemm_bf16_8192": "gemm_bf16", "gemm_f32_4096": "gemm_f32", "w8a16_m1": "w8a16_m1", "w8a16_m16": "w8a16_m16",
                 "w8a16_m256": "w8a16_m256", "attn_causal_f16_4x32x4096x128": "attn",
                 "attn_causal_f16_1x32x16384x128": "attn_long", "attn_masked_f16_32x2048x128": "attn_masked"}
 
@@ -435,14 +438,14 @@ def report(wl, ms):
     if wl.bound == "hbm":
         achieved, peak, unit = wl.work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
     else:
-        achieved, peak, unit = wl.work / (ms * 1e-3) / 1e12, MFMA_PEAK_TFLOPS, "TFLOP/s"
+        achieved, peak, unit = wl.work / (ms * 1e-3) / 1e12, getattr(wl, "peak", MFMA_PEAK_TFLOPS), "TFLOP/s"
     return {"bound": wl.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
             "frac": round(achieved / peak, 4), "traffic": measured_traffic(wl), "kernel": wl.kernel,
             "work_per_step": wl.work}
 
 
 def steps_for(wl, steps):
-    if wl.name.startswith("gemm_bf16_8192") or "16384" in wl.name:
+    if wl.name.startswith("gemm_bf16_8192") or wl.name.startswith("gemm_f32") or "16384" in wl.name:
         return max(5, steps // 5)
     return steps
 

@@ -881,8 +881,9 @@ void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT*
 }
 
 // fp32 inputs (the reference's torch-mlir graphs multiply fp32 matrices, e.g.
-// test/python/torch-mlir/test_add_matmul_softmax.py:25-29): 64x64 tile, K in steps of 16 through LDS, every thread a
-// 4x4 block of fp32 FMAs. Any shape; not a matrix-core path (no fp16 rounding of the operands).
+// test/python/torch-mlir/test_add_matmul_softmax.py:25-29) whose shape or alignment the matrix-core kernel of
+// gemm_f32.hip does not take: 64x64 tile, K in steps of 16 through LDS, every thread a 4x4 block of fp32 FMAs.
+// Any shape.
 template <bool TRANS_B>
 __global__ __launch_bounds__(256)
 void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C, int M, int N,
@@ -943,11 +944,13 @@ void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, f
 
 int launch_f32(bool trans_b, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
                int64_t ldb, int64_t ldc, hipStream_t s) {
-  dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
-  if (grid.y > 65535) return HEXMI_ENOTSUP;
   const float* a = static_cast<const float*>(A);
   const float* b = static_cast<const float*>(B);
   float* c = static_cast<float*>(C);
+  int status = HEXMI_OK;
+  if (gemm_f32_mfma(trans_b, a, b, c, M, N, K, lda, ldb, ldc, s, &status)) return status;   // matrix cores
+  dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+  if (grid.y > 65535) return HEXMI_ENOTSUP;
   if (trans_b)
     hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, s, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc);
   else

@@ -143,4 +143,9 @@ inline int dtype_size(int dtype) {
 int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,
                      hipStream_t stream);
 
+// fp32 GEMM on the matrix cores (gemm_f32.hip): launches and returns true when the shapes fit (K % 32 == 0, aligned
+// operands), with the launch status in *status; false leaves the product to the vector-ALU kernel.
+bool gemm_f32_mfma(bool trans_b, const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
+                   int64_t lda, int64_t ldb, int64_t ldc, hipStream_t stream, int* status);
+
 }  // namespace hexmi

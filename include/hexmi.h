@@ -101,9 +101,11 @@ int hexmi_matmul_f16f16_f32(int64_t n_row, int64_t n_col, int64_t n_inner,
  *     test/python/torch-mlir/test_hexkl_macro_matmul.py:24-28).
  * in_dtype: HEXMI_F16 or HEXMI_BF16 (A and B). out_dtype: in_dtype or HEXMI_F32
  * (the fp16 x fp16 -> fp32 form of docs/tutorials/triton/matmul_hexkl.md:61-97).
- * in_dtype == out_dtype == HEXMI_F32: fp32 operands, fp32 FMAs (no matrix cores,
- * no rounding of the operands): the fp32 matmuls of the reference's torch-mlir
- * graphs (test/python/torch-mlir/test_add_matmul_softmax.py:25-29). */
+ * in_dtype == out_dtype == HEXMI_F32: fp32 operands multiplied in fp32 (no
+ * rounding of the operands): the fp32 matmuls of the reference's torch-mlir
+ * graphs (test/python/torch-mlir/test_add_matmul_softmax.py:25-29). K % 32 == 0
+ * with 16-byte aligned rows runs on the fp32 matrix cores, other shapes on the
+ * vector ALUs. */
 int hexmi_gemm(int64_t M, int64_t N, int64_t K, const void *A, int64_t lda,
                const void *B, int64_t ldb, void *C, int64_t ldc, int in_dtype,
                int out_dtype, int trans_b, hexmi_stream_t stream);

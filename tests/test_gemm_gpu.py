@@ -212,7 +212,11 @@ def test_gemm_argument_errors(hexmi):
 
 
 @pytest.mark.parametrize("trans_b", [False, True])
-@pytest.mark.parametrize("shape", [(32, 32, 32), (1, 1, 1), (65, 130, 17), (200, 77, 300), (512, 512, 512)])
+@pytest.mark.parametrize("shape", [(32, 32, 32), (1, 1, 1), (65, 130, 17), (200, 77, 300), (512, 512, 512),
+                                   # K % 32 == 0 (and N % 4 == 0 for [K,N] operands): the matrix-core kernel; ragged
+                                   # tiles on both sides, fewer rows than a fragment, several slabs, odd slab counts
+                                   (128, 128, 32), (5, 4, 64), (300, 264, 160), (129, 1028, 96), (1000, 520, 1024),
+                                   (2048, 384, 224), (64, 132, 4096)])
 def test_matmul_fp32(hexmi, oracle, shape, trans_b):
     M, N, K = shape
     g = torch.Generator().manual_seed(40)
@@ -224,6 +228,27 @@ def test_matmul_fp32(hexmi, oracle, shape, trans_b):
     assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5 * (K ** 0.5))
     with pytest.raises(TypeError):
         hexmi.matmul(a.cuda(), b.cuda(), trans_b=trans_b, out_dtype=torch.float16)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_matmul_fp32_strided_and_exact(hexmi, trans_b):
+    # operands that are views into wider buffers (leading dimensions larger than the rows), an output view, and
+    # small-integer operands whose products and sums are exact in fp32: the result must be exact, whatever the order
+    M, N, K = 200, 136, 96
+    g = torch.Generator().manual_seed(45)
+    abuf = torch.randint(-8, 9, (M, K + 32), generator=g).float().cuda()
+    bbuf = (torch.randint(-8, 9, (N, K + 64), generator=g) if trans_b else torch.randint(-8, 9, (K, N + 24), generator=g)).float().cuda()
+    cbuf = torch.full((M, N + 8), -1.0, device="cuda")
+    a, b, c = abuf[:, :K], (bbuf[:, :K] if trans_b else bbuf[:, :N]), cbuf[:, :N]
+    lib, st = hexmi.lib(), torch.cuda.current_stream().cuda_stream
+    from hexmi import _lib
+    rc = lib.hexmi_gemm(M, N, K, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), c.data_ptr(), c.stride(0),
+                        _lib.F32, _lib.F32, int(trans_b), st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    want = a.double().cpu() @ (b.double().cpu().t() if trans_b else b.double().cpu())
+    assert torch.equal(c.cpu().double(), want)
+    assert (cbuf[:, N:] == -1.0).all()                       # nothing written past the N columns
 
 
 def test_add_matmul_softmax_reference_graph(hexmi):
