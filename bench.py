@@ -255,6 +255,25 @@ class Attention(Workload):
         return t * (Z * H / heads), "%d of %d heads, fp32 F.scaled_dot_product_attention(is_causal=True) on CPU, time scaled" % (heads, Z * H)
 
 
+class AttentionF32(Attention):
+    """The reference test's own dtype (fp32 Q, K, V: test/python/triton/test_flash_attention.py:171-173) at a size
+    that fills the chip; priced against the fp32 matrix peak."""
+    dtype, kernel, peak = "f32", "flash_fwd_f32_kernel", MFMA_F32_PEAK_TFLOPS
+
+    def __init__(self, Z, H, S, D):
+        self.shape = (Z, H, S, D)
+        self.name = "attn_causal_f32_%dx%dx%dx%d" % self.shape
+        self.desc = "causal flash-attention fwd fp32 [%d,%d,%d,%d] N(0,1), scale 1/sqrt(%d)" % (Z, H, S, D, D)
+
+    def setup(self, torch, hexmi):
+        from hexmi.workloads import attention_inputs, attention_flops
+        self.hexmi, self.host = hexmi, attention_inputs(*self.shape, dtype=torch.float32)
+        self.work = attention_flops(*self.shape, causal=True)
+        t = {k: v for k, v in self.host.items() if k != "sm_scale"}
+        self.sets = _sets(torch, t, 0, rotate=False)
+        self.sets[0]["out"] = torch.empty_like(self.sets[0]["q"])
+
+
 class Elementwise(Workload):
     """The reference's small tutorial kernels at a size that needs HBM: GELU-tanh / SiLU over fp16 [8192,4096],
     RoPE over fp16 [4,4096,32,128], one sum per 4096-element program over fp32 [8192*4096]."""
@@ -369,14 +388,14 @@ def _time_cpu(fn, iters):
 def make_workloads():
     return {w.name: w for w in (
         Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"), Gemm(4096, "f32"),
-        W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
+        W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), AttentionF32(4, 32, 2048, 64), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
         Elementwise("sum"),
         CopyCalibration())}
 
 
 ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "gemm": "gemm_f16_4096",
            "gemm_bf16": "gemm_bf16_8192", "gemm_f32": "gemm_f32_4096", "attn": "attn_causal_f16_4x32x4096x128",
-           "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
+           "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128", "attn_f32": "attn_causal_f32_4x32x2048x64", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
            "rope": "rope_f16_4x4096x32x128", "sum": "block_sum_f32_8192x4096", "rms_norm": "rms_norm_f16_8192x4096",
            "layer_norm": "layer_norm_f16_8192x4096"}
 

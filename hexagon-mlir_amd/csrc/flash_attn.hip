@@ -628,8 +628,13 @@ int attention_any(const void* Q, const void* K, const void* V, const void* mask,
   if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F32) return dispatch_half<f16, float>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
   if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_BF16) return dispatch_half<bf16, bf16>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
   if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_F32) return dispatch_half<bf16, float>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
-  if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32)
+  if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) {
+    int status = HEXMI_OK;
+    if (flash_attn_f32_mfma(static_cast<const float*>(Q), static_cast<const float*>(K), static_cast<const float*>(V),
+                            static_cast<const float*>(mask), static_cast<float*>(O), ZH, S, Skv, D, c, cz, st, &status))
+      return status;
     return launch_rowwise<float, float>(Q, K, V, mask, O, ZH, S, Skv, D, c, cz, st);
+  }
   return HEXMI_ENOTSUP;
 }
 

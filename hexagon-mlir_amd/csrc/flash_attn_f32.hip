@@ -1,0 +1,266 @@
+// Flash-attention forward for fp32 operands on the fp32 matrix cores (v_mfma_f32_32x32x2_f32): the dtype of the
+// reference's own test (test/python/triton/test_flash_attention.py:171-173: torch.rand fp32 Q, K, V, [1,1,1024,64],
+// scale 0.5). Same scheme as the 16-bit kernel of flash_attn.hip, nothing rounded below fp32:
+//   a workgroup of 4 waves owns 128 query rows (32 per wave), keys walk in blocks of BN (64 for D = 64, 32 for
+//   D = 128), K and V blocks are copied global -> LDS with buffer loads, double buffered;
+//   S^T = K Q^T: a lane holds 16 scores per 32-key tile of ONE query row (row lane%32), Q stays in registers;
+//   online softmax in fp32 with exp2 (scale*log2e folded in), the reference maximum may lag by kRescaleLagF32;
+//   O^T += V^T P^T: the probabilities go from the score registers straight into the MFMA (score register r is k
+//   slot r: keys 8*(r/4) + r%4 for lanes 0..31 and + 4 for lanes 32..63), V values are read from LDS one per lane.
+// An MFMA of this shape takes 64 cycles, so a key block is 8192 matrix cycles per wave against about 500 of
+// vector work: the kernel is matrix-bound without any software pipelining.
+//
+// LDS tiles are [BN keys][D] fp32 in 16-byte chunks: K is read by 32 keys at one chunk position (chunk ^ key%16),
+// V by 32 consecutive d of two keys four apart (chunk ^ 8*((key/4)%2) puts the two half-waves on disjoint banks).
+#include "hexmi_common.h"
+
+namespace hexmi {
+namespace {
+
+constexpr float kRescaleLagF32 = 8.0f;
+typedef float f32x4a __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float other_half_f32(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned lo = r[0], hi = r[1];
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? lo : hi);
+}
+
+template <int D, int BN, bool CAUSAL, bool MASKED>
+__global__ __launch_bounds__(256, D == 64 ? 2 : 1)
+void flash_fwd_f32_kernel(const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
+                          float* __restrict__ O, int ZH, int S, int Skv, float scale_log2e,
+                          const float* __restrict__ Mk, float mask_factor) {
+  constexpr int NT = BN / 32;                       // 32-key score tiles per key block
+  constexpr int CPR = D / 4;                        // 16-byte chunks per row
+  constexpr int DT = D / 32;                        // 32-wide output tiles over the head dimension
+  constexpr int DQ = D / 8;                         // 16-byte chunks of Q per lane (one per 8 head dimensions)
+  constexpr int NI = BN * CPR / 64 / 4;             // copy instructions per wave and tile
+  constexpr int RPI = 64 / CPR;                     // rows per copy instruction
+  __shared__ __attribute__((aligned(16))) float k_s0[BN * D];
+  __shared__ __attribute__((aligned(16))) float k_s1[BN * D];
+  __shared__ __attribute__((aligned(16))) float v_s0[BN * D];
+  __shared__ __attribute__((aligned(16))) float v_s1[BN * D];
+
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int nqb = (S + 127) / 128;
+  const int zh = blockIdx.x % ZH;
+  const int qb = nqb - 1 - blockIdx.x / ZH;         // longest (last) query blocks first
+  const float* q_g = Q + (int64_t)zh * S * D;
+  const float* k_g = K + (int64_t)zh * Skv * D;
+  const float* v_g = V + (int64_t)zh * Skv * D;
+  const int q0 = qb * 128 + wave * 32;
+  const int r32 = lane % 32, kh = lane / 32;
+  const int qrow = q0 + r32;
+  const int qr = qrow < S ? qrow : S - 1;
+
+  // Q: chunk 2*dq + kh of the row: head dimensions 8*dq + 4*kh + e, the k slots of MFMA (dq, e)
+  f32x4a qf[DQ];
+#pragma unroll
+  for (int dq = 0; dq < DQ; ++dq)
+    qf[dq] = *reinterpret_cast<const f32x4a*>(q_g + (int64_t)qr * D + (2 * dq + kh) * 4);
+
+  f32x16 o_acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.0f;
+  float m_i = -INFINITY, l_i = 0.0f, neg_m = 0.0f;
+
+  const int key_end = CAUSAL ? ((qb + 1) * 128 < S ? (qb + 1) * 128 : S) : Skv;
+  const int n_steps = (key_end + BN - 1) / BN;
+
+  // ---- K / V tile copies
+  int row_c[NI], kcol[NI], vcol[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const int inst = j * 4 + wave;
+    row_c[j] = inst * RPI + lane / CPR;
+    const int pc = lane % CPR;
+    kcol[j] = (pc ^ (row_c[j] & 15)) * 4;
+    vcol[j] = (pc ^ (((row_c[j] >> 2) & 1) << 3)) * 4;
+  }
+  auto load_kv = [&](int step, float* k_dst, float* v_dst) __attribute__((always_inline)) {
+    const char* kb = reinterpret_cast<const char*>(k_g);
+    const char* vb = reinterpret_cast<const char*>(v_g);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      int key = step * BN + row_c[j];
+      key = key < Skv ? key : Skv - 1;                // rows past the end repeat the last key (masked below)
+      copy_to_lds(kb, (key * D + kcol[j]) * (int)sizeof(float), k_dst + (j * 4 + wave) * 256);
+      copy_to_lds(vb, (key * D + vcol[j]) * (int)sizeof(float), v_dst + (j * 4 + wave) * 256);
+    }
+  };
+
+  const float* mask_row = nullptr;
+  if constexpr (MASKED) mask_row = Mk + ((int64_t)zh * S + qr) * Skv;
+
+  auto process = [&](int step, const float* ks, const float* vs) __attribute__((always_inline)) {
+    const int n0 = step * BN;
+    if (CAUSAL && n0 > q0 + 31) return;               // wholly past this wave's rows (wave-uniform)
+    f32x4a mk[NT][4];
+    if constexpr (MASKED) {
+#pragma unroll
+      for (int jt = 0; jt < NT; ++jt)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          int key = n0 + jt * 32 + 8 * g4 + 4 * kh;
+          key = key + 4 <= Skv ? key : Skv - 4;       // past the end: any valid run, those scores are dropped
+          mk[jt][g4] = *reinterpret_cast<const f32x4a*>(mask_row + key);
+        }
+    }
+    // ---- scores: two accumulators per tile, so a chain never waits for its own previous MFMA (one when the mask
+    //      values already hold 16 registers per tile)
+    constexpr bool kDual = !MASKED;
+    f32x16 s[NT], s2[kDual ? NT : 1];
+#pragma unroll
+    for (int jt = 0; jt < NT; ++jt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        s[jt][r] = 0.0f;
+        if (kDual) s2[jt][r] = 0.0f;
+      }
+#pragma unroll
+    for (int dq = 0; dq < DQ; ++dq) {
+#pragma unroll
+      for (int jt = 0; jt < NT; ++jt) {
+        const int row = jt * 32 + r32;
+        const f32x4a kf = *reinterpret_cast<const f32x4a*>(ks + row * D + (((2 * dq + kh) ^ (row & 15)) * 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (!kDual || e % 2 == 0) s[jt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[dq][e], s[jt], 0, 0, 0);
+          else s2[jt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[dq][e], s2[jt], 0, 0, 0);
+        }
+      }
+    }
+    if constexpr (kDual) {
+#pragma unroll
+      for (int jt = 0; jt < NT; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[jt][r] += s2[jt][r];
+    }
+    if constexpr (MASKED) {
+      // softmax(scale*s + mask) = softmax(scale * (s + mask/scale))
+#pragma unroll
+      for (int jt = 0; jt < NT; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[jt][r] = fmaf(mk[jt][r / 4][r % 4], mask_factor, s[jt][r]);
+    }
+    const bool need_mask = (CAUSAL && n0 + BN - 1 > q0) || (n0 + BN > Skv);
+    if (need_mask) {
+#pragma unroll
+      for (int jt = 0; jt < NT; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = n0 + jt * 32 + 8 * (r / 4) + 4 * kh + r % 4;
+          if ((CAUSAL && key > qrow) || key >= Skv) s[jt][r] = -INFINITY;
+        }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int jt = 0; jt < NT; ++jt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[jt][r]);
+    mx = fmaxf(mx, other_half_f32(mx));
+    const float m_blk = mx * scale_log2e;
+    const bool grow = m_blk > m_i + kRescaleLagF32;
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float m_new = grow ? m_blk : m_i;
+      const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_new) : 1.0f;
+      l_i *= alpha;
+      m_i = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+      neg_m = m_i == -INFINITY ? 0.0f : -m_i;       // a row with every key masked so far: exp2(-inf) = 0, not NaN
+    }
+    // ---- O^T += V^T P^T: score register r of a lane is k slot r
+#pragma unroll
+    for (int jt = 0; jt < NT; ++jt) {
+      float p[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        p[r] = __builtin_amdgcn_exp2f(fmaf(s[jt][r], scale_log2e, neg_m));
+        l_i += p[r];
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = jt * 32 + 8 * (r / 4) + 4 * kh + r % 4;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const float vv = vs[key * D + ((dt * 32 + r32) ^ (kh << 5))];
+          o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, p[r], o_acc[dt], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  load_kv(0, k_s0, v_s0);
+  int step = 0;
+  for (; step + 1 < n_steps; step += 2) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    load_kv(step + 1, k_s1, v_s1);
+    process(step, k_s0, v_s0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (step + 2 < n_steps) load_kv(step + 2, k_s0, v_s0);
+    process(step + 1, k_s1, v_s1);
+  }
+  if (step < n_steps) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    process(step, k_s0, v_s0);
+  }
+
+  // ---- o_acc[dt][r] is O[qrow][dt*32 + 8*(r/4) + 4*kh + r%4] * l
+  const float l_tot = l_i + other_half_f32(l_i);
+  const float inv_l = 1.0f / l_tot;
+  if (qrow < S) {
+    float* o_row = O + ((int64_t)zh * S + qrow) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *reinterpret_cast<f32x4a*>(o_row + dt * 32 + 8 * q4 + 4 * kh) =
+            f32x4a{o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l, o_acc[dt][q4 * 4 + 2] * inv_l,
+                   o_acc[dt][q4 * 4 + 3] * inv_l};
+  }
+}
+
+template <int D, int BN>
+int launch(const float* Q, const float* K, const float* V, const float* mask, float* O, int64_t ZH, int64_t S,
+           int64_t Skv, float scale_log2e, bool causal, hipStream_t st) {
+  const int64_t blocks = (S + 127) / 128 * ZH;
+  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  const float mask_factor = mask ? 1.44269504088896340736f / scale_log2e : 0.0f;      // mask / sm_scale
+#define HEXMI_FA32(CZ, MK) \
+  hipLaunchKernelGGL((flash_fwd_f32_kernel<D, BN, CZ, MK>), dim3((unsigned)blocks), dim3(256), 0, st, Q, K, V, O, \
+                     (int)ZH, (int)S, (int)Skv, scale_log2e, mask, mask_factor)
+  if (mask) HEXMI_FA32(false, true);
+  else if (causal) HEXMI_FA32(true, false);
+  else HEXMI_FA32(false, false);
+#undef HEXMI_FA32
+  return launch_status();
+}
+
+}  // namespace
+
+// True (and the kernel launched, status in *status) for head sizes 64 and 128 with 16-byte aligned operands; a mask
+// needs whole 16-byte runs (Skv % 4 == 0) and excludes causal.
+bool flash_attn_f32_mfma(const float* Q, const float* K, const float* V, const float* mask, float* O, int64_t ZH,
+                         int64_t S, int64_t Skv, int64_t D, float scale_log2e, bool causal, hipStream_t st,
+                         int* status) {
+  if (D != 64 && D != 128) return false;
+  if (!aligned_to(Q, 16) || !aligned_to(K, 16) || !aligned_to(V, 16) || !aligned_to(O, 16)) return false;
+  if (Skv * D * (int64_t)sizeof(float) >= 0x7fffffff) return false;     // 32-bit byte offsets inside a head
+  if (causal && (mask || Skv != S)) return false;
+  if (mask && (Skv % 4 != 0 || Skv < 4 || !aligned_to(mask, 16) || scale_log2e == 0.0f)) return false;
+  *status = D == 64 ? launch<64, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, causal, st)
+                    : launch<128, 32>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, causal, st);
+  return true;
+}
+
+}  // namespace hexmi

@@ -54,7 +54,10 @@ def test_attention_parity_half(hexmi, oracle, case, dtype, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("case", [(1, 1, 1024, 64), (1, 2, 100, 128), (2, 2, 65, 32), (1, 1, 130, 80)])
+@pytest.mark.parametrize("case", [(1, 1, 1024, 64), (1, 2, 100, 128), (2, 2, 65, 32), (1, 1, 130, 80),
+                                  # head sizes 64 and 128 run on the fp32 matrix cores: ragged query and key blocks,
+                                  # several workgroups per head, a single row
+                                  (2, 3, 333, 64), (1, 2, 515, 128), (1, 1, 1, 64), (3, 1, 129, 128)])
 def test_attention_parity_fp32(hexmi, oracle, case, causal):
     # (1,1,1024,64) rand inputs, scale 0.5, non-causal is test_flash_attention.py:20-34,171-213
     Z, H, S, D = case
@@ -62,6 +65,21 @@ def test_attention_parity_fp32(hexmi, oracle, case, causal):
     got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), 0.5, causal).cpu()
     want = _oracle(oracle, q, k, v, 0.5, causal)
     assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("case", [(2, 8, 2048, 64), (1, 4, 1536 + 40, 128)])
+def test_attention_fp32_larger_and_randn(hexmi, case, causal):
+    # N(0,1) operands (scores of both signs, running maxima that move) at sizes with many key blocks. Oracle: the
+    # PyTorch CPU call the reference's test uses (test/python/triton/test_flash_attention.py:212), in float64.
+    Z, H, S, D = case
+    q, k, v = _qkv(Z, H, S, D, torch.float32, seed=11)
+    scale = 1.0 / math.sqrt(D)
+    got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal).cpu()
+    want = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double(), is_causal=causal,
+                                                            scale=scale)
+    assert got.dtype == torch.float32
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=2e-6)
 
 
 def test_reference_call_site(hexmi, oracle):
@@ -183,7 +201,9 @@ def test_masked_attention_parity_half(hexmi, oracle, case, dtype, with_mask):
     assert (got32 - want).abs().max() <= (5e-3 if dtype == torch.float16 else 3e-2)
 
 
-@pytest.mark.parametrize("case", [(2, 50, 70, 32), (1, 64, 64, 128), (1, 33, 129, 64)])
+@pytest.mark.parametrize("case", [(2, 50, 70, 32), (1, 64, 64, 128), (1, 33, 129, 64),
+                                  # Skv % 4 == 0 with head size 64 / 128: the fp32 matrix-core kernel with a mask
+                                  (2, 200, 72, 64), (1, 130, 516, 128), (3, 129, 1028, 64)])
 def test_masked_attention_parity_fp32(hexmi, oracle, case):
     B, Sq, Skv, D = case
     g = _gen(23)
