@@ -230,6 +230,191 @@ void flash_fwd_f32_kernel(const float* __restrict__ Q, const float* __restrict__
   }
 }
 
+// Small grids (fewer 128-row workgroups than half the CUs, e.g. the reference test's single head of 1024 rows):
+// a workgroup owns 32 query rows and its NW waves split the KEYS (wave w takes the w-th run of 32-key blocks), each
+// with its own double-buffered K / V tiles, so a wave waits only for its own copies and the loop has no barrier.
+// The NW partial results (m, l, O) of a row meet in LDS at the end. Four times (D = 64) or twice (D = 128) the
+// workgroups of the row-split kernel, each wave with a quarter or half of the keys.
+template <int D, int NW, bool CAUSAL>
+__global__ __launch_bounds__(NW * 64, 1)
+void flash_fwd_f32_split_kernel(const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
+                                float* __restrict__ O, int ZH, int S, float scale_log2e) {
+  constexpr int BN = 32, CPR = D / 4, DT = D / 32, DQ = D / 8;
+  constexpr int TILE = BN * D;                      // floats per K or V tile
+  constexpr int NI = BN * CPR / 64;                 // copy instructions per tile (one wave issues them all)
+  constexpr int RPI = 64 / CPR;
+  __shared__ __attribute__((aligned(16))) float stage[NW * 4 * TILE];   // [wave][buffer][K, V][TILE]: 128 KiB
+  __shared__ float m_s[NW][32], l_s[NW][32];
+
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int nqb = (S + 31) / 32;
+  const int zh = blockIdx.x % ZH;
+  const int qb = nqb - 1 - blockIdx.x / ZH;
+  const float* q_g = Q + (int64_t)zh * S * D;
+  const float* k_g = K + (int64_t)zh * S * D;
+  const float* v_g = V + (int64_t)zh * S * D;
+  const int q0 = qb * 32;
+  const int r32 = lane % 32, kh = lane / 32;
+  const int qrow = q0 + r32;
+  const int qr = qrow < S ? qrow : S - 1;
+
+  f32x4a qf[DQ];
+#pragma unroll
+  for (int dq = 0; dq < DQ; ++dq)
+    qf[dq] = *reinterpret_cast<const f32x4a*>(q_g + (int64_t)qr * D + (2 * dq + kh) * 4);
+  f32x16 o_acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.0f;
+  float m_i = -INFINITY, l_i = 0.0f, neg_m = 0.0f;
+
+  const int key_end = CAUSAL ? (q0 + 32 < S ? q0 + 32 : S) : S;
+  const int n_steps = (key_end + BN - 1) / BN;
+  const int per = (n_steps + NW - 1) / NW;
+  const int s_begin = wave * per;
+  const int s_end = s_begin + per < n_steps ? s_begin + per : n_steps;
+
+  int row_c[NI], kcol[NI], vcol[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    row_c[j] = j * RPI + lane / CPR;
+    const int pc = lane % CPR;
+    kcol[j] = (pc ^ (row_c[j] & 15)) * 4;
+    vcol[j] = (pc ^ (((row_c[j] >> 2) & 1) << 3)) * 4;
+  }
+  float* my = stage + wave * (4 * TILE);
+  auto load_kv = [&](int step, float* k_dst, float* v_dst) __attribute__((always_inline)) {
+    const char* kb = reinterpret_cast<const char*>(k_g);
+    const char* vb = reinterpret_cast<const char*>(v_g);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      int key = step * BN + row_c[j];
+      key = key < S ? key : S - 1;
+      // wave-private tiles at a run-time base: copies the compiler does not see, waits of our own (below)
+      copy_to_lds_asm(kb, (key * D + kcol[j]) * (int)sizeof(float), k_dst + j * 256);
+      copy_to_lds_asm(vb, (key * D + vcol[j]) * (int)sizeof(float), v_dst + j * 256);
+    }
+  };
+  auto process = [&](int step, const float* ks, const float* vs) __attribute__((always_inline)) {
+    const int n0 = step * BN;
+    f32x16 s, s2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s[r] = 0.0f; s2[r] = 0.0f; }
+#pragma unroll
+    for (int dq = 0; dq < DQ; ++dq) {
+      const f32x4a kf = *reinterpret_cast<const f32x4a*>(ks + r32 * D + (((2 * dq + kh) ^ (r32 & 15)) * 4));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (e % 2 == 0) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[dq][e], s, 0, 0, 0);
+        else s2 = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[dq][e], s2, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] += s2[r];
+    if ((CAUSAL && n0 + BN - 1 > q0) || n0 + BN > S) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = n0 + 8 * (r / 4) + 4 * kh + r % 4;
+        if ((CAUSAL && key > qrow) || key >= S) s[r] = -INFINITY;
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
+    mx = fmaxf(mx, other_half_f32(mx));
+    const float m_blk = mx * scale_log2e;
+    const bool grow = m_blk > m_i + kRescaleLagF32;
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float m_new = grow ? m_blk : m_i;
+      const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_new) : 1.0f;
+      l_i *= alpha;
+      m_i = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+      neg_m = m_i == -INFINITY ? 0.0f : -m_i;
+    }
+    float p[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2e, neg_m));
+      l_i += p[r];
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = 8 * (r / 4) + 4 * kh + r % 4;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const float vv = vs[key * D + ((dt * 32 + r32) ^ (kh << 5))];
+        o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, p[r], o_acc[dt], 0, 0, 0);
+      }
+    }
+  };
+
+  float* k0 = my, *v0 = my + TILE, *k1 = my + 2 * TILE, *v1 = my + 3 * TILE;
+  if (s_begin < s_end) load_kv(s_begin, k0, v0);
+  // Q has landed before the loop: left to the compiler, its wait (down to vmcnt(0)) would sit at Q's first use
+  // inside the loop and wait for the copies in flight as well, in every key block
+  __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0) only
+  int step = s_begin;
+  for (; step + 1 < s_end; step += 2) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    load_kv(step + 1, k1, v1);
+    process(step, k0, v0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (step + 2 < s_end) load_kv(step + 2, k0, v0);
+    process(step + 1, k1, v1);
+  }
+  if (step < s_end) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    process(step, k0, v0);
+  }
+
+  // ---- the NW partial results of a row meet in LDS: this wave's O (still times its own l) over its first tile
+  const float l_w = l_i + other_half_f32(l_i);
+  if (kh == 0) {
+    m_s[wave][r32] = m_i;
+    l_s[wave][r32] = l_w;
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4)
+      *reinterpret_cast<f32x4a*>(my + r32 * D + dt * 32 + 8 * q4 + 4 * kh) =
+          f32x4a{o_acc[dt][q4 * 4 + 0], o_acc[dt][q4 * 4 + 1], o_acc[dt][q4 * 4 + 2], o_acc[dt][q4 * 4 + 3]};
+  __syncthreads();
+  {
+    constexpr int TPR = NW * 2;                      // threads per row
+    constexpr int FPT = D / TPR;                     // floats per thread
+    const int q = threadIdx.x / TPR, part = threadIdx.x % TPR;
+    float m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) m = fmaxf(m, m_s[w][q]);
+    float sc[NW], l = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      sc[w] = m_s[w][q] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_s[w][q] - m);
+      l += l_s[w][q] * sc[w];
+    }
+    const float inv = 1.0f / l;
+    if (q0 + q < S) {
+      float* o_row = O + ((int64_t)zh * S + q0 + q) * D + part * FPT;
+#pragma unroll
+      for (int f = 0; f < FPT; f += 4) {
+        f32x4a acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+          const f32x4a v = *reinterpret_cast<const f32x4a*>(stage + w * (4 * TILE) + q * D + part * FPT + f);
+          acc += v * sc[w];
+        }
+        *reinterpret_cast<f32x4a*>(o_row + f) = acc * inv;
+      }
+    }
+  }
+}
+
 template <int D, int BN>
 int launch(const float* Q, const float* K, const float* V, const float* mask, float* O, int64_t ZH, int64_t S,
            int64_t Skv, float scale_log2e, bool causal, hipStream_t st) {
@@ -258,6 +443,20 @@ bool flash_attn_f32_mfma(const float* Q, const float* K, const float* V, const f
   if (Skv * D * (int64_t)sizeof(float) >= 0x7fffffff) return false;     // 32-bit byte offsets inside a head
   if (causal && (mask || Skv != S)) return false;
   if (mask && (Skv % 4 != 0 || Skv < 4 || !aligned_to(mask, 16) || scale_log2e == 0.0f)) return false;
+  const int cus = hexmi_num_cus();
+  const int64_t row_split_groups = (S + 127) / 128 * ZH;
+  if (!mask && Skv == S && row_split_groups * 2 < (cus > 0 ? cus : 256) && (S + 31) / 32 * ZH <= 0x7fffffff) {
+    // too few 128-row workgroups for the chip: 32-row workgroups whose waves split the keys
+    const unsigned blocks = (unsigned)((S + 31) / 32 * ZH);
+#define HEXMI_FA32S(DD, NWW, CZ) \
+  hipLaunchKernelGGL((flash_fwd_f32_split_kernel<DD, NWW, CZ>), dim3(blocks), dim3(NWW * 64), 0, st, Q, K, V, O, \
+                     (int)ZH, (int)S, scale_log2e)
+    if (D == 64) { if (causal) HEXMI_FA32S(64, 4, true); else HEXMI_FA32S(64, 4, false); }
+    else { if (causal) HEXMI_FA32S(128, 2, true); else HEXMI_FA32S(128, 2, false); }
+#undef HEXMI_FA32S
+    *status = launch_status();
+    return true;
+  }
   *status = D == 64 ? launch<64, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, causal, st)
                     : launch<128, 32>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, causal, st);
   return true;

@@ -128,6 +128,35 @@ __device__ __forceinline__ void copy_to_lds(const char* base, int voff, T* lds) 
 #endif
 }
 
+// copy_to_lds written as asm, for kernels whose LDS destination the compiler cannot name (a stage picked at run
+// time, a wave-private region at a run-time base): a copy into LDS with an unknown target makes the compiler wait
+// for ALL copies in flight (vmcnt(0)) before every later LDS read that might alias it. A kernel that uses this for
+// its copies does its own waiting (s_waitcnt vmcnt) before reading what they fill: the compiler does not know the
+// copies exist. Its own vmcnt waits for other loads only get stronger (the counter counts these copies too, and
+// loads complete in issue order). M0 (the LDS destination of such a copy) is saved and restored because the
+// compiler tracks its own uses of it. lds must be wave-uniform.
+template <typename T>
+__device__ __forceinline__ void copy_to_lds_asm(const char* base, int voff, T* lds) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef int i32x4_rsrc __attribute__((ext_vector_type(4)));
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  i32x4_rsrc rsrc;
+  rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+  rsrc[1] = __builtin_amdgcn_readfirstlane((int)((uint32_t)(b >> 32) & 0xffffu));
+  rsrc[2] = 0x7fffffff;
+  rsrc[3] = 0x00020000;
+  const uint32_t dst = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(lds)));
+  uint32_t saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %2, %3, 0 offen lds\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "s"(dst), "v"(voff), "s"(rsrc)
+      : "memory");
+#endif
+}
+
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 inline int dtype_size(int dtype) {
