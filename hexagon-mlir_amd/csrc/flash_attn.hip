@@ -12,7 +12,8 @@
 // Causal: key blocks past the diagonal are skipped, the diagonal blocks are masked element-wise, and workgroups
 // are numbered so the longest (last) query blocks start first.
 //
-// fp32 inputs take a plain one-wave-per-query-row kernel (no fp32 matrix-core path is needed by any caller).
+// fp32 inputs with head size 64 or 128 run the fp32 matrix-core kernels of flash_attn_f32.hip; other head sizes and
+// unaligned operands take the plain one-wave-per-query-row kernel below.
 #include "hexmi_common.h"
 
 namespace hexmi {
