@@ -439,7 +439,7 @@ def measure(torch, wl, steps, warmup, use_graph=True):
 PROFILE_KEYS = {"norms_f16_8192x4096": "norms", "softmax_f32_4096x1024": "softmax", "gemm_f16_4096": "gemm",
                 "gemm_bf16_8192": "gemm_bf16", "gemm_f32_4096": "gemm_f32", "w8a16_m1": "w8a16_m1", "w8a16_m16": "w8a16_m16",
                 "w8a16_m256": "w8a16_m256", "attn_causal_f16_4x32x4096x128": "attn",
-                "attn_causal_f16_1x32x16384x128": "attn_long", "attn_masked_f16_32x2048x128": "attn_masked"}
+                "attn_causal_f16_1x32x16384x128": "attn_long", "attn_masked_f16_32x2048x128": "attn_masked", "attn_causal_f32_4x32x2048x64": "attn_f32"}
 
 
 def measured_traffic(wl):
