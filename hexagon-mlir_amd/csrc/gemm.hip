@@ -638,10 +638,6 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
     if constexpr (B_I8) return read_i8row(src, (wn * TN + j) * 16 + lane % 16, lane / 16);
     else return u32x4{};
   };
-  auto mfma_row = [&](const Frag* af, const Frag* bf, int i) __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j) Mfma16<T>::run(bf[j], af[i], acc[i][j]);
-  };
   const int KT = K / BK2;
   auto clampj = [&](int j) { return j < KT ? j : KT - 1; };      // past the end: reload the last slab (never used)
 
