@@ -414,6 +414,9 @@ def binary(op, a, b, out=None):
     return _finish(od, out)
 
 
+_TWO_PASS_MIN_BLOCK, _TWO_PASS_RUN = 1 << 16, 4096
+
+
 def block_sum(x, block=None, out=None):
     """out[p] = sum of the p-th run of `block` elements of x (flattened); block=None sums everything into out[0]
     (`torch.sum(x)`, test/python/triton/test_sum.py:30-47)."""
@@ -426,7 +429,15 @@ def block_sum(x, block=None, out=None):
     dev = _device() if x.device.type != "cuda" else x.device
     xd = _stage(x, dev).reshape(-1)
     od = _out_like(out, (programs,), x.dtype, dev)
-    torch.ops.hexmi.block_sum(xd, int(block), od)
+    if x.dtype == torch.float32 and block >= _TWO_PASS_MIN_BLOCK and (programs == 1 or block % _TWO_PASS_RUN == 0):
+        # A program is one workgroup in the library (as it is one Triton program in the reference): a few huge
+        # programs - the reference test sums 2^20 elements in one - leave the chip idle. fp32 partial sums of runs
+        # of 4096 lose nothing, so they are formed by many workgroups first and summed per program afterwards.
+        parts = torch.empty((n + _TWO_PASS_RUN - 1) // _TWO_PASS_RUN, dtype=torch.float32, device=dev)
+        torch.ops.hexmi.block_sum(xd, _TWO_PASS_RUN, parts)
+        torch.ops.hexmi.block_sum(parts, parts.numel() if programs == 1 else block // _TWO_PASS_RUN, od)
+    else:
+        torch.ops.hexmi.block_sum(xd, int(block), od)
     return _finish(od, out)
 
 

@@ -137,6 +137,21 @@ def test_block_sum_parity(hexmi, oracle, dtype, n, block):
         assert close16(got, want, max_ulp=1, atol=4e-3 * max(1.0, block ** 0.5 / 64))
 
 
+@pytest.mark.parametrize("n,block", [(1 << 20, None), (300000, 131072), (1 << 21, 1 << 16), (70001, 70001)])
+def test_block_sum_large_fp32_programs(hexmi, n, block):
+    # fp32 programs of 2^16 elements and more are summed in two passes (runs of 4096 by many workgroups, then per
+    # program): same sums as one pass through the library and as float64 on the CPU, ragged tails included
+    x = torch.randn(n, generator=_gen(43))
+    got = hexmi.block_sum(x.cuda(), block).cpu()
+    b = n if block is None else block
+    want = torch.stack([x[i:i + b].double().sum() for i in range(0, n, b)])
+    assert got.shape == want.shape and got.dtype == torch.float32
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=2e-6 * b ** 0.5)
+    one_pass = torch.empty_like(got).cuda()
+    torch.ops.hexmi.block_sum(x.cuda(), b, one_pass)
+    assert torch.allclose(got, one_pass.cpu(), rtol=1e-5, atol=2e-6 * b ** 0.5)
+
+
 def test_reference_sum_call_site(hexmi):
     # test_sum.py:22-47: one program over 1024*1024 elements, atol 1e-2
     for dtype in (torch.float16, torch.float32):
