@@ -74,36 +74,42 @@ template <typename T, int D, bool IS_V, int NW = 4>
 struct KvTileLoader {
   static constexpr int CPR = D / 8;                       // chunks per row
   static constexpr int NI = kBlockN * CPR / 64 / NW;      // instructions per wave
-  int off[NI];                                            // element offset of this lane's chunk inside a tile
-  int row[NI];
-  int col[NI];
-  int lds_off[NI];
+  static constexpr int kRowsPerInst = 64 / CPR;           // rows one wave-wide instruction covers
+  static constexpr int kRowStep = NW * kRowsPerInst;      // rows between this wave's instructions j and j+1
+  // The swizzles repeat every 16 rows (32 for D = 64) and kRowStep is a multiple of that, so instruction j reads
+  // the lane's chunk of instruction 0 moved down by j*kRowStep rows: one offset, one row and one column per lane.
+  static_assert(kRowStep % (D == 128 ? 16 : 32) == 0, "swizzle period");
+  int off0;                                               // element offset of this lane's chunk inside a tile, j = 0
+  int row0, col0;
+  int lds_off0;
   __device__ __forceinline__ void init(int wave, int lane) {
-#pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      const int inst = j * NW + wave;
-      const int lin = inst * 64 + lane;
-      row[j] = lin / CPR;
-      col[j] = ((lin % CPR) ^ (IS_V ? swz_vtile<D>(row[j]) : swz_ktile<D>(row[j]))) * 8;
-      off[j] = row[j] * D + col[j];
-      lds_off[j] = inst * 64 * 8;
-    }
+    const int lin = wave * 64 + lane;
+    row0 = lin / CPR;
+    col0 = ((lin % CPR) ^ (IS_V ? swz_vtile<D>(row0) : swz_ktile<D>(row0))) * 8;
+    off0 = row0 * D + col0;
+    lds_off0 = wave * 64 * 8;
   }
-  __device__ __forceinline__ void issue(const T* __restrict__ g, int key0, int S, T* lds) const {
+  // instruction j of this wave's share of a tile that lies wholly inside the sequence
+  __device__ __forceinline__ void issue_one_whole(int j, const T* __restrict__ g, int key0, T* lds) const {
+    const char* base = reinterpret_cast<const char*>(g + ((int64_t)key0 + j * kRowStep) * D);
+    copy_to_lds(base, off0 * (int)sizeof(T), lds + lds_off0 + j * (NW * 64 * 8));
+  }
+  // instruction j of this wave's share of the tile
+  __device__ __forceinline__ void issue_one(int j, const T* __restrict__ g, int key0, int S, T* lds) const {
+    T* dst = lds + lds_off0 + j * (NW * 64 * 8);
     if (key0 + kBlockN <= S) {
-      const char* base = reinterpret_cast<const char*>(g + (int64_t)key0 * D);
-#pragma unroll
-      for (int j = 0; j < NI; ++j) copy_to_lds(base, off[j] * (int)sizeof(T), lds + lds_off[j]);
+      issue_one_whole(j, g, key0, lds);
     } else {
       // ragged last tile: rows clamped to the last key, offsets from the head's first key (S*D*sizeof(T) < 2^31)
       const char* base = reinterpret_cast<const char*>(g);
-#pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        int key = key0 + row[j];
-        key = key < S ? key : S - 1;
-        copy_to_lds(base, (key * D + col[j]) * (int)sizeof(T), lds + lds_off[j]);
-      }
+      int key = key0 + row0 + j * kRowStep;
+      key = key < S ? key : S - 1;
+      copy_to_lds(base, (key * D + col0) * (int)sizeof(T), dst);
     }
+  }
+  __device__ __forceinline__ void issue(const T* __restrict__ g, int key0, int S, T* lds) const {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) issue_one(j, g, key0, S, lds);
   }
 };
 
@@ -126,14 +132,15 @@ struct MaskTileLoader {
     col0 = ((lane % 8) ^ ((lane / 16) & 7)) * 8;            // swizzle (row/2)%8 = (lane/16 + 4*(j%2)) % 8
   }
   // mask_wg: the mask row of the workgroup's first query; lds: this wave's [32][64] tile of the stage
-  __device__ __forceinline__ void issue(const T* __restrict__ mask_wg, int key0, int Skv, T* lds) const {
+  __device__ __forceinline__ void issue_one(int j, const T* __restrict__ mask_wg, int key0, int Skv, T* lds) const {
     const char* base = reinterpret_cast<const char*>(mask_wg);
+    int key = key0 + (col0 ^ ((j & 1) * 32));
+    key = key + 8 <= Skv ? key : Skv - 8;
+    copy_to_lds(base, (rowoff[j] + key) * (int)sizeof(T), lds + j * 512);
+  }
+  __device__ __forceinline__ void issue(const T* __restrict__ mask_wg, int key0, int Skv, T* lds) const {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int key = key0 + (col0 ^ ((j & 1) * 32));
-      key = key + 8 <= Skv ? key : Skv - 8;
-      copy_to_lds(base, (rowoff[j] + key) * (int)sizeof(T), lds + j * 512);
-    }
+    for (int j = 0; j < 4; ++j) issue_one(j, mask_wg, key0, Skv, lds);
   }
 };
 
@@ -257,6 +264,15 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       v_loader.issue(v_g, step * kBlockN, Skv, v_dst);
       if constexpr (MASK_LDS) m_loader.issue(mask_wg, step * kBlockN, Skv, m_dst + wave * (32 * kBlockN));
     };
+    // The same copies one instruction at a time (c = 0 .. kCopies-1: K, then V, then the mask), for issuing
+    // them between the score MFMAs of the block before. Whole tiles only: a ragged last tile is copied by load_kv.
+    constexpr int kNI = KvTileLoader<T, D, false, NW>::NI;
+    constexpr int kCopies = 2 * kNI + (MASK_LDS ? 4 : 0);
+    auto load_one = [&](int c, int step, T* k_dst, T* v_dst, T* m_dst) __attribute__((always_inline)) {
+      if (c < kNI) k_loader.issue_one_whole(c, k_g, step * kBlockN, k_dst);
+      else if (c < 2 * kNI) v_loader.issue_one_whole(c - kNI, v_g, step * kBlockN, v_dst);
+      else if constexpr (MASK_LDS) m_loader.issue_one(c - 2 * kNI, mask_wg, step * kBlockN, Skv, m_dst + wave * (32 * kBlockN));
+    };
 
     // Online softmax of one 64-key block (two 32-key score tiles): mask, row max, (rare) rescale; the exponentials
     // follow per tile (exp_tile). The reference maximum m_i may lag the true running maximum by up to kRescaleLag
@@ -348,10 +364,17 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       if (Mk) mask_row = Mk + ((int64_t)zh * S + (qrow < S ? qrow : S - 1)) * Skv;
     }
 
-    auto process = [&](int step, const T* k_src, const T* v_src, const T* m_src) __attribute__((always_inline)) {
+    // One key block. The global -> LDS copies of the next block (next >= 0, into the other stage) are issued a
+    // few at a time between the score MFMAs: issued in one burst after the barrier, the 32 KiB of a block keep the
+    // CU's vector memory pipe busy for about 500 cycles, during which every wave sits in its copy instructions
+    // and the matrix cores have nothing queued.
+    auto process = [&](int step, const T* k_src, const T* v_src, const T* m_src, int next, T* k_dst, T* v_dst,
+                       T* m_dst) __attribute__((always_inline)) {
       const int n0 = step * kBlockN;
       // causal: a key block wholly past this wave's 32 rows contributes nothing (wave-uniform; the workgroup's
-      // barriers and copies are outside)
+      // barriers are outside)
+      const bool spread = next >= 0 && (next + 1) * kBlockN <= Skv && !(CAUSAL && n0 > q0 + 31);
+      if (next >= 0 && !spread) load_kv(next, k_dst, v_dst, m_dst);
       if (CAUSAL && n0 > q0 + 31) return;
       // mask values of this lane's 32 scores: four runs of four consecutive keys per 32-key tile
       typedef T MaskRun __attribute__((ext_vector_type(4)));
@@ -398,6 +421,11 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
           }
           s[0] = MfmaT<T>::run(kf[0][ds], qf[ds], s[0]);
           s[1] = MfmaT<T>::run(kf[1][ds], qf[ds], s[1]);
+          if (spread) {
+#pragma unroll
+            for (int c = 0; c < kCopies; ++c)
+              if (c * DS / kCopies == ds) load_one(c, next, k_dst, v_dst, m_dst);
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -442,17 +470,15 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     for (; step + 1 < n_steps; step += 2) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      load_kv(step + 1, k_lds1, v_lds1, m_lds1);
-      process(step, k_lds0, v_lds0, m_lds0);
+      process(step, k_lds0, v_lds0, m_lds0, step + 1, k_lds1, v_lds1, m_lds1);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (step + 2 < n_steps) load_kv(step + 2, k_lds0, v_lds0, m_lds0);
-      process(step + 1, k_lds1, v_lds1, m_lds1);
+      process(step + 1, k_lds1, v_lds1, m_lds1, step + 2 < n_steps ? step + 2 : -1, k_lds0, v_lds0, m_lds0);
     }
     if (step < n_steps) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      process(step, k_lds0, v_lds0, m_lds0);
+      process(step, k_lds0, v_lds0, m_lds0, -1, k_lds1, v_lds1, m_lds1);
     }
 
     // ---- epilogue: o_acc[dt][r] is O[qrow][dt*32 + 8*(r/4) + 4*half + r%4] * l
