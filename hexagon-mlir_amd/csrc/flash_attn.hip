@@ -177,7 +177,7 @@ template <> __device__ __forceinline__ void store4o<bf16>(bf16* p, float a, floa
 // like K and V (no registers, whole 128-byte rows), instead of being loaded into registers in 8-byte runs at the
 // top of the block that uses them.
 template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, int NW = 4, bool MASK_LDS = false>
-__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1)
+__global__ __launch_bounds__(NW * 64, NW == 4 ? (D == 64 && !GENERAL ? 3 : 2) : 1)
 void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                       OutT* __restrict__ O, int ZH, int S, float scale_log2e, const T* __restrict__ Mk = nullptr,
                       int Skv_arg = 0, float mask_factor = 0.0f) {
@@ -564,11 +564,11 @@ inline int64_t resident_grid(int64_t units, int per_cu) {
 
 template <typename T, typename OutT, int D, bool CAUSAL, int NW>
 int launch_mfma_nw(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
-                   hipStream_t st) {
+                   hipStream_t st, int per_cu = NW == 4 ? 2 : 1) {
   const int64_t nqb = (S + NW * 32 - 1) / (NW * 32);
   const int64_t units = nqb * ZH;
   if (units > 0x7fffffff) return HEXMI_ENOTSUP;
-  const int64_t blocks = resident_grid(units, NW == 4 ? 2 : 1);
+  const int64_t blocks = resident_grid(units, per_cu);
   if (blocks <= 0) return HEXMI_ELAUNCH;
   hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, CAUSAL, false, NW>), dim3((unsigned)blocks), dim3(NW * 64), 0, st,
                      static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
@@ -582,6 +582,13 @@ int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH
   // 256-row workgroups halve the L2 -> LDS copy traffic (1-9 % faster from 2048 keys on), if there are enough of
   // them to fill the chip; smaller problems keep the larger number of 128-row workgroups
   const bool wide = S >= kWideMinS && ZH * ((S + 255) / 256) >= hexmi_num_cus();
+  // D = 64 leaves room for three 128-row workgroups per CU (144-154 registers): 6-9 % faster than the 256-row ones
+  // between 2048 and 4095 keys when every workgroup still gets two units or more; fewer units balance better two per CU
+  const bool three = D == 64 && S >= kWideMinS && S < 4096 && ZH * ((S + 127) / 128) >= 6 * (int64_t)hexmi_num_cus();
+  if (three) {
+    if (causal) return launch_mfma_nw<T, OutT, D, true, 4>(Q, K, V, O, ZH, S, scale_log2e, st, 3);
+    return launch_mfma_nw<T, OutT, D, false, 4>(Q, K, V, O, ZH, S, scale_log2e, st, 3);
+  }
   if (causal) {
     if (wide) return launch_mfma_nw<T, OutT, D, true, 8>(Q, K, V, O, ZH, S, scale_log2e, st);
     return launch_mfma_nw<T, OutT, D, true, 4>(Q, K, V, O, ZH, S, scale_log2e, st);

@@ -297,6 +297,21 @@ def test_attention_256_row_workgroups(hexmi, case, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("case", [(2, 52, 2048, torch.float16), (1, 100, 2048 + 40, torch.bfloat16)])
+def test_attention_three_workgroups_per_cu(hexmi, case, causal):
+    # D = 64 between 2048 and 4095 keys with six or more 128-row units per CU runs three 128-row workgroups per CU
+    # (a persistent grid of 768): head counts off the XCD multiple, a ragged length, both dtypes. Oracle: the
+    # PyTorch CPU call the reference's test uses (test/python/triton/test_flash_attention.py:212).
+    Z, H, S, dtype = case
+    q, k, v = _qkv(Z, H, S, 64, dtype, seed=13)
+    scale = 1.0 / math.sqrt(64)
+    got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal, out_dtype=torch.float32).cpu()
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal,
+                                                            scale=scale)
+    assert (got - want).abs().max() <= (5e-3 if dtype == torch.float16 else 3e-2)
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("case", [(2, 36, 1280, 64), (1, 72, 1024, 128), (5, 13, 777, 128)])
 def test_attention_more_units_than_resident_workgroups(hexmi, case, causal):
     # more (head, query block) units than the persistent grid holds, head counts that are and are not multiples of
