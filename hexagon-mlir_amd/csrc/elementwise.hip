@@ -135,9 +135,10 @@ void binary_scalar_kernel(const T* __restrict__ a, const T* __restrict__ b, T* _
 // order (per-thread strided partials, wave butterfly, waves in order): the result does not depend on timing.
 // kSumThreads threads per program: 1024 for large blocks (a single program must pull its block through one CU),
 // 256 for blocks up to 64 KiB (several 16-byte loads in flight per thread, a cheaper final exchange).
-template <typename T, int kSumThreads>
+// TIn / TOut differ in the two-pass form below: fp32 partial sums of 16-bit inputs, a 16-bit result of fp32 partials.
+template <typename T, typename TOut, int kSumThreads>
 __global__ __launch_bounds__(kSumThreads)
-void block_sum_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t block, int64_t n) {
+void block_sum_kernel(const T* __restrict__ x, TOut* __restrict__ out, int64_t block, int64_t n) {
   constexpr int N = Chunk<T>::N;
   __shared__ float part[kSumThreads / kWave];
   const int64_t begin = (int64_t)blockIdx.x * block;
@@ -170,10 +171,15 @@ void block_sum_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t bloc
     float t = 0.0f;
 #pragma unroll
     for (int w = 0; w < kSumThreads / kWave; ++w) t += part[w];
-    out[blockIdx.x] = from_f32<T>(t);
+    out[blockIdx.x] = from_f32<TOut>(t);
   }
 }
 
+// A program is one workgroup (as it is one Triton program in the reference), so a launch of a few huge programs -
+// the reference test sums 2^20 elements in ONE - would leave the chip idle. Programs of kTwoPassMinBlock elements
+// and more are therefore summed in two passes when a scratch buffer is at hand: fp32 partial sums of runs of
+// kSumRun elements by many workgroups (the runs of a program are whole when block % kSumRun == 0 or there is one
+// program), then one sum per program over its partials. fp32 partials lose nothing for any input type.
 // ---- rotary embedding ----------------------------------------------------------------------------------------
 // x, y: [batch, seq, heads, feat] contiguous; features are rotated in adjacent pairs (2i, 2i+1) by the angle
 // m * theta^(-2i/feat), m the sequence position (test/python/triton/test_rope.py:43-57 compute_thetas,
@@ -301,17 +307,27 @@ int dispatch_binary(int op, const void* a, const void* b, void* y, int64_t n, hi
   }
 }
 
-template <typename T>
-int launch_block_sum(const void* x, void* out, int64_t n, int64_t block, hipStream_t s) {
+template <typename T, typename TOut>
+int launch_block_sum_pass(const T* x, TOut* out, int64_t n, int64_t block, hipStream_t s) {
   const int64_t programs = (n + block - 1) / block;
   if (programs > 0x7fffffff) return HEXMI_ENOTSUP;
   if (block * (int64_t)sizeof(T) <= 65536)
-    hipLaunchKernelGGL((block_sum_kernel<T, 256>), dim3((unsigned)programs), dim3(256), 0, s,
-                       static_cast<const T*>(x), static_cast<T*>(out), block, n);
+    hipLaunchKernelGGL((block_sum_kernel<T, TOut, 256>), dim3((unsigned)programs), dim3(256), 0, s, x, out, block, n);
   else
-    hipLaunchKernelGGL((block_sum_kernel<T, 1024>), dim3((unsigned)programs), dim3(1024), 0, s,
-                       static_cast<const T*>(x), static_cast<T*>(out), block, n);
+    hipLaunchKernelGGL((block_sum_kernel<T, TOut, 1024>), dim3((unsigned)programs), dim3(1024), 0, s, x, out, block, n);
   return launch_status();
+}
+
+// partials == nullptr: one pass. Otherwise partials holds at least ceil(n / kSumRun) floats and two_pass_sum(n, block).
+template <typename T>
+int launch_block_sum(const void* xv, void* outv, int64_t n, int64_t block, float* partials, hipStream_t s) {
+  const T* x = static_cast<const T*>(xv);
+  T* out = static_cast<T*>(outv);
+  if (!partials) return launch_block_sum_pass<T, T>(x, out, n, block, s);
+  const int64_t runs = (n + kSumRun - 1) / kSumRun;
+  const int rc = launch_block_sum_pass<T, float>(x, partials, n, kSumRun, s);
+  if (rc != HEXMI_OK) return rc;
+  return launch_block_sum_pass<float, T>(partials, out, runs, block >= n ? runs : block / kSumRun, s);
 }
 
 template <typename T>
@@ -340,6 +356,16 @@ int launch_rope(const void* xv, void* yv, int64_t batch, int64_t seq, int64_t he
 }
 
 }  // namespace
+
+int block_sum_any(const void* x, void* out, int64_t n, int64_t block, int dtype, float* partials, hipStream_t s) {
+  switch (dtype) {
+    case HEXMI_F32: return launch_block_sum<float>(x, out, n, block, partials, s);
+    case HEXMI_F16: return launch_block_sum<f16>(x, out, n, block, partials, s);
+    case HEXMI_BF16: return launch_block_sum<bf16>(x, out, n, block, partials, s);
+    default: return HEXMI_ENOTSUP;
+  }
+}
+
 }  // namespace hexmi
 
 using namespace hexmi;
@@ -349,6 +375,7 @@ extern "C" int hexmi_unary(int op, const void* x, void* y, int64_t n, int dtype,
   if (n == 0) return HEXMI_OK;
   if (!x || !y) return HEXMI_EINVAL;
   hipStream_t s = as_stream(stream);
+  begin_call();
   switch (dtype) {
     case HEXMI_F32: return dispatch_unary<float>(op, x, y, n, s);
     case HEXMI_F16: return dispatch_unary<f16>(op, x, y, n, s);
@@ -363,6 +390,7 @@ extern "C" int hexmi_binary(int op, const void* a, const void* b, void* y, int64
   if (n == 0) return HEXMI_OK;
   if (!a || !b || !y) return HEXMI_EINVAL;
   hipStream_t s = as_stream(stream);
+  begin_call();
   switch (dtype) {
     case HEXMI_F32: return dispatch_binary<float>(op, a, b, y, n, s);
     case HEXMI_F16: return dispatch_binary<f16>(op, a, b, y, n, s);
@@ -373,16 +401,27 @@ extern "C" int hexmi_binary(int op, const void* a, const void* b, void* y, int64
 
 extern "C" int hexmi_block_sum(const void* x, void* out, int64_t n, int64_t block, int dtype,
                                hexmi_stream_t stream) {
-  if (n < 0 || block <= 0) return HEXMI_EINVAL;
+  return hexmi_block_sum_ws(x, out, n, block, dtype, nullptr, 0, stream);
+}
+
+extern "C" int64_t hexmi_block_sum_workspace(int64_t n, int64_t block, int dtype) {
+  (void)dtype;
+  if (n <= 0 || block <= 0 || !two_pass_sum(n, block)) return 0;
+  return (n + kSumRun - 1) / kSumRun * (int64_t)sizeof(float);
+}
+
+extern "C" int hexmi_block_sum_ws(const void* x, void* out, int64_t n, int64_t block, int dtype, void* workspace,
+                                  int64_t workspace_bytes, hexmi_stream_t stream) {
+  if (n < 0 || block <= 0 || workspace_bytes < 0) return HEXMI_EINVAL;
   if (n == 0) return HEXMI_OK;
   if (!x || !out) return HEXMI_EINVAL;
-  hipStream_t s = as_stream(stream);
-  switch (dtype) {
-    case HEXMI_F32: return launch_block_sum<float>(x, out, n, block, s);
-    case HEXMI_F16: return launch_block_sum<f16>(x, out, n, block, s);
-    case HEXMI_BF16: return launch_block_sum<bf16>(x, out, n, block, s);
-    default: return HEXMI_ENOTSUP;
+  float* partials = nullptr;
+  if (workspace && two_pass_sum(n, block)) {
+    if (workspace_bytes < hexmi_block_sum_workspace(n, block, dtype) || !aligned_to(workspace, 4)) return HEXMI_EINVAL;
+    partials = static_cast<float*>(workspace);
   }
+  begin_call();
+  return block_sum_any(x, out, n, block, dtype, partials, as_stream(stream));
 }
 
 extern "C" int hexmi_rope(const void* x, void* y, int64_t batch, int64_t seq, int64_t heads, int64_t feat,
@@ -392,6 +431,7 @@ extern "C" int hexmi_rope(const void* x, void* y, int64_t batch, int64_t seq, in
   if (!x || !y) return HEXMI_EINVAL;
   if (batch > 0x7fffffff || seq > 0x7fffffff || heads > 0x7fffffff || feat > 0x7fffffff) return HEXMI_ENOTSUP;
   hipStream_t s = as_stream(stream);
+  begin_call();
   switch (dtype) {
     case HEXMI_F32: return launch_rope<float>(x, y, batch, seq, heads, feat, theta, s);
     case HEXMI_F16: return launch_rope<f16>(x, y, batch, seq, heads, feat, theta, s);

@@ -499,7 +499,7 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   }
 }
 
-// fp32 (or any dtype / head size <= 256): one wave per query row; lanes take keys lane, lane+64, ...; each lane
+// fp32 (or any dtype / head size <= DMAX): one wave per query row; lanes take keys lane, lane+64, ...; each lane
 // keeps its own (m, l, o[D]) and the 64 partial states are merged at the end.
 template <typename T, typename OutT, int DMAX>
 __global__ __launch_bounds__(256)
@@ -631,11 +631,17 @@ int launch_rowwise(const void* Q, const void* K, const void* V, const void* mask
                    int64_t Skv, int64_t D, float scale_log2e, bool causal, hipStream_t st) {
   const int64_t rows = ZH * S;
   const int64_t blocks = (rows + 3) / 4;
-  if (blocks > 0x7fffffff || D > 128) return HEXMI_ENOTSUP;
-  hipLaunchKernelGGL((flash_fwd_rowwise<T, OutT, 128>), dim3((unsigned)blocks), dim3(256), 0, st,
-                     static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
-                     static_cast<OutT*>(O), rows, (int)S, (int)D, scale_log2e, causal ? 1 : 0,
-                     static_cast<const T*>(mask), (int)Skv);
+  if (blocks > 0x7fffffff || D > 256) return HEXMI_ENOTSUP;
+  if (D <= 128)
+    hipLaunchKernelGGL((flash_fwd_rowwise<T, OutT, 128>), dim3((unsigned)blocks), dim3(256), 0, st,
+                       static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                       static_cast<OutT*>(O), rows, (int)S, (int)D, scale_log2e, causal ? 1 : 0,
+                       static_cast<const T*>(mask), (int)Skv);
+  else                                                    // 256 output registers per lane: one wave per SIMD
+    hipLaunchKernelGGL((flash_fwd_rowwise<T, OutT, 256>), dim3((unsigned)blocks), dim3(256), 0, st,
+                       static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                       static_cast<OutT*>(O), rows, (int)S, (int)D, scale_log2e, causal ? 1 : 0,
+                       static_cast<const T*>(mask), (int)Skv);
   return launch_status();
 }
 
@@ -644,12 +650,14 @@ template <typename T, typename OutT>
 int dispatch_half(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
                   int64_t Skv, int64_t D, float scale_log2e, bool causal, hipStream_t st) {
   // the matrix-core kernels address a head's keys with 32-bit byte offsets
+  // and take the row maximum of the raw scores before scaling them, which is the maximum of the scaled scores only
+  // for a positive scale: zero and negative scales go to the row-wise kernel, which scales first
   const bool ok = aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16) &&
-                  Skv * D * (int64_t)sizeof(T) < 0x7fffffff;
+                  Skv * D * (int64_t)sizeof(T) < 0x7fffffff && scale_log2e > 0.0f;
   const bool plain = !mask && Skv == S;
   if (ok && plain && D == 128) return launch_mfma<T, OutT, 128>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
   if (ok && plain && D == 64) return launch_mfma<T, OutT, 64>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
-  const bool general_ok = ok && !causal && Skv % 4 == 0 && Skv >= 4 && scale_log2e != 0.0f && (!mask || aligned_to(mask, 8));
+  const bool general_ok = ok && !causal && Skv % 4 == 0 && Skv >= 4 && (!mask || aligned_to(mask, 8));
   if (general_ok && D == 128) return launch_mfma_general<T, OutT, 128>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
   if (general_ok && D == 64) return launch_mfma_general<T, OutT, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
   return launch_rowwise<T, OutT>(Q, K, V, mask, O, ZH, S, Skv, D, scale_log2e, causal, st);
@@ -684,6 +692,7 @@ extern "C" int hexmi_flash_attn_fwd(const void* Q, const void* K, const void* V,
   if (Z == 0 || H == 0 || S == 0 || D == 0) return HEXMI_OK;
   if (!Q || !K || !V || !O) return HEXMI_EINVAL;
   if (S > 0x7fffffff / 2 || Z * H > 0x7fffffff) return HEXMI_ENOTSUP;
+  begin_call();
   return attention_any(Q, K, V, nullptr, O, Z * H, S, S, D, sm_scale, causal != 0, in_dtype, out_dtype,
                        as_stream(stream));
 }
@@ -696,6 +705,7 @@ extern "C" int hexmi_attention(const void* Q, const void* K, const void* V, cons
   if (seq_kv == 0) return HEXMI_EINVAL;                    // a softmax over no keys is undefined
   if (!Q || !K || !V || !O) return HEXMI_EINVAL;
   if (seq_q > 0x7fffffff / 2 || seq_kv > 0x7fffffff / 2 || batch > 0x7fffffff) return HEXMI_ENOTSUP;
+  begin_call();
   return attention_any(Q, K, V, mask, O, batch, seq_q, seq_kv, head_dim, sm_scale, false, in_dtype, out_dtype,
                        as_stream(stream));
 }

@@ -439,10 +439,12 @@ bool flash_attn_f32_mfma(const float* Q, const float* K, const float* V, const f
                          int64_t S, int64_t Skv, int64_t D, float scale_log2e, bool causal, hipStream_t st,
                          int* status) {
   if (D != 64 && D != 128) return false;
+  // the row maximum is taken on the raw scores and scaled afterwards: right for a positive scale only
+  if (!(scale_log2e > 0.0f)) return false;
   if (!aligned_to(Q, 16) || !aligned_to(K, 16) || !aligned_to(V, 16) || !aligned_to(O, 16)) return false;
   if (Skv * D * (int64_t)sizeof(float) >= 0x7fffffff) return false;     // 32-bit byte offsets inside a head
   if (causal && (mask || Skv != S)) return false;
-  if (mask && (Skv % 4 != 0 || Skv < 4 || !aligned_to(mask, 16) || scale_log2e == 0.0f)) return false;
+  if (mask && (Skv % 4 != 0 || Skv < 4 || !aligned_to(mask, 16))) return false;
   const int cus = hexmi_num_cus();
   const int64_t row_split_groups = (S + 127) / 128 * ZH;
   if (!mask && Skv == S && row_split_groups * 2 < (cus > 0 ? cus : 256) && (S + 31) / 32 * ZH <= 0x7fffffff) {

@@ -1035,7 +1035,24 @@ int launch_w8a16(const f16* A, const int8_t* W, const f16* scales, f16* C, int64
   return launch_status();
 }
 
+// one thread per element: only ever used for the result of a product over an empty inner dimension
+__global__ __launch_bounds__(256)
+void fill_zero_kernel(char* __restrict__ C, int64_t rows, int64_t cols, int64_t ld, int elem_size) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * cols) return;
+  char* p = C + ((i / cols) * ld + i % cols) * elem_size;
+  for (int b = 0; b < elem_size; ++b) p[b] = 0;
+}
+
 }  // namespace
+
+int fill_zero_2d(void* C, int64_t rows, int64_t cols, int64_t ld, int elem_size, hipStream_t stream) {
+  const int64_t blocks = (rows * cols + 255) / 256;
+  if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, static_cast<char*>(C), rows, cols,
+                     ld, elem_size);
+  return launch_status();
+}
 
 // K % 32 == 0, N % 8 == 0, 16-byte aligned A / W / C / scales (checked by the caller).
 int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,
@@ -1053,11 +1070,17 @@ extern "C" int hexmi_gemm(int64_t M, int64_t N, int64_t K, const void* A, int64_
                           void* C, int64_t ldc, int in_dtype, int out_dtype, int trans_b, hexmi_stream_t stream) {
   if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
   if (M == 0 || N == 0) return HEXMI_OK;
-  if (!A || !B || !C) return HEXMI_EINVAL;
+  if (!C || (K > 0 && (!A || !B))) return HEXMI_EINVAL;
   if (lda < K || ldc < N || ldb < (trans_b ? K : N)) return HEXMI_EINVAL;
   if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return HEXMI_ENOTSUP;
-  if (K == 0) return HEXMI_ENOTSUP;
   hipStream_t s = as_stream(stream);
+  begin_call();
+  if (K == 0) {                                              // an empty sum: C = 0, as torch.matmul gives
+    const int esz = dtype_size(out_dtype);
+    const bool known = (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) ||
+                       ((in_dtype == HEXMI_F16 || in_dtype == HEXMI_BF16) && (out_dtype == in_dtype || out_dtype == HEXMI_F32));
+    return known ? fill_zero_2d(C, M, N, ldc, esz, s) : HEXMI_ENOTSUP;
+  }
   const bool tb = trans_b != 0;
   if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) return launch_f32(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
   if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F16) return dispatch_trans<f16, f16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);

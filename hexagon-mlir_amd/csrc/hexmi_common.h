@@ -111,9 +111,18 @@ __device__ __forceinline__ void cvt16(const u32x4& w, f16x8& f0, f16x8& f1) {
 // ---- host helpers ---------------------------------------------------------
 inline hipStream_t as_stream(hexmi_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
+// Every entry point calls begin_call() once its arguments are accepted and before its first launch: HIP keeps one
+// pending error per host thread, and one left there by unrelated code would otherwise be reported (and cleared) by
+// the launch_status() of the next launch here.
+inline void begin_call() { (void)hipGetLastError(); }
+
 inline int launch_status() {
   return hipGetLastError() == hipSuccess ? HEXMI_OK : HEXMI_ELAUNCH;
 }
+
+// C[rows, cols] = 0 with leading dimension ld (elements of elem_size bytes): what a product over an empty inner
+// dimension is (gemm.hip).
+int fill_zero_2d(void* C, int64_t rows, int64_t cols, int64_t ld, int elem_size, hipStream_t stream);
 
 // 16 bytes per lane, global -> LDS, as a buffer load: the address is a uniform base (a buffer descriptor in scalar
 // registers, built by scalar arithmetic) plus a per-lane 32-bit byte offset, and the LDS destination (lds + lane*16
@@ -167,6 +176,18 @@ inline int dtype_size(int dtype) {
     default: return 0;
   }
 }
+
+// Block sums (elementwise.hip). A program of kTwoPassMinBlock elements and more is summed in two passes when a
+// scratch buffer for fp32 partial sums of runs of kSumRun elements is at hand (ceil(n / kSumRun) floats): the runs of
+// a program must be whole, which they are when block % kSumRun == 0 or there is a single program.
+constexpr int64_t kSumRun = 4096;
+constexpr int64_t kTwoPassMinBlock = 1 << 16;
+inline bool two_pass_sum(int64_t n, int64_t block) {
+  const int64_t programs = (n + block - 1) / block;
+  return block >= kTwoPassMinBlock && (programs == 1 || block % kSumRun == 0);
+}
+// partials == nullptr: one pass; otherwise two_pass_sum(n, block) holds and partials has room for every run.
+int block_sum_any(const void* x, void* out, int64_t n, int64_t block, int dtype, float* partials, hipStream_t s);
 
 // Tiled W8A16 GEMM for many activation rows (gemm.hip): C[M,N] = (A[M,K] * W[N,K]^T) * scales[N].
 int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,

@@ -9,6 +9,7 @@ extern "C" const char* hexmi_strerror(int status) {
     case HEXMI_EINVAL: return "invalid argument (null pointer, negative size, bad leading dimension or alignment)";
     case HEXMI_ENOTSUP: return "unsupported dtype or shape";
     case HEXMI_ELAUNCH: return "HIP launch failed";
+    case HEXMI_ETOOBIG: return "size exceeds the fixed capacity of this entry point";
     default: return "unknown status";
   }
 }

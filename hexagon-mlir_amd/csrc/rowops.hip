@@ -386,6 +386,7 @@ extern "C" int hexmi_softmax(const void* x, void* y, int64_t rows, int64_t cols,
   if (rows < 0 || cols < 0 || ld_x < cols || ld_y < cols) return HEXMI_EINVAL;
   if (rows == 0 || cols == 0) return HEXMI_OK;
   if (!x || !y) return HEXMI_EINVAL;
+  begin_call();
   return dispatch_dtype<kSoftmax>(dtype, x, y, nullptr, nullptr, nullptr, nullptr, rows, cols, ld_x, ld_y, 0.0f,
                                   as_stream(stream));
 }
@@ -395,6 +396,7 @@ extern "C" int hexmi_rms_norm(const void* x, const void* weight, void* y, int64_
   if (rows < 0 || cols < 0) return HEXMI_EINVAL;
   if (rows == 0 || cols == 0) return HEXMI_OK;
   if (!x || !y) return HEXMI_EINVAL;
+  begin_call();
   return dispatch_dtype<kRmsNorm>(dtype, x, y, weight, nullptr, nullptr, nullptr, rows, cols, cols, cols, eps,
                                   as_stream(stream));
 }
@@ -405,6 +407,7 @@ extern "C" int hexmi_layer_norm(const void* x, const void* weight, const void* b
   if (rows < 0 || cols < 0) return HEXMI_EINVAL;
   if (rows == 0 || cols == 0) return HEXMI_OK;
   if (!x || !y) return HEXMI_EINVAL;
+  begin_call();
   return dispatch_dtype<kLayerNorm>(dtype, x, y, weight, bias, mean, rstd, rows, cols, cols, cols, eps,
                                     as_stream(stream));
 }

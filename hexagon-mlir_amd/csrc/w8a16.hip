@@ -510,6 +510,35 @@ void dequant_kernel(const int8_t* __restrict__ W, const f16* __restrict__ scales
   }
 }
 
+// Any K and any alignment (the shapes the 16-byte-load kernels above do not take): one wave per output channel
+// and block of MR activation rows, lanes stride over k, fp32 multiply-add of the exact int8 -> fp32 and
+// fp16 -> fp32 values, butterfly sum, the channel scale on the finished sum as everywhere else.
+template <int MR>
+__global__ __launch_bounds__(256)
+void w8a16_generic_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
+                          f16* __restrict__ C, int M, int N, int K) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n = blockIdx.x * 4 + wave;
+  const int m0 = blockIdx.y * MR;
+  if (n >= N) return;
+  const int8_t* wrow = W + (int64_t)n * K;
+  float acc[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+  for (int k = lane; k < K; k += kWave) {
+    const float w = (float)wrow[k];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+      if (m0 + m < M) acc[m] = fmaf((float)A[(int64_t)(m0 + m) * K + k], w, acc[m]);
+  }
+  const float sc = (float)scales[n];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    const float tot = wave_sum(acc[m]);
+    if (lane == 0 && m0 + m < M) C[(int64_t)(m0 + m) * N + n] = (f16)(tot * sc);
+  }
+}
+
 template <int MT>
 int launch_pass(const f16* A, const int8_t* W, const f16* s, f16* C, int M, int N, int K, int m_base,
                 hipStream_t st) {
@@ -528,13 +557,22 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
   if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
   if (M == 0 || N == 0) return HEXMI_OK;
   if (!A || !W || !scales || !C) return HEXMI_EINVAL;
-  if (K == 0 || K % 64 != 0) return HEXMI_ENOTSUP;    // 16-byte weight loads, 64-wide K steps
-  if (!aligned_to(A, 16) || !aligned_to(W, 16)) return HEXMI_EINVAL;
   if (M > 0x7fffffff || N > 0x7fffffff - 16 || K > 0x7fffffff) return HEXMI_ENOTSUP;
   hipStream_t st = as_stream(stream);
   const f16* a = static_cast<const f16*>(A);
   const f16* s = static_cast<const f16*>(scales);
   f16* c = static_cast<f16*>(C);
+  begin_call();
+  if (K == 0) return fill_zero_2d(C, M, N, N, 2, st);      // an empty sum
+  // the fast kernels read 16 bytes of a weight row per lane in 64-wide K steps; other shapes take the generic one
+  if (K % 64 != 0 || !aligned_to(A, 16) || !aligned_to(W, 16)) {
+    constexpr int MR = 4;
+    const int64_t gy = (M + MR - 1) / MR;
+    if (gy > 65535) return HEXMI_ENOTSUP;
+    hipLaunchKernelGGL(w8a16_generic_kernel<MR>, dim3((unsigned)((N + 3) / 4), (unsigned)gy), dim3(256), 0, st, a, W, s,
+                       c, (int)M, (int)N, (int)K);
+    return launch_status();
+  }
   if (M <= 2 && (K == 1024 || K == 2048 || K == 4096 || K == 8192)) {
     constexpr int RPW = 2;
     const unsigned blocks = (unsigned)((N + 4 * RPW - 1) / (4 * RPW));
@@ -589,6 +627,7 @@ extern "C" int hexmi_pack_w8(int64_t N, int64_t K, const int8_t* W, int8_t* Wp, 
   const int64_t chunks = ((N + 15) / 16) * 16 * (K / 16);   // 16-byte chunks of the packed buffer
   const int64_t blocks = (chunks + 255) / 256;
   if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
+  begin_call();
   hipLaunchKernelGGL(pack_w8_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), W, Wp, N, K, chunks);
   return launch_status();
 }
@@ -605,6 +644,7 @@ extern "C" int hexmi_gemm_w8a16_packed(int64_t M, int64_t N, int64_t K, const vo
   const int cus = hexmi_num_cus();
   if (cus <= 0) return HEXMI_ELAUNCH;
   hipStream_t st = as_stream(stream);
+  begin_call();
   const int64_t tiles = (N + 15) / 16;
   const int tiles_per_wg = (int)((tiles + cus - 1) / cus);
   const int chan_per_wg = tiles_per_wg * 16;
@@ -628,6 +668,7 @@ extern "C" int hexmi_dequant_w8(int64_t N, int64_t K, const int8_t* W, const voi
   const int64_t total = N * K;
   int64_t blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;
+  begin_call();
   hipLaunchKernelGGL(dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), W,
                      static_cast<const f16*>(scales), out, N, K);
   return launch_status();

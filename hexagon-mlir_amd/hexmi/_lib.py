@@ -10,8 +10,8 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhexmi.so")
 
-OK, EINVAL, ENOTSUP, ELAUNCH = 0, -1, -2, -3
-F32, F16, BF16, I8 = 0, 1, 2, 3
+OK, EINVAL, ENOTSUP, ELAUNCH, ETOOBIG = 0, -1, -2, -3, -4
+F16, F32, I8, BF16 = 1, 2, 4, 16       # hexmi_dtype: the reference's tensor.h ids, bf16 outside its table
 
 
 class HexmiError(RuntimeError):
@@ -41,6 +41,8 @@ SIGNATURES = {
     "hexmi_unary": (_int, [_int, _ptr, _ptr, _i64, _int, _ptr]),
     "hexmi_binary": (_int, [_int, _ptr, _ptr, _ptr, _i64, _int, _ptr]),
     "hexmi_block_sum": (_int, [_ptr, _ptr, _i64, _i64, _int, _ptr]),
+    "hexmi_block_sum_workspace": (_i64, [_i64, _i64, _int]),
+    "hexmi_block_sum_ws": (_int, [_ptr, _ptr, _i64, _i64, _int, _ptr, _i64, _ptr]),
     "hexmi_rope": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _f64, _int, _ptr]),
     "hexmi_attention": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _ptr]),
 }

@@ -35,6 +35,25 @@ def _p(t):
     return None if t is None else t.data_ptr()
 
 
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on(device):
+    """Context that makes `device` current for the launch; free when it already is (the usual case: entering
+    torch.cuda.device() costs more than the shortest kernels here run)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
+
+
 # --------------------------------------------------------------------------
 # custom-op registration (schema: inputs..., Tensor(a!) out) -> ()
 # --------------------------------------------------------------------------
@@ -58,21 +77,21 @@ _LIBDEF.define("attention(Tensor q, Tensor k, Tensor v, Tensor? mask, float sm_s
 
 def _softmax_impl(x, out):
     rows, cols = x.shape
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(_lib.lib().hexmi_softmax(_p(x), _p(out), rows, cols, x.stride(0), out.stride(0), _dt(x),
                                             _stream()), "hexmi_softmax")
 
 
 def _rms_norm_impl(x, weight, eps, out):
     rows, cols = x.shape
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(_lib.lib().hexmi_rms_norm(_p(x), _p(weight), _p(out), rows, cols, eps, _dt(x), _stream()),
                    "hexmi_rms_norm")
 
 
 def _layer_norm_impl(x, weight, bias, eps, out, mean, rstd):
     rows, cols = x.shape
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(_lib.lib().hexmi_layer_norm(_p(x), _p(weight), _p(bias), _p(out), _p(mean), _p(rstd), rows, cols,
                                                eps, _dt(x), _stream()), "hexmi_layer_norm")
 
@@ -80,7 +99,7 @@ def _layer_norm_impl(x, weight, bias, eps, out, mean, rstd):
 def _matmul_impl(a, b, trans_b, out):
     M, K = a.shape
     N = b.shape[0] if trans_b else b.shape[1]
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         _lib.check(_lib.lib().hexmi_gemm(M, N, K, _p(a), a.stride(0), _p(b), b.stride(0), _p(out), out.stride(0),
                                          _dt(a), _dt(out), 1 if trans_b else 0, _stream()), "hexmi_gemm")
 
@@ -88,34 +107,34 @@ def _matmul_impl(a, b, trans_b, out):
 def _w8a16_impl(a, w, scales, out):
     M, K = a.shape
     N = w.shape[0]
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         _lib.check(_lib.lib().hexmi_gemm_w8a16(M, N, K, _p(a), _p(w), _p(scales), _p(out), _stream()),
                    "hexmi_gemm_w8a16")
 
 
 def _pack_impl(w, out):
     N, K = w.shape
-    with torch.cuda.device(w.device):
+    with _on(w.device):
         _lib.check(_lib.lib().hexmi_pack_w8(N, K, _p(w), _p(out), _stream()), "hexmi_pack_w8")
 
 
 def _w8a16_packed_impl(a, wp, scales, out):
     M, K = a.shape
     N = scales.shape[0]
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         _lib.check(_lib.lib().hexmi_gemm_w8a16_packed(M, N, K, _p(a), _p(wp), _p(scales), _p(out), _stream()),
                    "hexmi_gemm_w8a16_packed")
 
 
 def _dequant_impl(w, scales, out):
     N, K = w.shape
-    with torch.cuda.device(w.device):
+    with _on(w.device):
         _lib.check(_lib.lib().hexmi_dequant_w8(N, K, _p(w), _p(scales), _p(out), _stream()), "hexmi_dequant_w8")
 
 
 def _flash_impl(q, k, v, sm_scale, causal, out):
     Z, H, S, D = q.shape
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         _lib.check(_lib.lib().hexmi_flash_attn_fwd(_p(q), _p(k), _p(v), _p(out), Z, H, S, D, sm_scale,
                                                    1 if causal else 0, _dt(q), _dt(out), _stream()),
                    "hexmi_flash_attn_fwd")
@@ -124,29 +143,35 @@ def _flash_impl(q, k, v, sm_scale, causal, out):
 def _attention_impl(q, k, v, mask, sm_scale, out):
     B, Sq, D = q.shape
     Skv = k.shape[1]
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         _lib.check(_lib.lib().hexmi_attention(_p(q), _p(k), _p(v), _p(mask), _p(out), B, Sq, Skv, D, sm_scale,
                                               _dt(q), _dt(out), _stream()), "hexmi_attention")
 
 
 def _unary_impl(op, x, out):
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(_lib.lib().hexmi_unary(op, _p(x), _p(out), x.numel(), _dt(x), _stream()), "hexmi_unary")
 
 
 def _binary_impl(op, a, b, out):
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         _lib.check(_lib.lib().hexmi_binary(op, _p(a), _p(b), _p(out), a.numel(), _dt(a), _stream()), "hexmi_binary")
 
 
 def _block_sum_impl(x, block, out):
-    with torch.cuda.device(x.device):
-        _lib.check(_lib.lib().hexmi_block_sum(_p(x), _p(out), x.numel(), block, _dt(x), _stream()), "hexmi_block_sum")
+    n = x.numel()
+    need = _lib.lib().hexmi_block_sum_workspace(n, block, _dt(x))
+    # huge programs (the reference test sums 2^20 elements in one) are summed in two passes over the whole chip
+    # when the library is handed scratch for its fp32 partial sums
+    ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+    with _on(x.device):
+        _lib.check(_lib.lib().hexmi_block_sum_ws(_p(x), _p(out), n, block, _dt(x), _p(ws), need, _stream()),
+                   "hexmi_block_sum_ws")
 
 
 def _rope_impl(x, theta, out):
     B, L, H, D = x.shape
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(_lib.lib().hexmi_rope(_p(x), _p(out), B, L, H, D, theta, _dt(x), _stream()), "hexmi_rope")
 
 
@@ -200,7 +225,8 @@ def _out_like(out, shape, dtype, dev):
 
 
 # --------------------------------------------------------------------------
-# public operators
+# public operators. They call the implementations above directly: the same code `torch.ops.hexmi.*` runs, without
+# the dispatcher's round trip into Python (several microseconds, more than the shortest kernels here take).
 # --------------------------------------------------------------------------
 def softmax(x, out=None, dim=-1):
     """Softmax over the last dimension (`F.softmax(x, dim=1)` of
@@ -214,7 +240,7 @@ def softmax(x, out=None, dim=-1):
     od = _out_like(out, x.shape, x.dtype, dev)
     cols = x.shape[-1]
     rows = x.numel() // max(cols, 1)
-    torch.ops.hexmi.softmax(xd.view(rows, cols), od.view(rows, cols))
+    _softmax_impl(xd.view(rows, cols), od.view(rows, cols))
     return _finish(od, out)
 
 
@@ -227,7 +253,7 @@ def rms_norm(x, weight=None, eps=1e-5, out=None):
         raise ValueError("hexmi.rms_norm: weight must be [%d] of %s" % (cols, x.dtype))
     xd, wd = _stage(x, dev), _stage(weight, dev)
     od = _out_like(out, x.shape, x.dtype, dev)
-    torch.ops.hexmi.rms_norm(xd.view(rows, cols), wd, float(eps), od.view(rows, cols))
+    _rms_norm_impl(xd.view(rows, cols), wd, float(eps), od.view(rows, cols))
     return _finish(od, out)
 
 
@@ -244,7 +270,7 @@ def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=No
     od = _out_like(out, x.shape, x.dtype, dev)
     md = None if mean is None else _out_like(mean if mean.dtype == torch.float32 else None, (rows,), torch.float32, dev)
     rd = None if rstd is None else _out_like(rstd if rstd.dtype == torch.float32 else None, (rows,), torch.float32, dev)
-    torch.ops.hexmi.layer_norm(xd.view(rows, cols), wd, bd, float(eps), od.view(rows, cols), md, rd)
+    _layer_norm_impl(xd.view(rows, cols), wd, bd, float(eps), od.view(rows, cols), md, rd)
     if mean is not None:
         _finish(md, mean)
     if rstd is not None:
@@ -271,7 +297,7 @@ def matmul(a, b, out=None, out_dtype=None, trans_b=False):
     dev = _device() if a.device.type != "cuda" else a.device
     ad, bd = _stage(a, dev), _stage(b, dev)
     od = _out_like(out, (M, N), out_dtype, dev)
-    torch.ops.hexmi.matmul(ad, bd, bool(trans_b), od)
+    _matmul_impl(ad, bd, bool(trans_b), od)
     return _finish(od, out)
 
 
@@ -284,7 +310,7 @@ def w8a16_matmul(a, w_int8, scales, out=None):
     dev = _device() if a.device.type != "cuda" else a.device
     ad, wd, sd = _stage(a, dev), _stage(w_int8, dev), _stage(scales, dev)
     od = _out_like(out, (a.shape[0], w_int8.shape[0]), torch.float16, dev)
-    torch.ops.hexmi.w8a16_matmul(ad, wd, sd, od)
+    _w8a16_impl(ad, wd, sd, od)
     return _finish(od, out)
 
 
@@ -300,7 +326,7 @@ def pack_w8(w_int8):
     dev = _device() if w_int8.device.type != "cuda" else w_int8.device
     wd = _stage(w_int8, dev)
     out = torch.empty(((N + 15) // 16) * 16 * K, dtype=torch.int8, device=dev)
-    torch.ops.hexmi.pack_w8(wd, out)
+    _pack_impl(wd, out)
     return out
 
 
@@ -318,7 +344,7 @@ def w8a16_matmul_packed(a, w_packed, scales, out=None):
     dev = _device() if a.device.type != "cuda" else a.device
     ad, wd, sd = _stage(a, dev), _stage(w_packed, dev), _stage(scales, dev)
     od = _out_like(out, (M, N), torch.float16, dev)
-    torch.ops.hexmi.w8a16_matmul_packed(ad, wd, sd, od)
+    _w8a16_packed_impl(ad, wd, sd, od)
     return _finish(od, out)
 
 
@@ -329,7 +355,7 @@ def dequant_w8(w_int8, scales, out=None):
     dev = _device() if w_int8.device.type != "cuda" else w_int8.device
     wd, sd = _stage(w_int8, dev), _stage(scales, dev)
     od = _out_like(out, w_int8.shape, torch.float32, dev)
-    torch.ops.hexmi.dequant_w8(wd, sd, od)
+    _dequant_impl(wd, sd, od)
     return _finish(od, out)
 
 
@@ -347,7 +373,7 @@ def flash_attention(q, k, v, sm_scale=None, causal=False, out=None, out_dtype=No
     dev = _device() if q.device.type != "cuda" else q.device
     qd, kd, vd = _stage(q, dev), _stage(k, dev), _stage(v, dev)
     od = _out_like(out, q.shape, out_dtype, dev)
-    torch.ops.hexmi.flash_attention(qd, kd, vd, float(sm_scale), bool(causal), od)
+    _flash_impl(qd, kd, vd, float(sm_scale), bool(causal), od)
     return _finish(od, out)
 
 
@@ -370,7 +396,7 @@ def attention(q, k, v, mask=None, sm_scale=None, out=None, out_dtype=None):
     dev = _device() if q.device.type != "cuda" else q.device
     qd, kd, vd, md = _stage(q, dev), _stage(k, dev), _stage(v, dev), _stage(mask, dev)
     od = _out_like(out, q.shape, out_dtype, dev)
-    torch.ops.hexmi.attention(qd, kd, vd, md, float(sm_scale), od)
+    _attention_impl(qd, kd, vd, md, float(sm_scale), od)
     return _finish(od, out)
 
 
@@ -386,7 +412,7 @@ def unary(op, x, out=None):
     dev = _device() if x.device.type != "cuda" else x.device
     xd = _stage(x, dev)
     od = _out_like(out, x.shape, x.dtype, dev)
-    torch.ops.hexmi.unary(UNARY_OPS[op], xd, od)
+    _unary_impl(UNARY_OPS[op], xd, od)
     return _finish(od, out)
 
 
@@ -410,11 +436,8 @@ def binary(op, a, b, out=None):
     dev = _device() if a.device.type != "cuda" else a.device
     ad, bd = _stage(a, dev), _stage(b, dev)
     od = _out_like(out, a.shape, a.dtype, dev)
-    torch.ops.hexmi.binary(BINARY_OPS[op], ad, bd, od)
+    _binary_impl(BINARY_OPS[op], ad, bd, od)
     return _finish(od, out)
-
-
-_TWO_PASS_MIN_BLOCK, _TWO_PASS_RUN = 1 << 16, 4096
 
 
 def block_sum(x, block=None, out=None):
@@ -429,15 +452,7 @@ def block_sum(x, block=None, out=None):
     dev = _device() if x.device.type != "cuda" else x.device
     xd = _stage(x, dev).reshape(-1)
     od = _out_like(out, (programs,), x.dtype, dev)
-    if x.dtype == torch.float32 and block >= _TWO_PASS_MIN_BLOCK and (programs == 1 or block % _TWO_PASS_RUN == 0):
-        # A program is one workgroup in the library (as it is one Triton program in the reference): a few huge
-        # programs - the reference test sums 2^20 elements in one - leave the chip idle. fp32 partial sums of runs
-        # of 4096 lose nothing, so they are formed by many workgroups first and summed per program afterwards.
-        parts = torch.empty((n + _TWO_PASS_RUN - 1) // _TWO_PASS_RUN, dtype=torch.float32, device=dev)
-        torch.ops.hexmi.block_sum(xd, _TWO_PASS_RUN, parts)
-        torch.ops.hexmi.block_sum(parts, parts.numel() if programs == 1 else block // _TWO_PASS_RUN, od)
-    else:
-        torch.ops.hexmi.block_sum(xd, int(block), od)
+    _block_sum_impl(xd, int(block), od)
     return _finish(od, out)
 
 
@@ -449,7 +464,7 @@ def rope(x, theta=10000.0, out=None):
     dev = _device() if x.device.type != "cuda" else x.device
     xd = _stage(x, dev)
     od = _out_like(out, x.shape, x.dtype, dev)
-    torch.ops.hexmi.rope(xd, float(theta), od)
+    _rope_impl(xd, float(theta), od)
     return _finish(od, out)
 
 

@@ -8,7 +8,11 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
  *     calls enqueue work and return without synchronising;
  *   - the return value is HEXMI_OK or a negative hexmi_status; nothing throws;
- *   - calls are re-entrant; two calls may run concurrently on different streams.
+ *   - calls are re-entrant; two calls may run concurrently on different streams
+ *     (the one exception, hexmi_block_sum_static, says so);
+ *   - a HEXMI_ELAUNCH status describes the launches of that call only: an
+ *     error left pending on the calling thread by earlier HIP calls is
+ *     discarded on entry, not reported.
  *
  * Each declaration cites the reference interface it stands in for
  * (paths relative to the hexagon-mlir source tree).
@@ -28,17 +32,19 @@ typedef enum hexmi_status {
   HEXMI_OK = 0,
   HEXMI_EINVAL = -1,  /* null pointer, non-positive size, bad leading dim, misaligned */
   HEXMI_ENOTSUP = -2, /* dtype / shape combination with no kernel */
-  HEXMI_ELAUNCH = -3  /* hipLaunchKernel or another HIP call failed */
+  HEXMI_ELAUNCH = -3, /* hipLaunchKernel or another HIP call failed */
+  HEXMI_ETOOBIG = -4  /* size beyond the fixed capacity of an entry point that allocates nothing */
 } hexmi_status;
 
-/* Element types. Values match the reference's raw-tensor dtype ids where one
- * exists (test/utils/dsp/include/tensor.h:26-38 is the id table the device
- * harness and backend/utils.py:36-54 share). */
+/* Element types. The values are the reference's raw-tensor data type ids
+ * (enum DataType of test/utils/dsp/include/tensor.h:26-38, the table the device
+ * harness and backend/utils.py:36-54 share: Half = 1, Float = 2, Int8 = 4).
+ * bfloat16 has no id there; it takes a value outside that table (ids 0..10). */
 typedef enum hexmi_dtype {
-  HEXMI_F32 = 0,
   HEXMI_F16 = 1,
-  HEXMI_BF16 = 2,
-  HEXMI_I8 = 3
+  HEXMI_F32 = 2,
+  HEXMI_I8 = 4,
+  HEXMI_BF16 = 16
 } hexmi_dtype;
 
 /* Library / device ------------------------------------------------------- */
@@ -221,6 +227,22 @@ int hexmi_binary(int op, const void *a, const void *b, void *y, int64_t n,
  * 1024*1024 elements). fp32 accumulation in a fixed order; out has `dtype`. */
 int hexmi_block_sum(const void *x, void *out, int64_t n, int64_t block,
                     int dtype, hexmi_stream_t stream);
+
+/* hexmi_block_sum with a caller-owned scratch buffer. A program is one
+ * workgroup, as it is one Triton program in the reference, so a launch of a
+ * few huge programs (test/python/triton/test_sum.py:25-47 sums 2^20 elements
+ * in ONE program) would use one compute unit; with a workspace, programs of
+ * 65536 elements and more are summed in two passes over the whole chip (fp32
+ * partial sums of runs of 4096 elements, then one sum per program), for every
+ * dtype. hexmi_block_sum_workspace returns the bytes that takes for (n, block,
+ * dtype): 0 when one pass is used anyway (small programs, or several programs
+ * whose size is not a multiple of 4096). workspace may be NULL (one pass);
+ * a workspace smaller than the query's answer is HEXMI_EINVAL. The workspace
+ * holds no state between calls. */
+int64_t hexmi_block_sum_workspace(int64_t n, int64_t block, int dtype);
+int hexmi_block_sum_ws(const void *x, void *out, int64_t n, int64_t block,
+                       int dtype, void *workspace, int64_t workspace_bytes,
+                       hexmi_stream_t stream);
 
 /* Rotary position embedding of x [batch, seq, heads, feat] (contiguous, feat
  * even): adjacent feature pairs (2i, 2i+1) are rotated by m * theta^(-2i/feat),

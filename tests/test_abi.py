@@ -80,3 +80,29 @@ def test_kernel_front_checks_grid_and_options():
         k[(1,)](x, x, NUM_ROWS=2, NUM_COLS=2, BLOCK_SIZE=2, notAnOption=True)
     with pytest.raises(RuntimeError, match="outside"):
         k(x, x)
+
+
+def test_dtype_ids_are_the_reference_tensor_ids():
+    # enum DataType of the reference's test/utils/dsp/include/tensor.h:26-38: Half = 1, Float = 2, Int8 = 4;
+    # bfloat16 has no id there and sits outside the table (0..10)
+    from hexmi import _lib, tensor_file
+    text = open(HEADER).read()
+    ids = dict((k, int(v)) for k, v in re.findall(r"(HEXMI_(?:F16|F32|I8|BF16))\s*=\s*(\d+)", text))
+    assert ids == {"HEXMI_F16": 1, "HEXMI_F32": 2, "HEXMI_I8": 4, "HEXMI_BF16": 16}
+    assert (_lib.F16, _lib.F32, _lib.I8, _lib.BF16) == (1, 2, 4, 16)
+    import numpy as np
+    for code, np_type in ((_lib.F16, np.float16), (_lib.F32, np.float32), (_lib.I8, np.int8)):
+        assert tensor_file._ID_TO_NP[code] is np_type
+    assert _lib.BF16 not in tensor_file._ID_TO_NP
+
+
+def test_block_sum_workspace_query_needs_no_device():
+    from hexmi import _lib
+    lib = _lib.lib()
+    assert lib.hexmi_block_sum_workspace(1 << 20, 1 << 20, _lib.F16) == 256 * 4       # one program: two passes
+    assert lib.hexmi_block_sum_workspace(1 << 20, 4096, _lib.F32) == 0                # small programs: one pass
+    assert lib.hexmi_block_sum_workspace(300000, 131072, _lib.F32) == 74 * 4
+    assert lib.hexmi_block_sum_workspace(300000, 100000, _lib.F32) == 0               # runs would straddle programs
+    assert lib.hexmi_block_sum_workspace(0, 16, _lib.F32) == 0
+    assert lib.hexmi_block_sum_ws(None, None, -1, 4, _lib.F32, None, 0, None) == _lib.EINVAL
+    assert "capacity" in _lib.strerror(_lib.ETOOBIG)

@@ -147,9 +147,41 @@ def test_block_sum_large_fp32_programs(hexmi, n, block):
     want = torch.stack([x[i:i + b].double().sum() for i in range(0, n, b)])
     assert got.shape == want.shape and got.dtype == torch.float32
     assert torch.allclose(got.double(), want, rtol=1e-5, atol=2e-6 * b ** 0.5)
-    one_pass = torch.empty_like(got).cuda()
-    torch.ops.hexmi.block_sum(x.cuda(), b, one_pass)
+    from hexmi import _lib
+    xd, one_pass = x.cuda(), torch.empty_like(got).cuda()
+    assert _lib.lib().hexmi_block_sum(xd.data_ptr(), one_pass.data_ptr(), n, b, _lib.F32, None) == _lib.OK
     assert torch.allclose(got, one_pass.cpu(), rtol=1e-5, atol=2e-6 * b ** 0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_block_sum_workspace_entry(hexmi, dtype):
+    # the reference test's own shape through the C ABI: one program over 2^20 elements, summed by the whole chip
+    # when the caller passes the scratch the size query asks for; 16-bit inputs keep fp32 partial sums
+    from hexmi import _lib
+    lib = _lib.lib()
+    code = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}[dtype]
+    n = 1 << 20
+    x = torch.randn(n, generator=_gen(44)).to(dtype)
+    want = x.double().sum().item()
+    xd = x.cuda()
+    need = lib.hexmi_block_sum_workspace(n, n, code)
+    assert need == (n // 4096) * 4
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    out = torch.zeros(1, dtype=dtype, device="cuda")
+    assert lib.hexmi_block_sum_ws(xd.data_ptr(), out.data_ptr(), n, n, code, ws.data_ptr(), need, None) == _lib.OK
+    tol = 1e-2 if dtype == torch.float32 else 0.51 if dtype == torch.float16 else 4.1
+    assert abs(out.double().item() - want) <= tol
+    # too small a workspace is refused; none at all is the one-pass sum
+    assert lib.hexmi_block_sum_ws(xd.data_ptr(), out.data_ptr(), n, n, code, ws.data_ptr(), need - 4, None) == _lib.EINVAL
+    assert lib.hexmi_block_sum_ws(xd.data_ptr(), out.data_ptr(), n, n, code, None, 0, None) == _lib.OK
+    assert abs(out.double().item() - want) <= tol
+    # several programs, ragged last one
+    n2, b2 = 300000, 131072
+    assert lib.hexmi_block_sum_workspace(n2, b2, code) == ((n2 + 4095) // 4096) * 4
+    out3 = torch.zeros(3, dtype=dtype, device="cuda")
+    assert lib.hexmi_block_sum_ws(xd.data_ptr(), out3.data_ptr(), n2, b2, code, ws.data_ptr(), need, None) == _lib.OK
+    want3 = torch.stack([x[i:i + b2].double().sum() for i in range(0, n2, b2)])
+    assert (out3.double().cpu() - want3).abs().max() <= tol
 
 
 def test_reference_sum_call_site(hexmi):

@@ -158,6 +158,27 @@ def test_attention_errors(hexmi):
                                  torch.empty(1, 2, 0, 64, device="cuda", dtype=torch.float16)).shape == (1, 2, 0, 64)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("scale", [0.0, -0.3])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_attention_zero_and_negative_scale(hexmi, oracle, dtype, scale, causal):
+    # the matrix-core kernels take the row maximum before scaling, which is right for a positive scale only: other
+    # scales must still give softmax(scale * Q K^T) V (scale 0: the mean of the visible V rows)
+    q, k, v = _qkv(1, 2, 200, 128, dtype, seed=11)
+    o = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal, out_dtype=torch.float32).cpu()
+    want = _oracle(oracle, q, k, v, scale, causal)
+    assert torch.isfinite(o).all()
+    assert (o - want).abs().max() <= (2e-2 if dtype == torch.float16 else 1e-5 * want.abs().max())
+    if scale == 0.0 and not causal:
+        assert (o - v.float().mean(2, keepdim=True)).abs().max() <= 2e-3
+
+
+def test_attention_head_size_256(hexmi, oracle):
+    q, k, v = _qkv(1, 2, 70, 256, torch.float16, seed=12)
+    o = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), 1 / 16.0, True, out_dtype=torch.float32).cpu()
+    assert (o - _oracle(oracle, q, k, v, 1 / 16.0, True)).abs().max() <= 2e-2
+
+
 # ---- tm_tensor.attention: [B, S, D] operands, rectangular scores, additive mask -----------------------------
 def _oracle_masked(oracle, q, k, v, mask, scale):
     qn, tag = to_np(q)

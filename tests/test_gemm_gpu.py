@@ -198,6 +198,22 @@ def test_gemm_config_sizes(hexmi, oracle, dtype, size):
     assert torch.equal(c_t, c)
 
 
+def test_gemm_empty_inner_dimension_is_zero(hexmi):
+    # a product over K = 0 is all zeros (torch.matmul gives the same), for every output type, with a leading dimension
+    for dt, odt in ((torch.float16, torch.float16), (torch.bfloat16, torch.float32), (torch.float32, torch.float32)):
+        buf = torch.full((5, 12), 3.0, dtype=odt, device="cuda")
+        out = buf[:, :7]
+        from hexmi import _lib
+        code = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
+        rc = _lib.lib().hexmi_gemm(5, 7, 0, None, 0, None, 7, out.data_ptr(), 12, code[dt], code[odt], 0, None)
+        assert rc == _lib.OK
+        torch.cuda.synchronize()
+        assert torch.equal(buf[:, :7].cpu(), torch.zeros(5, 7, dtype=odt))
+        assert torch.equal(buf[:, 7:].cpu(), torch.full((5, 5), 3.0, dtype=odt))       # past N: untouched
+    assert hexmi.matmul(torch.zeros(4, 0, dtype=torch.float16, device="cuda"),
+                        torch.zeros(0, 8, dtype=torch.float16, device="cuda")).abs().sum().item() == 0
+
+
 def test_gemm_argument_errors(hexmi):
     from hexmi import _lib
     a = torch.zeros(8, 8, device="cuda", dtype=torch.float16)

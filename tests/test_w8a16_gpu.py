@@ -113,9 +113,28 @@ def test_w8a16_errors(hexmi):
         hexmi.w8a16_matmul(a.float(), torch.zeros(4, 64, dtype=torch.int8), torch.zeros(4, dtype=torch.float16))
     with pytest.raises(ValueError):
         hexmi.w8a16_matmul(a, torch.zeros(4, 32, dtype=torch.int8), torch.zeros(4, dtype=torch.float16))
-    with pytest.raises(hexmi.HexmiError):                     # K not a multiple of 64
-        hexmi.w8a16_matmul(torch.zeros(2, 40, dtype=torch.float16).cuda(), torch.zeros(4, 40, dtype=torch.int8).cuda(),
-                           torch.zeros(4, dtype=torch.float16).cuda())
+
+
+@pytest.mark.parametrize("M,N,K", [(2, 4, 40), (5, 33, 1), (17, 130, 100), (3, 64, 4100), (70, 20, 72), (4, 32, 128)])
+def test_w8a16_any_inner_size(hexmi, oracle, M, N, K):
+    # K % 64 != 0 takes the generic kernel: same oracle, same bar
+    a, w, s = _inputs(M, N, K, seed=5)
+    got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
+    want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w.numpy(), s.numpy()))
+    assert close16(got, want, max_ulp=1, atol=2e-4)
+    # unaligned activations (a view that starts 2 bytes into an allocation) take it too, whatever K is
+    buf = torch.zeros(M * K + 1, dtype=torch.float16, device="cuda")
+    av = buf[1:].view(M, K)
+    av.copy_(a)
+    assert torch.equal(hexmi.w8a16_matmul(av, w.cuda(), s.cuda()).cpu(), got)
+
+
+def test_w8a16_empty_inner_dimension_is_zero(hexmi):
+    out = torch.full((3, 8), 7.0, dtype=torch.float16, device="cuda")
+    hexmi.w8a16_matmul(torch.zeros(3, 0, dtype=torch.float16, device="cuda"),
+                       torch.zeros(8, 0, dtype=torch.int8, device="cuda"),
+                       torch.ones(8, dtype=torch.float16, device="cuda"), out=out)
+    assert torch.equal(out.cpu(), torch.zeros(3, 8, dtype=torch.float16))
 
 
 @pytest.mark.parametrize("N,K", [(48, 1024), (1000, 2048), (11008, 4096), (17, 1024)])
