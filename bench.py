@@ -11,7 +11,12 @@ its own roofline fraction. `cpu_baseline` times the reference's CPU path (the Py
 oracle) on the host cores for the primary workload; suite entries carry their own `cpu` leg.
 
 Kernel launch durations are measured with HIP events on the stream the kernels are launched on (torch's
-current stream, which hexmi passes to the C ABI).
+current stream, which hexmi passes to the C ABI): the K steps are captured into one HIP graph and the graph is
+replayed REPLAYS times, each replay timed on its own; `ms_per_step` is the median replay, `ms_min` the fastest.
+`targets` lists the ten configurations that carry a throughput target with fraction, target and met / missed.
+HBM-bound entries also carry a `hot` figure (one buffer set, served by the 256 MB Infinity Cache where it fits):
+the rotated one is the HBM claim. `--workload mfma_peak` times a registers-only MFMA stream (zeros and U(-1,1)
+operands, both instruction shapes, about a second each): the data-dependent ceiling of the matrix cores on this box.
 """
 import argparse
 import json
@@ -28,7 +33,13 @@ for _p in (ROOT, os.path.join(ROOT, "hexagon-mlir_amd")):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 / bf16 matrix, published
 MFMA_F32_PEAK_TFLOPS = 157.3   # MI355X fp32 matrix, published
-ROTATE_BYTES = 640 << 20       # rotate HBM-bound workloads over more than 2x the 256 MB Infinity Cache
+ROTATE_BYTES = 1024 << 20      # rotate HBM-bound workloads over 4x the 256 MB Infinity Cache
+REPLAYS = 7                    # timed replays of the K-step graph: median and min are reported
+TARGETS = {                    # fraction of the published peak each configuration is asked to reach
+    "softmax_f32_4096x1024": 0.70, "rms_norm_f16_8192x4096": 0.70, "layer_norm_f16_8192x4096": 0.70,
+    "gemm_f16_4096": 0.60, "gemm_bf16_8192": 0.60, "w8a16_m1": 0.60, "w8a16_m16": 0.60, "w8a16_m256": 0.60,
+    "attn_causal_f16_4x32x4096x128": 0.60, "attn_causal_f16_1x32x16384x128": 0.60,
+}
 
 
 class Workload:
@@ -83,13 +94,17 @@ class CopyCalibration(Workload):
 
 
 class Softmax(Workload):
-    name, bound, dtype, kernel = "softmax_f32_4096x1024", "hbm", "f32", "row_kernel"
-    desc = "row softmax fp32 [4096,1024] N(0,1) seed 0"
+    bound, dtype, kernel = "hbm", "f32", "row_kernel"
+
+    def __init__(self, rows=4096, cols=1024):
+        self.rows, self.cols = rows, cols
+        self.name = "softmax_f32_%dx%d" % (rows, cols)
+        self.desc = "row softmax fp32 [%d,%d] N(0,1) seed 0" % (rows, cols)
 
     def setup(self, torch, hexmi):
         from hexmi.workloads import softmax_inputs, softmax_bytes
-        self.hexmi, self.host = hexmi, softmax_inputs()
-        self.work = softmax_bytes(4096, 1024, 4)
+        self.hexmi, self.host = hexmi, softmax_inputs(self.rows, self.cols)
+        self.work = softmax_bytes(self.rows, self.cols, 4)
         self.sets = _sets(torch, self.host, self.work)
         for s in self.sets:
             s["out"] = torch.empty_like(s["x"])
@@ -100,7 +115,10 @@ class Softmax(Workload):
 
     def cpu(self, torch):
         from oracle import torch_cpu
-        return _time_cpu(lambda: torch_cpu.softmax(self.host["x"]), 5), "full [4096,1024], torch.softmax on CPU"
+        x = self.host["x"][:4096]
+        t = _time_cpu(lambda: torch_cpu.softmax(x), 5) * (self.rows / 4096)
+        return t, "rows 0..4096 of [%d,%d], torch.softmax on CPU%s" % (self.rows, self.cols,
+                                                                     ", time scaled" if self.rows > 4096 else "")
 
 
 class Norms(Workload):
@@ -119,11 +137,15 @@ class Norms(Workload):
             s["out"] = torch.empty_like(s["x"])
 
     def step(self, i):
-        s = self.sets[i % len(self.sets)]
+        n = len(self.sets)
+        s = self.sets[i % n]
         if "rms" in self.which:
             self.hexmi.rms_norm(s["x"], s["weight"], 1e-5, out=s["out"])
         if "ln" in self.which:
-            self.hexmi.layer_norm(s["x"], s["weight"], s["bias"], 1e-5, out=s["out"])
+            # with both kernels in a step the second reads a set half the rotation away, not the 64 MiB the first
+            # has just pulled through the Infinity Cache
+            t = self.sets[(i + n // 2) % n] if "rms" in self.which else s
+            self.hexmi.layer_norm(t["x"], t["weight"], t["bias"], 1e-5, out=t["out"])
 
     def cpu(self, torch):
         from oracle import torch_cpu
@@ -374,6 +396,39 @@ class MaskedAttention(Workload):
         return t * (B / n), "%d of %d batch entries, fp32 F.scaled_dot_product_attention(attn_mask=...) on CPU, time scaled" % (n, B)
 
 
+class MfmaPeak(Workload):
+    """Registers-only MFMA stream (hexmi_mfma_peak): the rate the matrix cores sustain on given operand data."""
+    bound, kernel = "mfma", "mfma_peak_kernel"
+
+    def __init__(self, shape, dtype_name, data, waves=2):
+        self.shape, self.dtype, self.data, self.waves = shape, dtype_name, data, waves
+        self.name = "mfma_peak_%s_%s_%s" % ("32x32x16" if shape == 0 else "16x16x32", dtype_name, data)
+        self.desc = ("v_mfma_f32_%s_%s only, %d waves per SIMD, operands %s, accumulators in registers"
+                     % ("32x32x16" if shape == 0 else "16x16x32", dtype_name, waves,
+                        "all zero" if data == "zeros" else "U(-1,1)"))
+        self.iters = 20000 if shape == 0 else 20000
+
+    def setup(self, torch, hexmi):
+        from hexmi import _lib
+        self.lib, self._lib = _lib.lib(), _lib
+        dt = torch.float16 if self.dtype == "f16" else torch.bfloat16
+        g = torch.Generator().manual_seed(0)
+        ops = torch.zeros(1024) if self.data == "zeros" else 2 * torch.rand(1024, generator=g) - 1
+        self.ops = ops.to(dt).cuda()
+        self.sink = torch.empty(self.lib.hexmi_num_cus() * 256 * self.waves, device="cuda")
+        self.work = int(self.lib.hexmi_mfma_peak_flops(self.shape, self.waves, self.iters))
+        self.code = _lib.F16 if self.dtype == "f16" else _lib.BF16
+        self.stream = torch.cuda.current_stream
+        self.sets = [None]
+
+    def step(self, i):
+        self._lib.check(self.lib.hexmi_mfma_peak(self.shape, self.code, self.ops.data_ptr(), self.iters, self.waves,
+                                                 self.sink.data_ptr(), self.stream().cuda_stream), "hexmi_mfma_peak")
+
+    def cpu(self, torch):
+        return float("nan"), "no CPU counterpart"
+
+
 def _time_cpu(fn, iters):
     fn()                                                # warm-up
     ts = []
@@ -387,25 +442,35 @@ def _time_cpu(fn, iters):
 
 def make_workloads():
     return {w.name: w for w in (
-        Norms(), Softmax(), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"), Gemm(4096, "f32"),
-        W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256), Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), AttentionF32(4, 32, 2048, 64), MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
-        Elementwise("sum"),
-        CopyCalibration())}
+        Norms(), Softmax(), Softmax(65536, 1024), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
+        Gemm(4096, "f32"), W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256),
+        Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), AttentionF32(4, 32, 2048, 64),
+        MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
+        Elementwise("sum"), CopyCalibration())}
 
 
-ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024", "gemm": "gemm_f16_4096",
+def peak_workloads():
+    return [MfmaPeak(shape, dt, data) for dt in ("f16", "bf16") for shape in (0, 1) for data in ("zeros", "uniform")]
+
+
+ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024",
+           "softmax_big": "softmax_f32_65536x1024", "gemm": "gemm_f16_4096",
            "gemm_bf16": "gemm_bf16_8192", "gemm_f32": "gemm_f32_4096", "attn": "attn_causal_f16_4x32x4096x128",
-           "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128", "attn_f32": "attn_causal_f32_4x32x2048x64", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
+           "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128",
+           "attn_f32": "attn_causal_f32_4x32x2048x64", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
            "rope": "rope_f16_4x4096x32x128", "sum": "block_sum_f32_8192x4096", "rms_norm": "rms_norm_f16_8192x4096",
-           "layer_norm": "layer_norm_f16_8192x4096"}
+           "layer_norm": "layer_norm_f16_8192x4096", "w8a16_m1": "w8a16_m1", "w8a16_m16": "w8a16_m16",
+           "w8a16_m64": "w8a16_m64", "w8a16_m256": "w8a16_m256"}
 
 
-def measure(torch, wl, steps, warmup, use_graph=True):
-    """ms per step from HIP events around `steps` steps on the current stream.
+def measure(torch, wl, steps, warmup, use_graph=True, replays=REPLAYS):
+    """Per-step times (ms) from HIP events on the current stream: {"ms": median, "min": ..., "max": ...,
+    "wall": host wall-clock ms per step of the same replays, "graph": bool}.
 
-    The steps are captured once into a HIP graph and replayed, so the figure is the GPU's time for back-to-back
-    launches and not the host's launch cadence (a Python -> ctypes launch costs more than the shortest kernels
-    here run). Falls back to direct launches if capture is unavailable."""
+    The K steps are captured once into a HIP graph; the graph is replayed `replays` times and every replay (exactly
+    K steps) is timed on its own, so the figure is the GPU's time for back-to-back launches and not the host's launch
+    cadence (a Python -> ctypes launch costs more than the shortest kernels here run). Falls back to direct launches
+    if capture is unavailable."""
     for i in range(warmup):
         wl.step(i)
     torch.cuda.synchronize()
@@ -422,18 +487,32 @@ def measure(torch, wl, steps, warmup, use_graph=True):
             print("# graph capture failed (%s); timing direct launches" % exc, file=sys.stderr)
             graph = None
             torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(replays)]
     t0 = time.perf_counter()
-    e0.record()
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(steps):
-            wl.step(warmup + i)
-    e1.record()
+    for e0, e1 in events:
+        e0.record()
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                wl.step(warmup + i)
+        e1.record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return e0.elapsed_time(e1) / steps, wall_ms, graph is not None
+    wall_ms = (time.perf_counter() - t0) * 1e3 / (steps * replays)
+    per = sorted(e0.elapsed_time(e1) / steps for e0, e1 in events)
+    return {"ms": per[len(per) // 2], "min": per[0], "max": per[-1], "wall": wall_ms, "graph": graph is not None,
+            "replays": replays}
+
+
+def measure_hot(torch, wl, steps, warmup, use_graph):
+    """The same steps on ONE buffer set (what the Infinity Cache serves when the set fits in it), or None."""
+    if wl.bound != "hbm" or not wl.sets or len(wl.sets) < 2:
+        return None
+    all_sets, wl.sets = wl.sets, wl.sets[:1]
+    try:
+        return measure(torch, wl, steps, warmup, use_graph, replays=3)
+    finally:
+        wl.sets = all_sets
 
 
 PROFILE_KEYS = {"norms_f16_8192x4096": "norms", "softmax_f32_4096x1024": "softmax", "gemm_f16_4096": "gemm",
@@ -469,6 +548,75 @@ def steps_for(wl, steps):
     return steps
 
 
+def entry_for(torch, wl, m, hot, cores, with_cpu):
+    entry = {"workload": wl.name, "ms": round(m["ms"], 5), "ms_min": round(m["min"], 5), "ms_max": round(m["max"], 5),
+             "replays": m["replays"]}
+    entry.update(report(wl, m["ms"]))
+    entry["frac_best"] = round(report(wl, m["min"])["frac"], 4)
+    if hot is not None:
+        entry["hot"] = {"ms": round(hot["ms"], 5), "frac": report(wl, hot["ms"])["frac"],
+                        "note": "one buffer set: Infinity-Cache resident where it fits, not an HBM figure"}
+    if wl.name == "w8a16_m256":
+        # 23 GFLOP: this shape is matrix-bound, not weight-stream-bound; both fractions are reported
+        flop = 2.0 * 256 * 11008 * 4096
+        entry["mfma_frac"] = round(flop / (m["ms"] * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)
+    if with_cpu:
+        sec, sample = wl.cpu(torch)
+        if sec == sec:                                  # not NaN
+            entry["cpu"] = {"ms": round(sec * 1e3, 3), "cores": cores, "sample": sample,
+                            "value": round(wl.work / sec / (1e9 if wl.bound == "hbm" else 1e12), 4)}
+    return entry
+
+
+def direct_launch_cost(torch, wl, steps=300):
+    """Host wall-clock per call (us) of direct launches from Python, GPU idle-waited only at the end."""
+    for i in range(20):
+        wl.step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        wl.step(i)
+    host = (time.perf_counter() - t0) * 1e6 / steps     # time to enqueue
+    torch.cuda.synchronize()
+    total = (time.perf_counter() - t0) * 1e6 / steps    # enqueue + drain
+    return {"host_us_per_call": round(host, 2), "wall_us_per_call": round(total, 2)}
+
+
+def run_peak(torch, hexmi, args):
+    """--workload mfma_peak: one JSON line with the sustained rate of every (dtype, shape, data) combination."""
+    rows = []
+    for wl in peak_workloads():
+        wl.setup(torch, hexmi)
+        wl.step(0)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        wl.step(0)
+        e1.record()
+        torch.cuda.synchronize()
+        one = e0.elapsed_time(e1)
+        k = max(5, int(math.ceil(1000.0 / max(one, 1e-3) / REPLAYS)))    # >= 1 s of back-to-back launches in all
+        m = measure(torch, wl, k, 2, not args.no_graph)
+        r = report(wl, m["ms"])
+        rows.append({"workload": wl.name, "description": wl.desc, "ms": round(m["ms"], 4), "ms_min": round(m["min"], 4),
+                     "launches": k * m["replays"], "sustained_s": round(m["ms"] * k * m["replays"] / 1e3, 2),
+                     "achieved": r["achieved"], "unit": r["unit"], "frac": r["frac"],
+                     "frac_best": report(wl, m["min"])["frac"],
+                     "equivalent_clock_ghz": round(r["frac"] * 2.4, 3)})
+        print("# %s: %.1f TFLOP/s (%.3f of peak)" % (wl.name, r["achieved"], r["frac"]), file=sys.stderr, flush=True)
+    best = max(rows, key=lambda r: r["achieved"])
+    line = {"metric": "GEMM/attn TFLOP/s + softmax/norm GB/s, % of MI355X roofline, 1 GPU", "value": best["achieved"],
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": best["ms"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16/bf16", "data": "synthetic",
+            "config": {"workload": "mfma_peak", "description": "registers-only MFMA streams, a calibration of the "
+                       "matrix cores' data-dependent ceiling, not a product kernel; equivalent_clock_ghz = fraction "
+                       "of the published peak x the 2.4 GHz it is quoted at"},
+            "roofline": {"bound": "mfma", "achieved": best["achieved"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": best["frac"], "traffic": None, "kernel": "mfma_peak_kernel"},
+            "mfma_peak": rows}
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -478,6 +626,7 @@ def main():
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time direct launches instead of a HIP graph replay")
+    ap.add_argument("--only", default="", help="comma-separated suite entries to measure (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -492,22 +641,32 @@ def main():
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
 
+    if args.workload == "mfma_peak":
+        return run_peak(torch, hexmi, args)
+
     wls = make_workloads()
     primary = wls[ALIASES.get(args.workload, args.workload)]
     primary.setup(torch, hexmi)
-    ms, wall_ms, graphed = measure(torch, primary, args.steps, args.warmup, not args.no_graph)
-    roof = report(primary, ms)
+    m = measure(torch, primary, args.steps, args.warmup, not args.no_graph)
+    hot = measure_hot(torch, primary, args.steps, args.warmup, not args.no_graph)
+    roof = report(primary, m["ms"])
     unit = roof["unit"]
     line = {
         "metric": "GEMM/attn TFLOP/s + softmax/norm GB/s, % of MI355X roofline, 1 GPU",
         "value": roof["achieved"], "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 5), "wall_ms_per_step": round(wall_ms, 5), "higher_is_better": True,
+        "ms_per_step": round(m["ms"], 5), "ms_per_step_min": round(m["min"], 5), "ms_per_step_max": round(m["max"], 5),
+        "timed_replays": m["replays"], "wall_ms_per_step": round(m["wall"], 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": primary.dtype, "data": "synthetic",
         "config": {"workload": primary.name, "description": primary.desc,
                    "buffers": "%d rotated sets" % len(primary.sets),
-                   "launch": "hip graph replay" if graphed else "direct"},
+                   "launch": "hip graph replay" if m["graph"] else "direct",
+                   "timing": "median of %d replays of the %d-step graph, each replay timed with HIP events"
+                             % (m["replays"], args.steps)},
         "roofline": roof,
     }
+    if hot is not None:
+        line["hot_cache"] = {"ms_per_step": round(hot["ms"], 5), "frac": report(primary, hot["ms"])["frac"],
+                             "note": "one buffer set (Infinity-Cache resident where it fits); not the HBM claim"}
     if not args.no_cpu:
         sec, sample = primary.cpu(torch)
         cpu_val = primary.work / sec / (1e9 if primary.bound == "hbm" else 1e12)
@@ -517,25 +676,33 @@ def main():
     torch.cuda.empty_cache()
 
     if not args.no_suite:
-        suite = []
+        suite, only = [], [ALIASES.get(n, n) for n in args.only.split(",") if n]
         for name, wl in wls.items():
-            if wl is primary or name in ("norms_f16_8192x4096", "copy_64MiB"):
+            if wl is primary or name in ("norms_f16_8192x4096", "copy_64MiB") or (only and name not in only):
                 continue
             print("# measuring %s" % name, file=sys.stderr, flush=True)
             wl.setup(torch, hexmi)
             k = steps_for(wl, args.steps)
-            wms, _, _ = measure(torch, wl, k, args.warmup, not args.no_graph)
-            entry = {"workload": name, "ms": round(wms, 5), "steps": k}
-            entry.update(report(wl, wms))
-            if not args.no_cpu:
-                sec, sample = wl.cpu(torch)
-                entry["cpu"] = {"ms": round(sec * 1e3, 3), "cores": cores, "sample": sample,
-                                "value": round(wl.work / sec / (1e9 if wl.bound == "hbm" else 1e12), 4)}
+            wm = measure(torch, wl, k, args.warmup, not args.no_graph)
+            whot = measure_hot(torch, wl, k, args.warmup, not args.no_graph)
+            entry = entry_for(torch, wl, wm, whot, cores, not args.no_cpu)
+            entry["steps"] = k
+            if name in ("softmax_f32_4096x1024", "w8a16_m1"):
+                entry["direct_launch"] = direct_launch_cost(torch, wl)
             suite.append(entry)
             wl.sets = None
             wl.host = None
             torch.cuda.empty_cache()
         line["suite"] = suite
+        by_name = {e["workload"]: e for e in suite}
+        targets = []
+        for name, want in TARGETS.items():
+            e = by_name.get(name)
+            if e is not None:
+                targets.append({"workload": name, "frac": e["frac"], "frac_best": e["frac_best"], "target": want,
+                                "met": bool(e["frac"] >= want)})
+        line["targets"] = targets
+        line["targets_met"] = "%d of %d" % (sum(t["met"] for t in targets), len(targets))
     print(json.dumps(line), flush=True)
 
 

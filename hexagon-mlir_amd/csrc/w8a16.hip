@@ -556,7 +556,7 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
                                 void* C, hexmi_stream_t stream) {
   if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
   if (M == 0 || N == 0) return HEXMI_OK;
-  if (!A || !W || !scales || !C) return HEXMI_EINVAL;
+  if (!C || (K > 0 && (!A || !W || !scales))) return HEXMI_EINVAL;
   if (M > 0x7fffffff || N > 0x7fffffff - 16 || K > 0x7fffffff) return HEXMI_ENOTSUP;
   hipStream_t st = as_stream(stream);
   const f16* a = static_cast<const f16*>(A);

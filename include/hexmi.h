@@ -253,6 +253,23 @@ int hexmi_rope(const void *x, void *y, int64_t batch, int64_t seq,
                int64_t heads, int64_t feat, double theta, int dtype,
                hexmi_stream_t stream);
 
+/* Measurement aid -------------------------------------------------------- */
+
+/* A stream of nothing but MFMAs (operands and accumulators in registers, no
+ * memory traffic): what the matrix cores of this GPU sustain for one
+ * instruction shape on operands of the caller's choice. It has no counterpart
+ * in the reference; bench.py uses it to put the data-dependent, power-limited
+ * ceiling of the MFMA-bound kernels on record next to the published peak.
+ * shape: 0 = v_mfma_f32_32x32x16, 1 = v_mfma_f32_16x16x32; dtype HEXMI_F16 or
+ * HEXMI_BF16; operands: 2 KiB, 16-byte aligned (lane l takes its A fragment at
+ * byte 16*l and its B fragment at byte 1024 + 16*l, every wave the same);
+ * waves_per_simd: 1 or 2; one workgroup per compute unit; sink: one float per
+ * thread (hexmi_num_cus() * 256 * waves_per_simd), written once at the end.
+ * hexmi_mfma_peak_flops is the FLOP count of such a launch on this device. */
+double hexmi_mfma_peak_flops(int shape, int waves_per_simd, int64_t iters);
+int hexmi_mfma_peak(int shape, int dtype, const void *operands, int64_t iters,
+                    int waves_per_simd, float *sink, hexmi_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
