@@ -43,6 +43,8 @@ SIGNATURES = {
     "hexmi_block_sum": (_int, [_ptr, _ptr, _i64, _i64, _int, _ptr]),
     "hexmi_block_sum_workspace": (_i64, [_i64, _i64, _int]),
     "hexmi_block_sum_ws": (_int, [_ptr, _ptr, _i64, _i64, _int, _ptr, _i64, _ptr]),
+    "hexmi_block_sum_static_max_n": (_i64, []),
+    "hexmi_block_sum_static": (_int, [_ptr, _ptr, _i64, _i64, _int, _ptr]),
     "hexmi_rope": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _f64, _int, _ptr]),
     "hexmi_mfma_peak_flops": (_f64, [_int, _int, _i64]),
     "hexmi_mfma_peak": (_int, [_int, _int, _ptr, _i64, _int, _ptr, _ptr]),

@@ -244,6 +244,20 @@ int hexmi_block_sum_ws(const void *x, void *out, int64_t n, int64_t block,
                        int dtype, void *workspace, int64_t workspace_bytes,
                        hexmi_stream_t stream);
 
+/* hexmi_block_sum_ws without the workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc). It has no counterpart in the reference.
+ * The partial sums live in a fixed 1 MiB device array of the library (one
+ * copy per GPU, held until the process ends), which bounds the input:
+ * n <= hexmi_block_sum_static_max_n() = 2^30 elements, HEXMI_ETOOBIG beyond.
+ * Same kernels and same results, bit for bit, as hexmi_block_sum_ws with a
+ * workspace. The call allocates and frees nothing. Every call on one GPU uses
+ * that GPU's one array: two calls that overlap on the same GPU (different
+ * streams or threads) race; calls on one stream are ordered and safe. */
+int64_t hexmi_block_sum_static_max_n(void);
+int hexmi_block_sum_static(const void *x, void *out, int64_t n, int64_t block,
+                           int dtype, hexmi_stream_t stream);
+
 /* Rotary position embedding of x [batch, seq, heads, feat] (contiguous, feat
  * even): adjacent feature pairs (2i, 2i+1) are rotated by m * theta^(-2i/feat),
  * m the sequence position: `rope_kernel` of test/python/triton/test_rope.py:97-197
