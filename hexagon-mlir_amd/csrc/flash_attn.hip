@@ -14,8 +14,6 @@
 //
 // fp32 inputs with head size 64 or 128 run the fp32 matrix-core kernels of flash_attn_f32.hip; other head sizes and
 // unaligned operands take the plain one-wave-per-query-row kernel below.
-#include <cstdlib>
-#include <type_traits>
 #include "flash_attn_tiles.h"
 
 namespace hexmi {
@@ -542,14 +540,7 @@ int dispatch_half(const void* Q, const void* K, const void* V, const void* mask,
   const bool ok = aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16) &&
                   Skv * D * (int64_t)sizeof(T) < 0x7fffffff && scale_log2e > 0.0f;
   const bool plain = !mask && Skv == S;
-  if (ok && plain && D == 128) {
-    int status = HEXMI_OK;
-    constexpr int in_dt = std::is_same<T, f16>::value ? HEXMI_F16 : HEXMI_BF16;
-    constexpr int out_dt = std::is_same<OutT, float>::value ? HEXMI_F32 : in_dt;
-    static const bool pipe_off = getenv("HEXMI_ATTN_PIPE_OFF") != nullptr;
-    if (!pipe_off && flash_attn_pipe(Q, K, V, O, ZH, S, D, scale_log2e, causal, in_dt, out_dt, st, &status)) return status;
-    return launch_mfma<T, OutT, 128>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
-  }
+  if (ok && plain && D == 128) return launch_mfma<T, OutT, 128>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
   if (ok && plain && D == 64) return launch_mfma<T, OutT, 64>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
   const bool general_ok = ok && !causal && Skv % 4 == 0 && Skv >= 4 && (!mask || aligned_to(mask, 8));
   if (general_ok && D == 128) return launch_mfma_general<T, OutT, 128>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);

@@ -1,4 +1,4 @@
-// Pieces shared by the 16-bit flash-attention kernels (flash_attn.hip, flash_attn_pipe.hip): MFMA wrappers, the
+// Pieces of the 16-bit flash-attention kernels (flash_attn.hip): MFMA wrappers, the
 // swizzled [64 keys][D] LDS tile and its global -> LDS loader, half-wave exchange, 4-element stores.
 #pragma once
 #include "hexmi_common.h"

@@ -198,12 +198,6 @@ int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t
 bool gemm_f32_mfma(bool trans_b, const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K,
                    int64_t lda, int64_t ldb, int64_t ldc, hipStream_t stream, int* status);
 
-// 16-bit flash attention with the softmax of one row tile pipelined under the MFMAs of the other inside each wave
-// (flash_attn_pipe.hip): launches and returns true when the shape fits (D = 128, S % 64 == 0, enough 256-row
-// units to fill the chip), with the launch status in *status.
-bool flash_attn_pipe(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, int64_t D,
-                     float scale_log2e, bool causal, int in_dtype, int out_dtype, hipStream_t stream, int* status);
-
 // fp32 flash attention on the fp32 matrix cores (flash_attn_f32.hip): launches and returns true when the shapes fit
 // (head size 64 or 128, aligned operands), with the launch status in *status.
 bool flash_attn_f32_mfma(const float* Q, const float* K, const float* V, const float* mask, float* O, int64_t ZH,
