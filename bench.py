@@ -396,6 +396,86 @@ class MaskedAttention(Workload):
         return t * (B / n), "%d of %d batch entries, fp32 F.scaled_dot_product_attention(attn_mask=...) on CPU, time scaled" % (n, B)
 
 
+class LinearFused(Workload):
+    """A GPT-2 style projection with bias and residual: one launch (hexmi_gemm_ex) against the same result from the
+    GEMM followed by two element-wise add launches."""
+    bound, kernel, dtype = "mfma", "gemm_kernel_k64", "f16"
+    launches_separate = 3
+
+    def __init__(self, M=8192, N=768, K=3072):
+        self.M, self.N, self.K = M, N, K
+        self.name = "linear_bias_residual_f16_%dx%dx%d" % (M, N, K)
+        self.desc = ("C = A[%d,%d].B[%d,%d] + bias[%d] + residual[%d,%d], fp16, fp32 accumulate, one rounding; "
+                     "the GPT-2 small MLP projection over 8 sequences of 1024 tokens" % (M, K, K, N, N, M, N))
+
+    def setup(self, torch, hexmi):
+        g = torch.Generator().manual_seed(7)
+        self.hexmi = hexmi
+        self.host = {"a": torch.rand(self.M, self.K, generator=g).mul_(2).sub_(1).half(),
+                     "b": torch.rand(self.K, self.N, generator=g).mul_(2).sub_(1).half(),
+                     "bias": torch.rand(self.N, generator=g).half(),
+                     "resid": torch.rand(self.M, self.N, generator=g).half()}
+        self.work = 2.0 * self.M * self.N * self.K
+        self.sets = _sets(torch, self.host, 0, rotate=False)
+        s = self.sets[0]
+        s["out"] = torch.empty(self.M, self.N, dtype=torch.float16, device="cuda")
+        s["tmp"] = torch.empty_like(s["out"])
+        s["bias_rows"] = s["bias"].expand(self.M, self.N).contiguous()
+
+    def step(self, i):
+        s = self.sets[0]
+        self.hexmi.matmul(s["a"], s["b"], out=s["out"], bias=s["bias"], residual=s["resid"])
+
+    def step_separate(self, i):
+        s = self.sets[0]
+        self.hexmi.matmul(s["a"], s["b"], out=s["tmp"])
+        self.hexmi.binary("add", s["tmp"], s["bias_rows"], out=s["tmp"])
+        self.hexmi.binary("add", s["tmp"], s["resid"], out=s["out"])
+
+    def cpu(self, torch):
+        a, b = self.host["a"].float(), self.host["b"].float()
+        bias, resid = self.host["bias"].float(), self.host["resid"].float()
+        rows = self.M // 8
+        t = _time_cpu(lambda: torch.addmm(resid[:rows] + bias, a[:rows], b), 2)
+        return t * 8, "rows 0..%d of %d, fp32 torch.addmm on CPU, time scaled to the full product" % (rows, self.M)
+
+
+class AddMatmulSoftmax(Workload):
+    """softmax((x + y) z) in one launch against add -> GEMM -> softmax (three launches)."""
+    bound, kernel = "mfma", "add_matmul_softmax_kernel"
+    launches_separate = 3
+
+    def __init__(self, M, N, K, dtype_name):
+        self.M, self.N, self.K, self.dtype = M, N, K, dtype_name
+        self.name = "add_matmul_softmax_%s_%dx%dx%d" % (dtype_name, M, N, K)
+        self.desc = "softmax((x + y)[%d,%d] . z[%d,%d]) over rows, %s, N(0,1) inputs" % (M, K, K, N, dtype_name)
+
+    def setup(self, torch, hexmi):
+        dt = {"f16": torch.float16, "f32": torch.float32}[self.dtype]
+        if self.dtype == "f32":
+            self.peak = MFMA_F32_PEAK_TFLOPS
+        g = torch.Generator().manual_seed(9)
+        self.hexmi = hexmi
+        self.host = {"x": torch.randn(self.M, self.K, generator=g).to(dt), "y": torch.randn(self.M, self.K, generator=g).to(dt),
+                     "z": torch.randn(self.K, self.N, generator=g).mul_(self.K ** -0.5).to(dt)}
+        self.work = 2.0 * self.M * self.N * self.K
+        self.sets = _sets(torch, self.host, 0, rotate=False)
+        self.sets[0]["out"] = torch.empty(self.M, self.N, dtype=dt, device="cuda")
+
+    def step(self, i):
+        s = self.sets[0]
+        self.hexmi.add_matmul_softmax(s["x"], s["y"], s["z"], out=s["out"], fused=True)
+
+    def step_separate(self, i):
+        s = self.sets[0]
+        self.hexmi.add_matmul_softmax(s["x"], s["y"], s["z"], out=s["out"], fused=False)
+
+    def cpu(self, torch):
+        x, y, z = (self.host[k].float() for k in "xyz")
+        t = _time_cpu(lambda: torch.softmax((x + y) @ z, dim=-1), 5)
+        return t, "the whole graph, fp32 torch on CPU"
+
+
 class MfmaPeak(Workload):
     """Registers-only MFMA stream (hexmi_mfma_peak): the rate the matrix cores sustain on given operand data."""
     bound, kernel = "mfma", "mfma_peak_kernel"
@@ -446,7 +526,8 @@ def make_workloads():
         Gemm(4096, "f32"), W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256),
         Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), AttentionF32(4, 32, 2048, 64),
         MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
-        Elementwise("sum"), CopyCalibration())}
+        Elementwise("sum"), LinearFused(), AddMatmulSoftmax(32, 32, 32, "f32"), AddMatmulSoftmax(512, 512, 64, "f16"),
+        CopyCalibration())}
 
 
 def peak_workloads():
@@ -460,7 +541,9 @@ ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "sof
            "attn_f32": "attn_causal_f32_4x32x2048x64", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
            "rope": "rope_f16_4x4096x32x128", "sum": "block_sum_f32_8192x4096", "rms_norm": "rms_norm_f16_8192x4096",
            "layer_norm": "layer_norm_f16_8192x4096", "w8a16_m1": "w8a16_m1", "w8a16_m16": "w8a16_m16",
-           "w8a16_m64": "w8a16_m64", "w8a16_m256": "w8a16_m256"}
+           "w8a16_m64": "w8a16_m64", "w8a16_m256": "w8a16_m256",
+           "linear": "linear_bias_residual_f16_8192x768x3072", "ams": "add_matmul_softmax_f32_32x32x32",
+           "ams_mid": "add_matmul_softmax_f16_512x512x64"}
 
 
 def measure(torch, wl, steps, warmup, use_graph=True, replays=REPLAYS):
@@ -687,6 +770,13 @@ def main():
             whot = measure_hot(torch, wl, k, args.warmup, not args.no_graph)
             entry = entry_for(torch, wl, wm, whot, cores, not args.no_cpu)
             entry["steps"] = k
+            if getattr(wl, "step_separate", None) is not None:
+                fused_step, wl.step = wl.step, wl.step_separate
+                sm = measure(torch, wl, k, args.warmup, not args.no_graph)
+                wl.step = fused_step
+                entry["separate_launches"] = {"launches": wl.launches_separate, "ms": round(sm["ms"], 5),
+                                              "ms_min": round(sm["min"], 5),
+                                              "speedup_fused": round(sm["ms"] / wm["ms"], 3)}
             if name in ("softmax_f32_4096x1024", "w8a16_m1"):
                 entry["direct_launch"] = direct_launch_cost(torch, wl)
             suite.append(entry)

@@ -176,21 +176,6 @@ __device__ __forceinline__ typename Mfma<T>::Frag read_nmajor(const T* lds, int 
   return u.f;
 }
 
-template <typename OutT>
-__device__ __forceinline__ void store4(OutT* p, float a, float b, float c, float d);
-template <> __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
-  f32x4 v = {a, b, c, d};
-  *reinterpret_cast<f32x4*>(p) = v;
-}
-template <> __device__ __forceinline__ void store4<f16>(f16* p, float a, float b, float c, float d) {
-  f16x4 v = {(f16)a, (f16)b, (f16)c, (f16)d};
-  *reinterpret_cast<f16x4*>(p) = v;
-}
-template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float a, float b, float c, float d) {
-  bf16x4 v = {(bf16)a, (bf16)b, (bf16)c, (bf16)d};
-  *reinterpret_cast<bf16x4*>(p) = v;
-}
-
 // Map the linear workgroup id to a C tile: consecutive ids go to different XCDs (each with its own L2), so
 // first give every XCD a contiguous run of logical ids, then walk tiles in bands of GROUP_M tile-rows so the
 // tiles resident on one XCD share A and B panels.
@@ -209,17 +194,42 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
   tn = in_group / gm;
 }
 
+// Epilogue operands of hexmi_gemm_ex: C = A B + bias[column] + residual[row, column], both of the output type, added
+// to the fp32 sums before the one rounding to the output type. ok4: the four columns col .. col+3 exist and the
+// operands may be read as one 4-element run (the fast kernels: N % 8 == 0, ldr % 4 == 0, aligned bases).
+template <typename OutT> struct Run4;
+template <> struct Run4<float> { typedef f32x4 V; };
+template <> struct Run4<f16> { typedef f16x4 V; };
+template <> struct Run4<bf16> { typedef bf16x4 V; };
+template <typename OutT>
+__device__ __forceinline__ void add_epilogue4(f32x4& a, const OutT* __restrict__ bias, const OutT* __restrict__ resid,
+                                              int64_t ldr, int row, int col) {
+  typedef typename Run4<OutT>::V V;
+  if (bias) {
+    const V b = *reinterpret_cast<const V*>(bias + col);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) a[r] += to_f32<OutT>(b[r]);
+  }
+  if (resid) {
+    const V v = *reinterpret_cast<const V*>(resid + (int64_t)row * ldr + col);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) a[r] += to_f32<OutT>(v[r]);
+  }
+}
+
 // K % 32 == 0. TAIL: the slab count is not a multiple of 4, so the last pass over the four stages guards its MFMAs.
 // B_I8: B is int8 [N,K] (weight-only quantisation, needs TRANS_B and T = fp16); its slabs are copied raw into
 // LDS, converted to fp16 LDS -> LDS one slab later, and the result is multiplied by scales[column].
 // NWN: waves along N (2: four waves, one per SIMD, each WM x WN tiles of 32x32; 4: eight waves, two per SIMD).
 // The eight-wave 256x256 form (WM = 4, WN = 2) measured the same as four waves with 4x4 tiles on both benchmark
 // shapes: on random data the kernel is held back by the power limit, not by issue stalls a second wave could fill.
-template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false, int NWN = 2>
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false, int NWN = 2,
+          bool EPI = false>
 __global__ __launch_bounds__(NWN * 128)
 void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __restrict__ C, int M, int N, int K,
                  int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
-                 const f16* __restrict__ scales = nullptr) {
+                 const f16* __restrict__ scales = nullptr, const OutT* __restrict__ bias = nullptr,
+                 const OutT* __restrict__ resid = nullptr, int64_t ldr = 0) {
   const T* B = static_cast<const T*>(Bv);
   typedef typename Mfma<T>::Frag Frag;
   constexpr int NW = 2 * NWN;                       // waves per workgroup
@@ -385,6 +395,27 @@ void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __r
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));       // drain the trailing copies before the workgroup's LDS goes away
 
   // acc[i][j][r]: row = lane%32 of the 32x32 tile, column = 8*(r/4) + 4*(lane/32) + r%4.
+  if constexpr (EPI) {
+    // bias and residual join the fp32 sums in registers, all loads issued before the first store (so the residual
+    // may be the output buffer itself)
+    static_assert(!B_I8, "the epilogue operands go with fp16 / bf16 B");
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      int row = m0 + (wm * WM + i) * 32 + lane % 32;
+      row = row < M ? row : M - 1;                  // past the edge: any valid row, those rows are not stored
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          int col = n0 + (wn * WN + j) * 32 + 8 * q + 4 * (lane / 32);
+          col = col < N - 4 ? col : N - 4;
+          f32x4 c = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+          add_epilogue4<OutT>(c, bias, resid, ldr, row, col);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[i][j][q * 4 + r] = c[r];
+        }
+    }
+  }
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
     const int row = m0 + (wm * WM + i) * 32 + lane % 32;
@@ -400,8 +431,9 @@ void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __r
             const f16x4 sc = *reinterpret_cast<const f16x4*>(scales + col);
             s0 = (float)sc[0]; s1 = (float)sc[1]; s2 = (float)sc[2]; s3 = (float)sc[3];
           }
-          store4<OutT>(C + (int64_t)row * ldc + col, acc[i][j][q * 4 + 0] * s0, acc[i][j][q * 4 + 1] * s1,
-                       acc[i][j][q * 4 + 2] * s2, acc[i][j][q * 4 + 3] * s3);
+          f32x4 c = {acc[i][j][q * 4 + 0] * s0, acc[i][j][q * 4 + 1] * s1, acc[i][j][q * 4 + 2] * s2,
+                     acc[i][j][q * 4 + 3] * s3};
+          store4<OutT>(C + (int64_t)row * ldc + col, c[0], c[1], c[2], c[3]);
         }
       }
     }
@@ -538,8 +570,8 @@ __device__ __forceinline__ f16x8 widen_i8(u32x2 raw) {
 
 // The accumulator is tied to the destination in inline assembly: left to the compiler, the 16x16x32 builtin gets
 // a destination register of its own and a copy back per instruction. Each accumulator is touched once per 64
-// MFMAs, far beyond the instruction's latency, and the epilogue reads them after the copy drain and its address
-// arithmetic, so no wait states are missing around the assembly.
+// MFMAs, far beyond the instruction's latency; the wait states before the epilogue's first read of an accumulator
+// are spent explicitly after the K loop.
 template <typename T> struct Mfma16;
 template <> struct Mfma16<f16> {
   static __device__ __forceinline__ void run(const f16x8& a, const f16x8& b, f32x4& c) {
@@ -561,11 +593,15 @@ template <> struct Mfma16<bf16> {
 // slab j and after all of slab j+1 has landed. NS = 4 stages (small tiles, whose slabs are too short to cover the
 // memory latency with one slab of lead) fill the stage of slab j with slab j+4 instead. TAIL: the slab count is not
 // a multiple of NS.
-template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false, int NS = 2>
+// EPI: the kernel adds bias and / or a residual in its epilogue (instantiated apart, so the plain product keeps its
+// register allocation).
+template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false, int NS = 2,
+          bool EPI = false>
 __global__ __launch_bounds__(256)
 void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __restrict__ C, int M, int N, int K,
                      int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
-                     const f16* __restrict__ scales = nullptr) {
+                     const f16* __restrict__ scales = nullptr, const OutT* __restrict__ bias = nullptr,
+                     const OutT* __restrict__ resid = nullptr, int64_t ldr = 0) {
   static_assert(!B_I8 || (TRANS_B && sizeof(T) == 2), "int8 B is [N,K] and multiplies fp16 A");
   const T* B = static_cast<const T*>(Bv);
   typedef typename Mfma<T>::Frag Frag;
@@ -598,6 +634,26 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+
+  // Epilogue operands are fetched up front, in the accumulators' layout (a lane's four columns of a row: 8 or 16
+  // bytes), so their latency passes under the K loop instead of at the end of a tile that has nothing left to
+  // overlap it with. Reading before any store of this tile also lets the residual be the output buffer itself.
+  typedef typename Run4<OutT>::V EpiRun;
+  EpiRun resid_frag[EPI ? TM : 1][EPI ? TN : 1], bias_frag[EPI ? TN : 1];
+  if constexpr (EPI) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int col = n0 + (wn * TN + j) * 16 + 4 * (lane / 16);
+      col = col < N - 4 ? col : N - 4;                // past the edge: any valid run, those columns are not stored
+      if (bias) bias_frag[j] = *reinterpret_cast<const EpiRun*>(bias + col);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        int row = m0 + (wm * TM + i) * 16 + lane % 16;
+        row = row < M ? row : M - 1;
+        if (resid) resid_frag[i][j] = *reinterpret_cast<const EpiRun*>(resid + (int64_t)row * ldr + col);
+      }
+    }
+  }
 
   KMajorLoader2<T, BM> load_a;
   load_a.init(lda, m0, M - 1, wave, lane);
@@ -774,6 +830,12 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
   }
 #undef HEXMI_FENCE
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));       // drain the trailing copies before the workgroup's LDS goes away
+  // The MFMAs are assembly, so the compiler does not count the wait states between the last of them and the first
+  // read of an accumulator (19 for the longest matrix instruction): spend them here, fenced so that no accumulator
+  // read is scheduled above them.
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
 
   // acc[i][j][r]: row lane%16 of tile row i, column 4*(lane/16) + r of tile column j
   if constexpr (B_I8) {
@@ -788,6 +850,18 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[i][j][r] *= (float)sc[r];
     }
+  }
+  if constexpr (EPI) {
+    // bias and residual join the fp32 sums in registers, before their one rounding to the output type
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (bias) acc[i][j][r] += to_f32<OutT>(bias_frag[j][r]);
+          if (resid) acc[i][j][r] += to_f32<OutT>(resid_frag[i][j][r]);
+        }
   }
   if constexpr (sizeof(OutT) == 2) {
     if (ldc % 8 == 0) {
@@ -840,7 +914,8 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
 template <typename T, typename OutT, bool TRANS_B>
 __global__ __launch_bounds__(256)
 void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT* __restrict__ C, int M, int N, int K,
-                         int64_t lda, int64_t ldb, int64_t ldc) {
+                         int64_t lda, int64_t ldb, int64_t ldc, const OutT* __restrict__ bias = nullptr,
+                         const OutT* __restrict__ resid = nullptr, int64_t ldr = 0) {
   typedef typename Mfma<T>::Frag Frag;
   constexpr int TB = 64, TK = 16, PAD = 8;
   __shared__ __attribute__((aligned(16))) T a_s[TB][TK + PAD];   // [m][k]
@@ -872,7 +947,12 @@ void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT*
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int col = n0 + wn * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
-    if (col < N) C[(int64_t)row * ldc + col] = from_f32<OutT>(acc[r]);
+    if (col < N) {
+      float c = acc[r];
+      if (bias) c += to_f32<OutT>(bias[col]);
+      if (resid) c += to_f32<OutT>(resid[(int64_t)row * ldr + col]);
+      C[(int64_t)row * ldc + col] = from_f32<OutT>(c);
+    }
   }
 }
 
@@ -883,7 +963,8 @@ void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT*
 template <bool TRANS_B>
 __global__ __launch_bounds__(256)
 void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C, int M, int N,
-                     int K, int64_t lda, int64_t ldb, int64_t ldc) {
+                     int K, int64_t lda, int64_t ldb, int64_t ldc, const float* __restrict__ bias = nullptr,
+                     const float* __restrict__ resid = nullptr, int64_t ldr = 0) {
   constexpr int TB = 64, TK = 16;
   __shared__ float a_s[TK][TB + 4];                  // [k][m]
   __shared__ float b_s[TK][TB + 4];                  // [k][n]
@@ -933,43 +1014,75 @@ void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, f
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int gn = n0 + tx * 4 + j;
-      if (gn < N) C[(int64_t)gm * ldc + gn] = acc[i][j];
+      if (gn < N) {
+        float c = acc[i][j];
+        if (bias) c += bias[gn];
+        if (resid) c += resid[(int64_t)gm * ldr + gn];
+        C[(int64_t)gm * ldc + gn] = c;
+      }
     }
   }
 }
 
 int launch_f32(bool trans_b, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
-               int64_t ldb, int64_t ldc, hipStream_t s) {
+               int64_t ldb, int64_t ldc, hipStream_t s, const void* bias_v = nullptr, const void* resid_v = nullptr,
+               int64_t ldr = 0) {
   const float* a = static_cast<const float*>(A);
   const float* b = static_cast<const float*>(B);
   float* c = static_cast<float*>(C);
+  const float* bias = static_cast<const float*>(bias_v);
+  const float* resid = static_cast<const float*>(resid_v);
   int status = HEXMI_OK;
-  if (gemm_f32_mfma(trans_b, a, b, c, M, N, K, lda, ldb, ldc, s, &status)) return status;   // matrix cores
+  // matrix cores (their kernel has no epilogue operands: a product with bias or residual takes the FMA kernel)
+  if (!bias && !resid && gemm_f32_mfma(trans_b, a, b, c, M, N, K, lda, ldb, ldc, s, &status)) return status;
   dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
   if (grid.y > 65535) return HEXMI_ENOTSUP;
   if (trans_b)
-    hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, s, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc);
+    hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, s, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, bias,
+                       resid, ldr);
   else
-    hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, s, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc);
+    hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, s, a, b, c, (int)M, (int)N, (int)K, lda, ldb, ldc, bias,
+                       resid, ldr);
   return launch_status();
 }
 
 template <typename T, typename OutT, int WM, int WN, bool TRANS_B, int NWN = 2>
 int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
-                 int64_t ldc, hipStream_t s) {
+                 int64_t ldc, hipStream_t s, const OutT* bias, const OutT* resid, int64_t ldr) {
   constexpr int BM = 2 * WM * 32, BN = NWN * WN * 32;
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   // K % 64 == 0: the paired-slab kernel; its per-lane copy offsets (up to 256 rows, or 64 rows of K) must stay
   // below 2^31 bytes
   if (NWN == 2 && K % BK2 == 0 && lda < (1 << 21) && ldb < (1 << 21)) {
     constexpr int NS = WM <= 2 ? 4 : 2;            // small tiles: four stages (their slabs are short)
+    if constexpr (WM == 2 && WN == 2) {
+      if (bias || resid) {                          // the instantiations that carry the epilogue operands
+        if ((K / BK2) % NS == 0)
+          hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, false, false, NS, true>),
+                             dim3(tiles_m * tiles_n), dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc,
+                             tiles_m, tiles_n, nullptr, bias, resid, ldr);
+        else
+          hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, true, false, NS, true>),
+                             dim3(tiles_m * tiles_n), dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc,
+                             tiles_m, tiles_n, nullptr, bias, resid, ldr);
+        return launch_status();
+      }
+    }
     if ((K / BK2) % NS == 0)
       hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, false, false, NS>), dim3(tiles_m * tiles_n),
-                         dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n, nullptr);
+                         dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
     else
       hipLaunchKernelGGL((gemm_kernel_k64<T, OutT, WM, WN, TRANS_B, true, false, NS>), dim3(tiles_m * tiles_n),
-                         dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n, nullptr);
+                         dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n);
     return launch_status();
+  }
+  if constexpr (WM == 2 && WN == 2) {
+    if (bias || resid) {
+      hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, true, false, NWN, true>), dim3(tiles_m * tiles_n),
+                         dim3(NWN * 128), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, tiles_m, tiles_n, nullptr,
+                         bias, resid, ldr);
+      return launch_status();
+    }
   }
   if ((K / BK) % 4 == 0)
     hipLaunchKernelGGL((gemm_kernel<T, OutT, WM, WN, TRANS_B, false, false, NWN>), dim3(tiles_m * tiles_n),
@@ -982,31 +1095,39 @@ int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t 
 
 template <typename T, typename OutT, bool TRANS_B>
 int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N, int64_t K, int64_t lda,
-                  int64_t ldb, int64_t ldc, hipStream_t s) {
+                  int64_t ldb, int64_t ldc, hipStream_t s, const void* bias_v, const void* resid_v, int64_t ldr) {
   const T* A = static_cast<const T*>(Av);
   const T* B = static_cast<const T*>(Bv);
   OutT* C = static_cast<OutT*>(Cv);
+  const OutT* bias = static_cast<const OutT*>(bias_v);
+  const OutT* resid = static_cast<const OutT*>(resid_v);
   // The tiled kernels copy 16-byte chunks and clamp (never mask) rows / column chunks, so they need whole
-  // chunks: K % 32 == 0, leading dimensions and N multiples of 8 elements, 16-byte aligned bases.
+  // chunks: K % 32 == 0, leading dimensions and N multiples of 8 elements, 16-byte aligned bases. Their epilogue
+  // reads bias and residual in runs of four columns.
+  const size_t run = 4 * sizeof(OutT);
   const bool fast = K % BK == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && N % 8 == 0 && N >= 8 &&
-                    aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(C, 16);
+                    aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(C, 16) && (!bias || aligned_to(bias, run)) &&
+                    (!resid || (aligned_to(resid, run) && ldr % 4 == 0));
   if (fast) {
     const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-    if (big_tiles >= 128) return launch_tiled<T, OutT, 4, 4, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s);
-    return launch_tiled<T, OutT, 2, 2, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s);
+    // the large-tile kernels sit at the register limit and carry no epilogue operands: a product with bias or
+    // residual runs on the 128x128 tiles at any size
+    if (big_tiles >= 128 && !bias && !resid)
+      return launch_tiled<T, OutT, 4, 4, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s, nullptr, nullptr, 0);
+    return launch_tiled<T, OutT, 2, 2, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s, bias, resid, ldr);
   }
   dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
   if (grid.y > 65535) return HEXMI_ENOTSUP;
   hipLaunchKernelGGL((gemm_kernel_generic<T, OutT, TRANS_B>), grid, dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K,
-                     lda, ldb, ldc);
+                     lda, ldb, ldc, bias, resid, ldr);
   return launch_status();
 }
 
 template <typename T, typename OutT>
 int dispatch_trans(bool trans_b, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
-                   int64_t ldb, int64_t ldc, hipStream_t s) {
-  return trans_b ? dispatch_gemm<T, OutT, true>(A, B, C, M, N, K, lda, ldb, ldc, s)
-                 : dispatch_gemm<T, OutT, false>(A, B, C, M, N, K, lda, ldb, ldc, s);
+                   int64_t ldb, int64_t ldc, hipStream_t s, const void* bias, const void* resid, int64_t ldr) {
+  return trans_b ? dispatch_gemm<T, OutT, true>(A, B, C, M, N, K, lda, ldb, ldc, s, bias, resid, ldr)
+                 : dispatch_gemm<T, OutT, false>(A, B, C, M, N, K, lda, ldb, ldc, s, bias, resid, ldr);
 }
 
 template <int WM, int WN>
@@ -1066,28 +1187,35 @@ int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t
 
 using namespace hexmi;
 
-extern "C" int hexmi_gemm(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb,
-                          void* C, int64_t ldc, int in_dtype, int out_dtype, int trans_b, hexmi_stream_t stream) {
+extern "C" int hexmi_gemm_ex(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb,
+                             void* C, int64_t ldc, const void* bias, const void* residual, int64_t ldr, int in_dtype,
+                             int out_dtype, int trans_b, hexmi_stream_t stream) {
   if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
   if (M == 0 || N == 0) return HEXMI_OK;
   if (!C || (K > 0 && (!A || !B))) return HEXMI_EINVAL;
-  if (lda < K || ldc < N || ldb < (trans_b ? K : N)) return HEXMI_EINVAL;
+  if (lda < K || ldc < N || ldb < (trans_b ? K : N) || (residual && ldr < N)) return HEXMI_EINVAL;
   if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return HEXMI_ENOTSUP;
   hipStream_t s = as_stream(stream);
   begin_call();
-  if (K == 0) {                                              // an empty sum: C = 0, as torch.matmul gives
+  if (K == 0 && !bias && !residual) {                        // an empty sum: C = 0, as torch.matmul gives
     const int esz = dtype_size(out_dtype);
     const bool known = (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) ||
                        ((in_dtype == HEXMI_F16 || in_dtype == HEXMI_BF16) && (out_dtype == in_dtype || out_dtype == HEXMI_F32));
     return known ? fill_zero_2d(C, M, N, ldc, esz, s) : HEXMI_ENOTSUP;
   }
+  if (K == 0) return HEXMI_ENOTSUP;                          // bias / residual of an empty product: not provided
   const bool tb = trans_b != 0;
-  if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) return launch_f32(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
-  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F16) return dispatch_trans<f16, f16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
-  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F32) return dispatch_trans<f16, float>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
-  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_BF16) return dispatch_trans<bf16, bf16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
-  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_F32) return dispatch_trans<bf16, float>(tb, A, B, C, M, N, K, lda, ldb, ldc, s);
+  if (in_dtype == HEXMI_F32 && out_dtype == HEXMI_F32) return launch_f32(tb, A, B, C, M, N, K, lda, ldb, ldc, s, bias, residual, ldr);
+  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F16) return dispatch_trans<f16, f16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s, bias, residual, ldr);
+  if (in_dtype == HEXMI_F16 && out_dtype == HEXMI_F32) return dispatch_trans<f16, float>(tb, A, B, C, M, N, K, lda, ldb, ldc, s, bias, residual, ldr);
+  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_BF16) return dispatch_trans<bf16, bf16>(tb, A, B, C, M, N, K, lda, ldb, ldc, s, bias, residual, ldr);
+  if (in_dtype == HEXMI_BF16 && out_dtype == HEXMI_F32) return dispatch_trans<bf16, float>(tb, A, B, C, M, N, K, lda, ldb, ldc, s, bias, residual, ldr);
   return HEXMI_ENOTSUP;
+}
+
+extern "C" int hexmi_gemm(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb,
+                          void* C, int64_t ldc, int in_dtype, int out_dtype, int trans_b, hexmi_stream_t stream) {
+  return hexmi_gemm_ex(M, N, K, A, lda, B, ldb, C, ldc, nullptr, nullptr, 0, in_dtype, out_dtype, trans_b, stream);
 }
 
 extern "C" int hexmi_matmul_f16f16_f32(int64_t n_row, int64_t n_col, int64_t n_inner, float* out, const void* act,

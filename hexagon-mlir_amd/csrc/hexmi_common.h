@@ -34,6 +34,22 @@ template <> __device__ __forceinline__ float from_f32<float>(float v) { return v
 template <> __device__ __forceinline__ f16 from_f32<f16>(float v) { return (f16)v; }   // round-to-nearest-even
 template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return (bf16)v; }  // round-to-nearest-even
 
+// four consecutive elements, rounded once to the output type, in one store (p aligned to 4 elements)
+template <typename OutT>
+__device__ __forceinline__ void store4(OutT* p, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
+  f32x4 v = {a, b, c, d};
+  *reinterpret_cast<f32x4*>(p) = v;
+}
+template <> __device__ __forceinline__ void store4<f16>(f16* p, float a, float b, float c, float d) {
+  f16x4 v = {(f16)a, (f16)b, (f16)c, (f16)d};
+  *reinterpret_cast<f16x4*>(p) = v;
+}
+template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float a, float b, float c, float d) {
+  bf16x4 v = {(bf16)a, (bf16)b, (bf16)c, (bf16)d};
+  *reinterpret_cast<bf16x4*>(p) = v;
+}
+
 // ---- wavefront reductions -----------------------------------------------
 // Butterfly over the 64 lanes on the vector ALU (no LDS round trips): DPP exchanges inside a row of 16 lanes
 // (quad permutes for lane^1 and lane^2; the half-row and row mirrors stand in for lane^4 and lane^8 because the

@@ -33,6 +33,10 @@ SIGNATURES = {
     "hexmi_layer_norm": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _f32, _int, _ptr]),
     "hexmi_matmul_f16f16_f32": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_gemm": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _int, _int, _ptr]),
+    "hexmi_gemm_ex": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _int, _int,
+                             _ptr]),
+    "hexmi_add_matmul_softmax_max_n": (_i64, []),
+    "hexmi_add_matmul_softmax": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _ptr]),
     "hexmi_gemm_w8a16": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_pack_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr]),
     "hexmi_gemm_w8a16_packed": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),

@@ -63,6 +63,8 @@ _LIBDEF.define("rms_norm(Tensor x, Tensor? weight, float eps, Tensor(a!) out) ->
 _LIBDEF.define("layer_norm(Tensor x, Tensor? weight, Tensor? bias, float eps, Tensor(a!) out, "
                "Tensor(b!)? mean, Tensor(c!)? rstd) -> ()")
 _LIBDEF.define("matmul(Tensor a, Tensor b, bool trans_b, Tensor(a!) out) -> ()")
+_LIBDEF.define("linear(Tensor a, Tensor b, Tensor? bias, Tensor? residual, bool trans_b, Tensor(a!) out) -> ()")
+_LIBDEF.define("add_matmul_softmax(Tensor x, Tensor y, Tensor z, Tensor(a!) out) -> ()")
 _LIBDEF.define("w8a16_matmul(Tensor a, Tensor w, Tensor scales, Tensor(a!) out) -> ()")
 _LIBDEF.define("dequant_w8(Tensor w, Tensor scales, Tensor(a!) out) -> ()")
 _LIBDEF.define("pack_w8(Tensor w, Tensor(a!) out) -> ()")
@@ -102,6 +104,24 @@ def _matmul_impl(a, b, trans_b, out):
     with _on(a.device):
         _lib.check(_lib.lib().hexmi_gemm(M, N, K, _p(a), a.stride(0), _p(b), b.stride(0), _p(out), out.stride(0),
                                          _dt(a), _dt(out), 1 if trans_b else 0, _stream()), "hexmi_gemm")
+
+
+def _linear_impl(a, b, bias, residual, trans_b, out):
+    M, K = a.shape
+    N = b.shape[0] if trans_b else b.shape[1]
+    with _on(a.device):
+        _lib.check(_lib.lib().hexmi_gemm_ex(M, N, K, _p(a), a.stride(0), _p(b), b.stride(0), _p(out), out.stride(0),
+                                            _p(bias), _p(residual), residual.stride(0) if residual is not None else 0,
+                                            _dt(a), _dt(out), 1 if trans_b else 0, _stream()), "hexmi_gemm_ex")
+
+
+def _add_matmul_softmax_impl(x, y, z, out):
+    M, K = x.shape
+    N = z.shape[1]
+    with _on(x.device):
+        _lib.check(_lib.lib().hexmi_add_matmul_softmax(M, N, K, _p(x), x.stride(0), _p(y), y.stride(0), _p(z),
+                                                       z.stride(0), _p(out), out.stride(0), _dt(x), _stream()),
+                   "hexmi_add_matmul_softmax")
 
 
 def _w8a16_impl(a, w, scales, out):
@@ -176,7 +196,8 @@ def _rope_impl(x, theta, out):
 
 
 for _name, _fn in (("softmax", _softmax_impl), ("rms_norm", _rms_norm_impl), ("layer_norm", _layer_norm_impl),
-                   ("matmul", _matmul_impl), ("w8a16_matmul", _w8a16_impl), ("dequant_w8", _dequant_impl), ("pack_w8", _pack_impl),
+                   ("matmul", _matmul_impl), ("linear", _linear_impl), ("add_matmul_softmax", _add_matmul_softmax_impl),
+                   ("w8a16_matmul", _w8a16_impl), ("dequant_w8", _dequant_impl), ("pack_w8", _pack_impl),
                    ("w8a16_matmul_packed", _w8a16_packed_impl),
                    ("flash_attention", _flash_impl), ("attention", _attention_impl),
                    ("unary", _unary_impl), ("binary", _binary_impl), ("block_sum", _block_sum_impl),
@@ -278,10 +299,14 @@ def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=No
     return _finish(od, out)
 
 
-def matmul(a, b, out=None, out_dtype=None, trans_b=False):
+def matmul(a, b, out=None, out_dtype=None, trans_b=False, bias=None, residual=None):
     """C = A @ B (or A @ B.T when trans_b), fp16/bf16 inputs with fp32 accumulation on the matrix cores, or fp32
-    inputs with fp32 FMAs. out_dtype: the input dtype (default) or torch.float32
-    (test/python/triton/test_matmul.py:35-91; docs/tutorials/triton/matmul_hexkl.md:61-111)."""
+    inputs multiplied in fp32. out_dtype: the input dtype (default) or torch.float32
+    (test/python/triton/test_matmul.py:35-91; docs/tutorials/triton/matmul_hexkl.md:61-111).
+    bias [N] and residual [M,N] (of the output dtype) are added to the fp32 sums inside the GEMM kernel, the way the
+    reference's fusion pass pulls the consumers of a matmul into its loop nest
+    (qcom_hexagon_backend/lib/Conversion/LinalgToLLVM/LinalgToLLVMPass.cpp:280-283): C = A @ B + bias + residual
+    with one rounding and no extra launch."""
     if a.dim() != 2 or b.dim() != 2:
         raise ValueError("hexmi.matmul takes 2-D tensors")
     if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16, torch.float32):
@@ -294,10 +319,17 @@ def matmul(a, b, out=None, out_dtype=None, trans_b=False):
         raise ValueError("hexmi.matmul: inner dimensions differ: %s x %s" % (tuple(a.shape), tuple(b.shape)))
     if out_dtype is None:
         out_dtype = out.dtype if out is not None else a.dtype
+    if bias is not None and (bias.shape != (N,) or bias.dtype != out_dtype):
+        raise ValueError("hexmi.matmul: bias must be [N] of the output dtype")
+    if residual is not None and (residual.shape != (M, N) or residual.dtype != out_dtype):
+        raise ValueError("hexmi.matmul: residual must be [M,N] of the output dtype")
     dev = _device() if a.device.type != "cuda" else a.device
     ad, bd = _stage(a, dev), _stage(b, dev)
     od = _out_like(out, (M, N), out_dtype, dev)
-    _matmul_impl(ad, bd, bool(trans_b), od)
+    if bias is None and residual is None:
+        _matmul_impl(ad, bd, bool(trans_b), od)
+    else:
+        _linear_impl(ad, bd, _stage(bias, dev), _stage(residual, dev), bool(trans_b), od)
     return _finish(od, out)
 
 
@@ -468,14 +500,33 @@ def rope(x, theta=10000.0, out=None):
     return _finish(od, out)
 
 
-def add_matmul_softmax(x, y, z, out=None):
+# Above this much multiply-add work the one-launch kernel (32 rows per workgroup, so few workgroups on small
+# problems, and scalar guarded copies) loses to add -> tiled GEMM -> softmax: measured 5.9 us against 6.2 us at
+# 32x32x32, 29 us against 10 us at 512x512x64. Below it the two saved launches and round trips win.
+_FUSED_MAX_MACS = 1 << 20
+
+
+def add_matmul_softmax(x, y, z, out=None, fused=None):
     """softmax((x + y) @ z, dim=-1): the graph of test/python/torch-mlir/test_add_matmul_softmax.py:19-29, which the
-    reference compiles into one fused kernel; here the three kernels run back to back on one stream."""
+    reference compiles into one fused kernel. One launch (`hexmi_add_matmul_softmax`) when the result has at most
+    1024 columns and the product is small; otherwise the three kernels run back to back on one stream.
+    fused=True / False forces one or the other."""
     if x.shape != y.shape or x.dim() != 2 or z.dim() != 2 or x.shape[1] != z.shape[0]:
         raise ValueError("hexmi.add_matmul_softmax: x, y [M,K] and z [K,N] required")
-    if not (x.dtype == y.dtype == z.dtype):
-        raise TypeError("hexmi.add_matmul_softmax: operand dtypes differ")
+    if not (x.dtype == y.dtype == z.dtype) or x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise TypeError("hexmi.add_matmul_softmax: x, y, z must share one of float16, bfloat16, float32")
     dev = _device() if x.device.type != "cuda" else x.device
+    M, K = x.shape
+    N = z.shape[1]
+    fits = 0 < N <= _lib.lib().hexmi_add_matmul_softmax_max_n()
+    if fused is None:
+        fused = fits and M * N * K <= _FUSED_MAX_MACS
+    if fused:
+        if not fits:
+            raise ValueError("hexmi.add_matmul_softmax: the one-launch kernel takes at most 1024 columns")
+        od = _out_like(out, (M, N), x.dtype, dev)
+        _add_matmul_softmax_impl(_stage(x, dev), _stage(y, dev), _stage(z, dev), od)
+        return _finish(od, out)
     total = binary("add", _stage(x, dev), _stage(y, dev))
     product = matmul(total, _stage(z, dev))
     return softmax(product, out=out)

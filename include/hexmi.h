@@ -116,6 +116,42 @@ int hexmi_gemm(int64_t M, int64_t N, int64_t K, const void *A, int64_t lda,
                const void *B, int64_t ldb, void *C, int64_t ldc, int in_dtype,
                int out_dtype, int trans_b, hexmi_stream_t stream);
 
+/* hexmi_gemm with the additions of a linear layer fused into its epilogue:
+ *   C[m,n] = sum_k A[m,k] * op(B)[k,n] + bias[n] + residual[m,n].
+ * bias ([N], contiguous) and residual ([M,N], leading dim ldr) are of the
+ * OUTPUT dtype, either may be NULL; both join the fp32 sums in registers and
+ * the result is rounded to out_dtype once (a separate add kernel rounds twice).
+ * residual may alias C (each element is read by the thread that writes it).
+ * Everything else as hexmi_gemm, which is this call with bias = residual =
+ * NULL. What it replaces on the reference side: the linalg.generic consumers
+ * (bias add, residual add) that the fusion pass pulls into the matmul's loop
+ * nest (qcom_hexagon_backend/lib/Conversion/LinalgToLLVM/LinalgToLLVMPass.cpp:
+ * 280-283) instead of leaving them as separate kernels behind the HexKL call
+ * (lib/Conversion/LinalgToLLVM/MatmulToHexKLPass.cpp:171-190); the GPT-2
+ * block of test/python/torch-mlir/test_gpt2_block.py is four such layers.
+ * K == 0 with a bias or residual: HEXMI_ENOTSUP. */
+int hexmi_gemm_ex(int64_t M, int64_t N, int64_t K, const void *A, int64_t lda,
+                  const void *B, int64_t ldb, void *C, int64_t ldc,
+                  const void *bias, const void *residual, int64_t ldr,
+                  int in_dtype, int out_dtype, int trans_b,
+                  hexmi_stream_t stream);
+
+/* out[M,N] = softmax((x[M,K] + y[M,K]) * z[K,N], over each row), one launch:
+ * the fused kernel the reference compiles from
+ * test/python/torch-mlir/test_add_matmul_softmax.py:19-29 (torch.add ->
+ * torch.matmul -> torch.softmax(dim=-1)). All four matrices row-major of one
+ * dtype (HEXMI_F32 / HEXMI_F16 / HEXMI_BF16) with leading dims ldx, ldy, ldz,
+ * ldo; the sum x + y is rounded to dtype as torch.add does, the scores stay
+ * fp32 until the division. A workgroup owns 32 whole rows, so N is limited:
+ * N > hexmi_add_matmul_softmax_max_n() (1024) returns HEXMI_ETOOBIG and the
+ * caller runs the three kernels (binary add, hexmi_gemm, hexmi_softmax).
+ * Any M, K, leading dims and alignment. */
+int64_t hexmi_add_matmul_softmax_max_n(void);
+int hexmi_add_matmul_softmax(int64_t M, int64_t N, int64_t K, const void *x,
+                             int64_t ldx, const void *y, int64_t ldy,
+                             const void *z, int64_t ldz, void *out,
+                             int64_t ldo, int dtype, hexmi_stream_t stream);
+
 /* Weight-only int8 GEMM (W8A16): C[m,n] = sum_k A[m,k] * (float(W[n,k]) *
  * float(scales[n])), fp32 accumulation, C fp16.
  * A fp16 [M,K]; W int8 [N,K] row-major (symmetric, zero-point 0); scales fp16

@@ -279,3 +279,158 @@ def test_add_matmul_softmax_reference_graph(hexmi):
     got16 = hexmi.add_matmul_softmax(x.half(), y.half(), z.half()).cpu()
     want16 = torch.nn.functional.softmax(torch.matmul((x.half() + y.half()).float(), z.half().float()), dim=-1)
     assert torch.allclose(got16.float(), want16, atol=2e-2)
+
+
+# ---- hexmi_gemm_ex: bias and residual in the GEMM epilogue ------------------------------------------------------
+def _linear_ref(a, b, bias, resid, trans_b):
+    c = a.double() @ (b.double().T if trans_b else b.double())
+    if bias is not None:
+        c = c + bias.double()
+    if resid is not None:
+        c = c + resid.double()
+    return c
+
+
+@pytest.mark.parametrize("dtype,out_dtype", [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+                                             (torch.float16, torch.float32), (torch.float32, torch.float32)])
+@pytest.mark.parametrize("shape", [(512, 2304, 768), (512, 768, 3072),      # GPT-2 small layers (64-k tiled kernel)
+                                   (256, 256, 96),                           # 32-k tiled kernel
+                                   (100, 72, 40), (33, 50, 17),              # generic kernel (ragged, unaligned)
+                                   (1024, 1024, 1024)])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gemm_ex_bias_and_residual(hexmi, dtype, out_dtype, shape, trans_b):
+    M, N, K = shape
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K + trans_b)
+    a = (torch.randn(M, K, generator=g) * 0.5).to(dtype)
+    b = (torch.randn((N, K) if trans_b else (K, N), generator=g) * 0.5).to(dtype)
+    bias = torch.randn(N, generator=g).to(out_dtype)
+    resid = torch.randn(M, N, generator=g).to(out_dtype)
+    tol = {torch.float16: 2e-2, torch.bfloat16: 1.5e-1, torch.float32: 2e-3 if dtype != torch.float32 else 2e-4}[out_dtype]
+    for use_bias, use_resid in ((True, True), (True, False), (False, True)):
+        got = hexmi.matmul(a.cuda(), b.cuda(), out_dtype=out_dtype, trans_b=trans_b,
+                           bias=bias.cuda() if use_bias else None, residual=resid.cuda() if use_resid else None)
+        want = _linear_ref(a, b, bias if use_bias else None, resid if use_resid else None, trans_b)
+        err = (got.cpu().double() - want).abs().max().item()
+        assert err <= tol * max(1.0, want.abs().max().item() / 16), (use_bias, use_resid, err)
+
+
+def test_gemm_ex_rounds_once(hexmi):
+    # fp16: A B + bias + residual rounded once from fp32 == the correctly rounded fp64 result on all but ties; the
+    # separate kernels (round the product, round the sum, round again) are measurably further away.
+    g = torch.Generator().manual_seed(11)
+    M, N, K = 256, 512, 256
+    a = torch.randn(M, K, generator=g).half()
+    b = torch.randn(K, N, generator=g).half()
+    bias = torch.randn(N, generator=g).half()
+    resid = torch.randn(M, N, generator=g).half()
+    want = _linear_ref(a, b, bias, resid, False)
+    fused = hexmi.matmul(a.cuda(), b.cuda(), bias=bias.cuda(), residual=resid.cuda()).cpu().double()
+    parts = hexmi.binary("add", hexmi.binary("add", hexmi.matmul(a.cuda(), b.cuda()),
+                                             bias.cuda().expand(M, N).contiguous()), resid.cuda()).cpu().double()
+    e_fused = (fused - want).abs().mean().item()
+    e_parts = (parts - want).abs().mean().item()
+    assert e_fused < e_parts
+    assert (fused - want.half().double()).abs().max().item() <= 2 * torch.finfo(torch.float16).eps * want.abs().max().item()
+
+
+def test_gemm_ex_residual_may_alias_output(hexmi):
+    g = torch.Generator().manual_seed(12)
+    M, N, K = 384, 768, 768
+    a = (torch.randn(M, K, generator=g) * 0.1).half().cuda()
+    b = (torch.randn(K, N, generator=g) * 0.1).half().cuda()
+    x = torch.randn(M, N, generator=g).half().cuda()
+    want = hexmi.matmul(a, b, residual=x)
+    acc = x.clone()
+    hexmi.matmul(a, b, residual=acc, out=acc)                       # x += a @ b, in place
+    assert torch.equal(acc, want)
+
+
+def test_gemm_ex_strided_residual_and_bad_arguments(hexmi):
+    from hexmi import _lib
+    lib = _lib.lib()
+    g = torch.Generator().manual_seed(13)
+    M, N, K = 128, 256, 128
+    a = torch.randn(M, K, generator=g).half().cuda()
+    b = torch.randn(K, N, generator=g).half().cuda()
+    wide = torch.randn(M, N + 64, generator=g).half().cuda()       # residual with a leading dimension of N + 64
+    c = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    st = lib.hexmi_gemm_ex(M, N, K, a.data_ptr(), K, b.data_ptr(), N, c.data_ptr(), N, None, wide.data_ptr(), N + 64,
+                           _lib.F16, _lib.F16, 0, s)
+    assert st == 0
+    want = _linear_ref(a.cpu(), b.cpu(), None, wide[:, :N].cpu(), False)
+    assert (c.cpu().double() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item() / 16)
+    # a residual narrower than the result is refused
+    assert lib.hexmi_gemm_ex(M, N, K, a.data_ptr(), K, b.data_ptr(), N, c.data_ptr(), N, None, wide.data_ptr(), N - 8,
+                             _lib.F16, _lib.F16, 0, s) == _lib.EINVAL
+    with pytest.raises(ValueError):
+        hexmi.matmul(a, b, bias=torch.zeros(N + 1, dtype=torch.float16, device="cuda"))
+    with pytest.raises(ValueError):
+        hexmi.matmul(a, b, residual=torch.zeros(M, N, dtype=torch.float32, device="cuda"))
+
+
+# ---- hexmi_add_matmul_softmax: the fused graph in one launch ----------------------------------------------------
+def _ams_ref(x, y, z):
+    total = (x + y)                                                  # torch.add rounds the sum to the dtype
+    return torch.softmax(total.double() @ z.double(), dim=-1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(32, 32, 32),                     # test_add_matmul_softmax.py:32-60
+                                   (1, 1, 1), (7, 5, 3), (100, 130, 70), (33, 257, 100), (64, 512, 48),
+                                   (50, 1000, 37), (96, 1024, 64), (512, 768, 768)])
+def test_add_matmul_softmax_one_launch(hexmi, dtype, shape):
+    M, N, K = shape
+    g = torch.Generator().manual_seed(M + N * 5 + K * 11)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    y = torch.randn(M, K, generator=g).to(dtype)
+    z = (torch.randn(K, N, generator=g) * (1.0 if K <= 64 else 0.2)).to(dtype)
+    got = hexmi.add_matmul_softmax(x.cuda(), y.cuda(), z.cuda(), fused=True).cpu()
+    want = _ams_ref(x, y, z)
+    assert got.dtype == dtype and got.shape == (M, N)
+    if dtype == torch.float32:
+        # the reference test's own bounds at its size; longer fp32 sums carry their rounding into the exponent
+        torch.testing.assert_close(got.double(), want, rtol=1e-5 if K <= 64 else 2e-4, atol=1e-6)
+    else:
+        eps = torch.finfo(dtype).eps
+        torch.testing.assert_close(got.double(), want, rtol=2 * eps, atol=eps * 0.25)
+    sums = got.double().sum(-1)
+    assert (sums - 1).abs().max().item() <= (1e-5 if dtype == torch.float32 else N ** 0.5 * torch.finfo(dtype).eps)
+    # the three-launch route agrees (it rounds the product to the dtype before the softmax, so only to that rounding)
+    three = hexmi.add_matmul_softmax(x.cuda(), y.cuda(), z.cuda(), fused=False).cpu()
+    tol = 1e-5 if dtype == torch.float32 else 0.02 if dtype == torch.float16 else 0.15
+    assert (three.double() - got.double()).abs().max().item() <= tol
+
+
+def test_add_matmul_softmax_limits_and_layouts(hexmi):
+    from hexmi import _lib
+    lib = _lib.lib()
+    assert lib.hexmi_add_matmul_softmax_max_n() == 1024
+    g = torch.Generator().manual_seed(3)
+    M, N, K = 40, 96, 24
+    s = torch.cuda.current_stream().cuda_stream
+    # leading dimensions wider than the rows, output at an odd element offset (no 4-element runs)
+    xw = torch.randn(M, K + 3, generator=g).cuda()
+    yw = torch.randn(M, K + 5, generator=g).cuda()
+    zw = torch.randn(K, N + 7, generator=g).cuda()
+    ow = torch.full((M * (N + 1) + 1,), -7.0, device="cuda")
+    st = lib.hexmi_add_matmul_softmax(M, N, K, xw.data_ptr(), K + 3, yw.data_ptr(), K + 5, zw.data_ptr(), N + 7,
+                                      ow.data_ptr() + 4, N + 1, _lib.F32, s)
+    assert st == 0
+    got = ow[1:].reshape(M, N + 1).cpu()
+    want = _ams_ref(xw[:, :K].cpu(), yw[:, :K].cpu(), zw[:, :N].cpu())
+    torch.testing.assert_close(got[:, :N].double(), want, rtol=1e-5, atol=1e-6)
+    assert (got[:, N] == -7.0).all() and ow[0].item() == -7.0       # nothing written outside the result
+    # too wide, and nonsense sizes
+    big = torch.zeros(8, 1025, device="cuda")
+    assert lib.hexmi_add_matmul_softmax(8, 1025, 8, big.data_ptr(), 8, big.data_ptr(), 8, big.data_ptr(), 1025,
+                                        big.data_ptr(), 1025, _lib.F32, s) == _lib.ETOOBIG
+    assert lib.hexmi_add_matmul_softmax(8, 16, 8, big.data_ptr(), 4, big.data_ptr(), 8, big.data_ptr(), 16,
+                                        big.data_ptr(), 16, _lib.F32, s) == _lib.EINVAL
+    assert lib.hexmi_add_matmul_softmax(0, 16, 8, None, 8, None, 8, None, 16, None, 16, _lib.F32, s) == 0
+    # K == 0: every score is an empty sum, every row uniform
+    out = torch.empty(5, 10, device="cuda")
+    assert lib.hexmi_add_matmul_softmax(5, 10, 0, None, 0, None, 0, None, 10, out.data_ptr(), 10, _lib.F32, s) == 0
+    torch.testing.assert_close(out.cpu(), torch.full((5, 10), 0.1))
+    with pytest.raises(ValueError):
+        hexmi.add_matmul_softmax(big, big, torch.zeros(1025, 2048, device="cuda"), fused=True)
