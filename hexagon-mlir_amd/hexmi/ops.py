@@ -27,7 +27,15 @@ def _dt(t):
         raise TypeError("hexmi: unsupported dtype %s" % t.dtype) from None
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_RAW_DEVICE = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """The current device's current HIP stream as an integer handle (the raw getters skip building a
+    torch.cuda.Stream object per call, which costs more than a ctypes call)."""
+    if _RAW_STREAM is not None and _RAW_DEVICE is not None:
+        return _RAW_STREAM(_RAW_DEVICE())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -49,7 +57,8 @@ _NO_SWITCH = _NoSwitch()
 def _on(device):
     """Context that makes `device` current for the launch; free when it already is (the usual case: entering
     torch.cuda.device() costs more than the shortest kernels here run)."""
-    if device.index is None or device.index == torch.cuda.current_device():
+    if device.index is None or device.index == (_RAW_DEVICE() if _RAW_DEVICE is not None
+                                                else torch.cuda.current_device()):
         return _NO_SWITCH
     return torch.cuda.device(device)
 
@@ -77,22 +86,28 @@ _LIBDEF.define("rope(Tensor x, float theta, Tensor(a!) out) -> ()")
 _LIBDEF.define("attention(Tensor q, Tensor k, Tensor v, Tensor? mask, float sm_scale, Tensor(a!) out) -> ()")
 
 
-def _softmax_impl(x, out):
-    rows, cols = x.shape
+def _softmax_impl(x, out, rows=None, cols=None):
+    """x, out: [rows, cols]; or contiguous tensors of any rank with rows and cols given (no view objects built)."""
+    if rows is None:
+        rows, cols = x.shape
+        ldx, ldo = x.stride(0), out.stride(0)
+    else:
+        ldx = ldo = cols
     with _on(x.device):
-        _lib.check(_lib.lib().hexmi_softmax(_p(x), _p(out), rows, cols, x.stride(0), out.stride(0), _dt(x),
-                                            _stream()), "hexmi_softmax")
+        _lib.check(_lib.lib().hexmi_softmax(_p(x), _p(out), rows, cols, ldx, ldo, _dt(x), _stream()), "hexmi_softmax")
 
 
-def _rms_norm_impl(x, weight, eps, out):
-    rows, cols = x.shape
+def _rms_norm_impl(x, weight, eps, out, rows=None, cols=None):
+    if rows is None:
+        rows, cols = x.shape
     with _on(x.device):
         _lib.check(_lib.lib().hexmi_rms_norm(_p(x), _p(weight), _p(out), rows, cols, eps, _dt(x), _stream()),
                    "hexmi_rms_norm")
 
 
-def _layer_norm_impl(x, weight, bias, eps, out, mean, rstd):
-    rows, cols = x.shape
+def _layer_norm_impl(x, weight, bias, eps, out, mean, rstd, rows=None, cols=None):
+    if rows is None:
+        rows, cols = x.shape
     with _on(x.device):
         _lib.check(_lib.lib().hexmi_layer_norm(_p(x), _p(weight), _p(bias), _p(out), _p(mean), _p(rstd), rows, cols,
                                                eps, _dt(x), _stream()), "hexmi_layer_norm")
@@ -261,7 +276,7 @@ def softmax(x, out=None, dim=-1):
     od = _out_like(out, x.shape, x.dtype, dev)
     cols = x.shape[-1]
     rows = x.numel() // max(cols, 1)
-    _softmax_impl(xd.view(rows, cols), od.view(rows, cols))
+    _softmax_impl(xd, od, rows, cols)
     return _finish(od, out)
 
 
@@ -274,7 +289,7 @@ def rms_norm(x, weight=None, eps=1e-5, out=None):
         raise ValueError("hexmi.rms_norm: weight must be [%d] of %s" % (cols, x.dtype))
     xd, wd = _stage(x, dev), _stage(weight, dev)
     od = _out_like(out, x.shape, x.dtype, dev)
-    _rms_norm_impl(xd.view(rows, cols), wd, float(eps), od.view(rows, cols))
+    _rms_norm_impl(xd, wd, float(eps), od, rows, cols)
     return _finish(od, out)
 
 
@@ -291,7 +306,7 @@ def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=No
     od = _out_like(out, x.shape, x.dtype, dev)
     md = None if mean is None else _out_like(mean if mean.dtype == torch.float32 else None, (rows,), torch.float32, dev)
     rd = None if rstd is None else _out_like(rstd if rstd.dtype == torch.float32 else None, (rows,), torch.float32, dev)
-    _layer_norm_impl(xd.view(rows, cols), wd, bd, float(eps), od.view(rows, cols), md, rd)
+    _layer_norm_impl(xd, wd, bd, float(eps), od, md, rd, rows, cols)
     if mean is not None:
         _finish(md, mean)
     if rstd is not None:
