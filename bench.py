@@ -172,11 +172,13 @@ class LayerNorm(Norms):
 class Gemm(Workload):
     bound, kernel = "mfma", "gemm_kernel_k64"
 
-    def __init__(self, size, dtype_name):
-        self.size, self.dtype = size, dtype_name
-        self.name = "gemm_%s_%d" % (dtype_name, size)
+    def __init__(self, size, dtype_name, packed=False):
+        self.size, self.dtype, self.packed = size, dtype_name, packed
+        self.name = "gemm_%s_%d%s" % (dtype_name, size, "_packed_weight" if packed else "")
         self.desc = "C=A.B %s [%d,%d]x[%d,%d] U(-1,1), fp32 accumulate, %s out" % (dtype_name, size, size, size, size,
                                                                                    dtype_name)
+        if packed:
+            self.desc += "; B re-laid-out once to [N,K] (hexmi_transpose16, outside the timed region) and multiplied as B^T"
 
     def setup(self, torch, hexmi):
         from hexmi.workloads import gemm_inputs, gemm_flops
@@ -187,10 +189,12 @@ class Gemm(Workload):
         self.work = gemm_flops(self.size, self.size, self.size)
         self.sets = _sets(torch, self.host, 0, rotate=False)
         self.sets[0]["out"] = torch.empty(self.size, self.size, dtype=dt, device="cuda")
+        if self.packed:
+            self.sets[0]["b"] = hexmi.pack_weight(self.sets[0]["b"])
 
     def step(self, i):
         s = self.sets[0]
-        self.hexmi.matmul(s["a"], s["b"], out=s["out"])
+        self.hexmi.matmul(s["a"], s["b"], out=s["out"], trans_b=self.packed)
 
     def cpu(self, torch):
         from oracle import torch_cpu
@@ -523,7 +527,7 @@ def _time_cpu(fn, iters):
 def make_workloads():
     return {w.name: w for w in (
         Norms(), Softmax(), Softmax(65536, 1024), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
-        Gemm(4096, "f32"), W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256),
+        Gemm(8192, "bf16", packed=True), Gemm(4096, "f32"), W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256),
         Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), AttentionF32(4, 32, 2048, 64),
         MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
         Elementwise("sum"), LinearFused(), AddMatmulSoftmax(32, 32, 32, "f32"), AddMatmulSoftmax(512, 512, 64, "f16"),
@@ -536,7 +540,7 @@ def peak_workloads():
 
 ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024",
            "softmax_big": "softmax_f32_65536x1024", "gemm": "gemm_f16_4096",
-           "gemm_bf16": "gemm_bf16_8192", "gemm_f32": "gemm_f32_4096", "attn": "attn_causal_f16_4x32x4096x128",
+           "gemm_bf16": "gemm_bf16_8192", "gemm_bf16_packed": "gemm_bf16_8192_packed_weight", "gemm_f32": "gemm_f32_4096", "attn": "attn_causal_f16_4x32x4096x128",
            "attn_long": "attn_causal_f16_1x32x16384x128", "attn_masked": "attn_masked_f16_32x2048x128",
            "attn_f32": "attn_causal_f32_4x32x2048x64", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
            "rope": "rope_f16_4x4096x32x128", "sum": "block_sum_f32_8192x4096", "rms_norm": "rms_norm_f16_8192x4096",

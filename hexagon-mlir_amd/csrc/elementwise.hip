@@ -355,6 +355,28 @@ int launch_rope(const void* xv, void* yv, int64_t batch, int64_t seq, int64_t he
   return launch_status();
 }
 
+// Out-of-place transpose of a matrix of 16-bit elements (bit patterns: fp16 and bf16 alike): 64 x 64 tiles through
+// LDS, rows of the source read and rows of the destination written as contiguous runs, the LDS pitch odd in 32-bit
+// words so neither side conflicts. Any shape and leading dimensions.
+__global__ __launch_bounds__(256)
+void transpose16_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int rows, int cols,
+                        int64_t ld_src, int64_t ld_dst) {
+  __shared__ uint16_t tile[64][66];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int r = r0 + ty + 4 * i, c = c0 + tx;
+    tile[ty + 4 * i][tx] = (r < rows && c < cols) ? src[(int64_t)r * ld_src + c] : (uint16_t)0;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int c = c0 + ty + 4 * i, r = r0 + tx;         // destination row c, column r
+    if (c < cols && r < rows) dst[(int64_t)c * ld_dst + r] = tile[tx][ty + 4 * i];
+  }
+}
+
 }  // namespace
 
 int block_sum_any(const void* x, void* out, int64_t n, int64_t block, int dtype, float* partials, hipStream_t s) {
@@ -438,4 +460,17 @@ extern "C" int hexmi_rope(const void* x, void* y, int64_t batch, int64_t seq, in
     case HEXMI_BF16: return launch_rope<bf16>(x, y, batch, seq, heads, feat, theta, s);
     default: return HEXMI_ENOTSUP;
   }
+}
+
+extern "C" int hexmi_transpose16(int64_t rows, int64_t cols, const void* src, int64_t ld_src, void* dst, int64_t ld_dst,
+                                 hexmi_stream_t stream) {
+  if (rows < 0 || cols < 0) return HEXMI_EINVAL;
+  if (rows == 0 || cols == 0) return HEXMI_OK;
+  if (!src || !dst || ld_src < cols || ld_dst < rows) return HEXMI_EINVAL;
+  const int64_t gx = (cols + 63) / 64, gy = (rows + 63) / 64;
+  if (rows > 0x7fffffff || cols > 0x7fffffff || gy > 65535) return HEXMI_ENOTSUP;
+  begin_call();
+  hipLaunchKernelGGL(transpose16_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint16_t*>(src), static_cast<uint16_t*>(dst), (int)rows, (int)cols, ld_src, ld_dst);
+  return launch_status();
 }

@@ -37,6 +37,7 @@ SIGNATURES = {
                              _ptr]),
     "hexmi_add_matmul_softmax_max_n": (_i64, []),
     "hexmi_add_matmul_softmax": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _ptr]),
+    "hexmi_transpose16": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr]),
     "hexmi_gemm_w8a16": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_pack_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr]),
     "hexmi_gemm_w8a16_packed": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),

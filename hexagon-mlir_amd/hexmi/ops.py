@@ -348,6 +348,22 @@ def matmul(a, b, out=None, out_dtype=None, trans_b=False, bias=None, residual=No
     return _finish(od, out)
 
 
+def pack_weight(w):
+    """One-time re-layout of a constant 16-bit weight [K,N] into the K-contiguous form [N,K] the GEMM streams fastest;
+    multiply with `matmul(a, packed, trans_b=True)`. The analogue of the reference folding the transpose of a
+    constant weight at compile time (qcom_hexagon_backend/lib/Transforms/FoldResourceTransposePass.cpp:21-110)."""
+    if w.dim() != 2 or w.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("hexmi.pack_weight: expected a 2-D float16 or bfloat16 tensor")
+    dev = _device() if w.device.type != "cuda" else w.device
+    wd = _stage(w, dev)
+    rows, cols = wd.shape
+    out = torch.empty((cols, rows), dtype=w.dtype, device=dev)
+    with _on(dev):
+        _lib.check(_lib.lib().hexmi_transpose16(rows, cols, _p(wd), wd.stride(0), _p(out), out.stride(0), _stream()),
+                   "hexmi_transpose16")
+    return out
+
+
 def w8a16_matmul(a, w_int8, scales, out=None):
     """C[m,n] = sum_k A[m,k] * (W[n,k] * scales[n]); A fp16 [M,K], W int8 [N,K], scales fp16 [N]."""
     if a.dtype != torch.float16 or w_int8.dtype != torch.int8 or scales.dtype != torch.float16:

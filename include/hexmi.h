@@ -294,6 +294,20 @@ int64_t hexmi_block_sum_static_max_n(void);
 int hexmi_block_sum_static(const void *x, void *out, int64_t n, int64_t block,
                            int dtype, hexmi_stream_t stream);
 
+/* One-time re-layout of a constant 16-bit weight matrix: dst[c, r] = src[r, c]
+ * for src [rows, cols] (leading dim ld_src >= cols), dst [cols, rows] (ld_dst >=
+ * rows); fp16 or bf16 alike (bit patterns are moved). What it replaces: the
+ * reference transposes constant rank-2 f16 weights once, at compile time,
+ * instead of at every run (qcom_hexagon_backend/lib/Transforms/
+ * FoldResourceTransposePass.cpp:21-110), and re-lays constant weights out for
+ * the matrix unit (lib/Transforms/PreprocessWeightsForHMXPass.cpp:39-117). Here
+ * the layout the matrix-core GEMM streams fastest is the K-contiguous one
+ * (hexmi_gemm with trans_b != 0), so a weight stored [K,N] is transposed once
+ * and multiplied as B^T from then on. Any shape with rows / 64 <= 65535. */
+int hexmi_transpose16(int64_t rows, int64_t cols, const void *src,
+                      int64_t ld_src, void *dst, int64_t ld_dst,
+                      hexmi_stream_t stream);
+
 /* Rotary position embedding of x [batch, seq, heads, feat] (contiguous, feat
  * even): adjacent feature pairs (2i, 2i+1) are rotated by m * theta^(-2i/feat),
  * m the sequence position: `rope_kernel` of test/python/triton/test_rope.py:97-197

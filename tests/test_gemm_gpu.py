@@ -434,3 +434,42 @@ def test_add_matmul_softmax_limits_and_layouts(hexmi):
     torch.testing.assert_close(out.cpu(), torch.full((5, 10), 0.1))
     with pytest.raises(ValueError):
         hexmi.add_matmul_softmax(big, big, torch.zeros(1025, 2048, device="cuda"), fused=True)
+
+
+# ---- hexmi_transpose16: one-time weight re-layout ----------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 70), (64, 64), (65, 129), (768, 3072), (1000, 37), (4096, 4096)])
+def test_pack_weight_is_the_transpose(hexmi, dtype, shape):
+    g = torch.Generator().manual_seed(shape[0] * 3 + shape[1])
+    w = torch.randn(*shape, generator=g).to(dtype)
+    w[0, 0] = float("inf")                                          # bit patterns are moved, whatever they are
+    got = hexmi.pack_weight(w.cuda())
+    assert got.shape == (shape[1], shape[0]) and got.dtype == dtype and got.is_contiguous()
+    assert torch.equal(got.cpu().view(torch.int16), w.t().contiguous().view(torch.int16))
+
+
+def test_packed_weight_product_is_the_same_product(hexmi):
+    # A . B and A . pack(B)^T multiply the same numbers: equal to the last bit in the fp32-output mode
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(256, 512, generator=g).half().cuda()
+    b = torch.randn(512, 384, generator=g).half().cuda()
+    bt = hexmi.pack_weight(b)
+    c1 = hexmi.matmul(a, b, out_dtype=torch.float32)
+    c2 = hexmi.matmul(a, bt, out_dtype=torch.float32, trans_b=True)
+    assert torch.equal(c1, c2)
+
+
+def test_transpose16_strides_and_bad_arguments(hexmi):
+    from hexmi import _lib
+    lib = _lib.lib()
+    s = torch.cuda.current_stream().cuda_stream
+    src = torch.arange(20 * 12, dtype=torch.int16, device="cuda").reshape(20, 12)        # rows 20, ld 12, cols 10 used
+    dst = torch.full((10, 24), -1, dtype=torch.int16, device="cuda")
+    assert lib.hexmi_transpose16(20, 10, src.data_ptr(), 12, dst.data_ptr(), 24, s) == 0
+    assert torch.equal(dst[:, :20].cpu(), src[:, :10].t().cpu())
+    assert (dst[:, 20:] == -1).all()
+    assert lib.hexmi_transpose16(20, 10, src.data_ptr(), 8, dst.data_ptr(), 24, s) == _lib.EINVAL
+    assert lib.hexmi_transpose16(20, 10, src.data_ptr(), 12, dst.data_ptr(), 16, s) == _lib.EINVAL
+    assert lib.hexmi_transpose16(0, 10, None, 12, None, 24, s) == 0
+    with pytest.raises(TypeError):
+        hexmi.pack_weight(torch.zeros(4, 4, device="cuda"))
