@@ -827,15 +827,18 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
       slab(a_p2, b_p2, a_p3, b_p3, a_p1, b_p1, j + 2);
       slab(a_p3, b_p3, a_p0, b_p0, a_p2, b_p2, j + 3);
     }
+    // The MFMAs are assembly, so the compiler does not count the wait states between the last of them and the
+    // first read of an accumulator (19 for the longest matrix instruction). They are spent here, at the end of the
+    // last pass and still inside the loop: the register allocator places its accumulator reads at the top of the
+    // block that follows the loop, above anything written there.
+    if (j + NS >= KT) {
+      HEXMI_FENCE;
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+      HEXMI_FENCE;
+    }
   }
 #undef HEXMI_FENCE
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));       // drain the trailing copies before the workgroup's LDS goes away
-  // The MFMAs are assembly, so the compiler does not count the wait states between the last of them and the first
-  // read of an accumulator (19 for the longest matrix instruction): spend them here, fenced so that no accumulator
-  // read is scheduled above them.
-  __builtin_amdgcn_sched_barrier(0);
-  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
 
   // acc[i][j][r]: row lane%16 of tile row i, column 4*(lane/16) + r of tile column j
   if constexpr (B_I8) {
