@@ -426,13 +426,27 @@ __global__ __launch_bounds__(256)
 void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
                        f16* __restrict__ C, int M, int N, int K) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int n0 = (blockIdx.x * 4 + wave) * RPW;
-  if (n0 >= N) return;
+  const int n0 = (blockIdx.x * 4 + wave) * RPW;            // may lie past N in the last workgroup: loads clamp, stores check
 
   // the channel scales first: they come from HBM and would otherwise be waited for after everything else
   f16 sc[RPW];
 #pragma unroll
   for (int r = 0; r < RPW; ++r) sc[r] = scales[n0 + r < N ? n0 + r : N - 1];
+  // activations: lane needs k in [1024*j + 16*lane, +16) for every j. The four waves of the workgroup need the same
+  // rows, so each fetches a quarter of them (requested before the weights: their wait then leaves the weight loads in
+  // flight) and all read their fragments back from LDS.
+  __shared__ __attribute__((aligned(16))) f16 a_lds[MR][KJ * 1024];
+  constexpr int kAChunks = (KJ * 128 + 255) / 256;
+  f16x8 a_in[MR][kAChunks];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    const f16* arow = A + (int64_t)(m < M ? m : 0) * K;
+#pragma unroll
+    for (int c = 0; c < kAChunks; ++c) {
+      const int chunk = c * 256 + threadIdx.x;
+      a_in[m][c] = *reinterpret_cast<const f16x8*>(arow + (chunk < KJ * 128 ? chunk : 0) * 8);
+    }
+  }
   u32x4 wv[RPW][KJ];
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
@@ -441,17 +455,22 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
 #pragma unroll
     for (int j = 0; j < KJ; ++j) wv[r][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + j * 1024));
   }
-  // activations: lane needs k in [1024*j + 16*lane, +16) for every j: two 16-byte loads per (row, j)
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int c = 0; c < kAChunks; ++c) {
+      const int chunk = c * 256 + threadIdx.x;
+      if (chunk < KJ * 128) *reinterpret_cast<f16x8*>(&a_lds[m][chunk * 8]) = a_in[m][c];
+    }
+  __syncthreads();
   f16x8 av[MR][KJ][2];
 #pragma unroll
-  for (int m = 0; m < MR; ++m) {
-    const f16* arow = A + (int64_t)(m < M ? m : 0) * K + lane * 16;
+  for (int m = 0; m < MR; ++m)
 #pragma unroll
     for (int j = 0; j < KJ; ++j) {
-      av[m][j][0] = *reinterpret_cast<const f16x8*>(arow + j * 1024);
-      av[m][j][1] = *reinterpret_cast<const f16x8*>(arow + j * 1024 + 8);
+      av[m][j][0] = *reinterpret_cast<const f16x8*>(&a_lds[m][j * 1024 + lane * 16]);
+      av[m][j][1] = *reinterpret_cast<const f16x8*>(&a_lds[m][j * 1024 + lane * 16 + 8]);
     }
-  }
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
     float acc[MR];
