@@ -421,12 +421,13 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
 // the row for j = 0..K/1024), all RPW rows in flight at once; the activations a lane needs (the same k for every
 // row) sit in registers as fp16 pairs. Products are v_dot2_f32_f16 (two exact fp16 products added into an fp32
 // accumulator), the 64 lane partials are summed with a butterfly, and lane 0 applies the channel scale.
-template <int MR, int RPW, int KJ>                          // KJ = K / 1024: 16-byte loads per lane per row
-__global__ __launch_bounds__(256)
+// NW waves per workgroup share the activation rows through LDS.
+template <int MR, int RPW, int KJ, int NW = 4>              // KJ = K / 1024: 16-byte loads per lane per row
+__global__ __launch_bounds__(NW * 64)
 void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
                        f16* __restrict__ C, int M, int N, int K) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int n0 = (blockIdx.x * 4 + wave) * RPW;            // may lie past N in the last workgroup: loads clamp, stores check
+  const int n0 = (blockIdx.x * NW + wave) * RPW;           // may lie past N in the last workgroup: loads clamp, stores check
 
   // the channel scales first: they come from HBM and would otherwise be waited for after everything else
   f16 sc[RPW];
@@ -436,14 +437,14 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
   // rows, so each fetches a quarter of them (requested before the weights: their wait then leaves the weight loads in
   // flight) and all read their fragments back from LDS.
   __shared__ __attribute__((aligned(16))) f16 a_lds[MR][KJ * 1024];
-  constexpr int kAChunks = (KJ * 128 + 255) / 256;
+  constexpr int kAChunks = (KJ * 128 + NW * 64 - 1) / (NW * 64);
   f16x8 a_in[MR][kAChunks];
 #pragma unroll
   for (int m = 0; m < MR; ++m) {
     const f16* arow = A + (int64_t)(m < M ? m : 0) * K;
 #pragma unroll
     for (int c = 0; c < kAChunks; ++c) {
-      const int chunk = c * 256 + threadIdx.x;
+      const int chunk = c * (NW * 64) + threadIdx.x;
       a_in[m][c] = *reinterpret_cast<const f16x8*>(arow + (chunk < KJ * 128 ? chunk : 0) * 8);
     }
   }
@@ -459,7 +460,7 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
   for (int m = 0; m < MR; ++m)
 #pragma unroll
     for (int c = 0; c < kAChunks; ++c) {
-      const int chunk = c * 256 + threadIdx.x;
+      const int chunk = c * (NW * 64) + threadIdx.x;
       if (chunk < KJ * 128) *reinterpret_cast<f16x8*>(&a_lds[m][chunk * 8]) = a_in[m][c];
     }
   __syncthreads();
@@ -593,9 +594,12 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     return launch_status();
   }
   if (M <= 2 && (K == 1024 || K == 2048 || K == 4096 || K == 8192)) {
-    constexpr int RPW = 2;
-    const unsigned blocks = (unsigned)((N + 4 * RPW - 1) / (4 * RPW));
-#define HEXMI_GEMV(MR, KJ) hipLaunchKernelGGL((w8a16_gemv_kernel<MR, RPW, KJ>), dim3(blocks), dim3(256), 0, st, a, W, s, c, (int)M, (int)N, (int)K)
+    // one channel per wave, eight waves per workgroup: measured against two and four channels per wave and
+    // workgroups of two, four and sixteen waves at N = 11008, K = 4096 (0.60 of the HBM figure against 0.57 for two
+    // channels x four waves on the same box)
+    constexpr int RPW = 1, NW = 8;
+    const unsigned blocks = (unsigned)((N + NW * RPW - 1) / (NW * RPW));
+#define HEXMI_GEMV(MR, KJ) hipLaunchKernelGGL((w8a16_gemv_kernel<MR, RPW, KJ, NW>), dim3(blocks), dim3(NW * 64), 0, st, a, W, s, c, (int)M, (int)N, (int)K)
 #define HEXMI_GEMV_K(MR) { if (K == 1024) HEXMI_GEMV(MR, 1); else if (K == 2048) HEXMI_GEMV(MR, 2); else if (K == 4096) HEXMI_GEMV(MR, 4); else HEXMI_GEMV(MR, 8); }
     if (M == 1) HEXMI_GEMV_K(1) else HEXMI_GEMV_K(2)
 #undef HEXMI_GEMV_K
