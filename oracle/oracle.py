@@ -122,6 +122,29 @@ def matmul(a, b, out_dtype=None, trans_b=False, dtype=None):
     return c
 
 
+def linear(a, b, bias=None, residual=None, out_dtype=None, trans_b=False):
+    """A op(B) + bias[n] + residual[m, n] with the sums kept in fp32 and ONE rounding to the output type: the linear
+    layer whose consumers the reference fuses into the matmul's loop nest
+    (qcom_hexagon_backend/lib/Conversion/LinalgToLLVM/LinalgToLLVMPass.cpp:280-283; the layers of
+    test/python/torch-mlir/test_gpt2_block.py). fp16 / fp32 only. Composed of matmul() above (fp32 output) and numpy."""
+    out_dtype = out_dtype or a.dtype
+    c = matmul(a, b, out_dtype=np.float32, trans_b=trans_b).astype(np.float64)
+    if bias is not None:
+        c = c + bias.astype(np.float64)[None, :]
+    if residual is not None:
+        c = c + residual.astype(np.float64)
+    return c.astype(np.float32).astype(out_dtype)
+
+
+def add_matmul_softmax(x, y, z):
+    """softmax((x + y) z) over each row: the graph of test/python/torch-mlir/test_add_matmul_softmax.py:19-29
+    (torch.add, torch.matmul, torch.softmax(dim=-1)), the sum rounded to the operands' type as torch.add rounds it,
+    the product and the softmax in fp32. Composed of matmul() and softmax() above."""
+    total = (x.astype(np.float32) + y.astype(np.float32)).astype(x.dtype)
+    scores = matmul(total, z, out_dtype=np.float32)
+    return softmax(scores).astype(x.dtype)
+
+
 def dequant_w8(w, scales):
     w, scales = _c(w), _c(scales)
     assert w.dtype == np.int8 and scales.dtype == np.float16

@@ -473,3 +473,29 @@ def test_transpose16_strides_and_bad_arguments(hexmi):
     assert lib.hexmi_transpose16(0, 10, None, 12, None, 24, s) == 0
     with pytest.raises(TypeError):
         hexmi.pack_weight(torch.zeros(4, 4, device="cuda"))
+
+
+def test_gemm_ex_and_fused_graph_against_the_oracle(hexmi, oracle):
+    # the C oracle's product with its numpy epilogue / softmax (oracle.linear, oracle.add_matmul_softmax), fp16 and fp32
+    g = torch.Generator().manual_seed(31)
+    a = torch.randn(192, 320, generator=g).half()
+    b = (torch.randn(320, 136, generator=g) * 0.2).half()
+    bias = torch.randn(136, generator=g).half()
+    res = torch.randn(192, 136, generator=g).half()
+    got = hexmi.matmul(a.cuda(), b.cuda(), bias=bias.cuda(), residual=res.cuda()).cpu()
+    want = torch.from_numpy(oracle.linear(a.numpy(), b.numpy(), bias.numpy(), res.numpy()))
+    assert close16(got, want, max_ulp=1, atol=2e-4)
+    got32 = hexmi.matmul(a.cuda(), b.cuda(), out_dtype=torch.float32, bias=bias.float().cuda(),
+                         residual=res.float().cuda()).cpu()
+    want32 = torch.from_numpy(oracle.linear(a.numpy(), b.numpy(), bias.float().numpy(), res.float().numpy(),
+                                            out_dtype=np.float32))
+    assert torch.allclose(got32, want32, rtol=1e-5, atol=1e-4)
+    for dtype in (torch.float32, torch.float16):
+        x, y = (torch.randn(70, 48, generator=g).to(dtype) for _ in range(2))
+        z = torch.randn(48, 200, generator=g).to(dtype)
+        gf = hexmi.add_matmul_softmax(x.cuda(), y.cuda(), z.cuda(), fused=True).cpu()
+        wf = torch.from_numpy(oracle.add_matmul_softmax(x.numpy(), y.numpy(), z.numpy()))
+        if dtype == torch.float32:
+            assert torch.allclose(gf, wf, rtol=1e-5, atol=1e-6)
+        else:
+            assert close16(gf, wf, max_ulp=1, atol=1e-5)

@@ -392,3 +392,49 @@ def test_pack_w8_is_the_documented_permutation(oracle):
     # every input byte appears exactly once (pure permutation plus zero padding)
     ids = (np.arange(48 * 192, dtype=np.int64) % 251).astype(np.int8).reshape(48, 192)
     assert sorted(oracle.pack_w8(ids).tolist()) == sorted(ids.reshape(-1).tolist())
+
+
+def test_linear_pins(oracle):
+    # (1) against torch's own fused form in fp64; (2) special cases a dropped or mis-indexed operand would fail:
+    # zero weights leave bias + residual exactly, a one-hot weight copies a column of A, the bias goes along columns
+    g = torch.Generator().manual_seed(21)
+    a = torch.randn(24, 40, generator=g).half()
+    b = torch.randn(40, 56, generator=g).half()
+    bias = torch.randn(56, generator=g).half()
+    res = torch.randn(24, 56, generator=g).half()
+    got = torch.from_numpy(oracle.linear(a.numpy(), b.numpy(), bias.numpy(), res.numpy()))
+    want = torch.addmm(res.double() + bias.double(), a.double(), b.double())
+    assert (got.double() - want).abs().max() <= 2e-2 * want.abs().max() / 16
+    got_t = torch.from_numpy(oracle.linear(a.numpy(), b.t().contiguous().numpy(), bias.numpy(), res.numpy(), trans_b=True))
+    assert torch.equal(got, got_t)
+    zero = torch.zeros_like(b)
+    only = torch.from_numpy(oracle.linear(a.numpy(), zero.numpy(), bias.numpy(), res.numpy(), out_dtype=np.float32))
+    assert torch.equal(only, (res.float() + bias.float()))
+    onehot = torch.zeros(40, 56).half()
+    onehot[7, 13] = 1
+    col = torch.from_numpy(oracle.linear(a.numpy(), onehot.numpy(), bias.numpy(), None, out_dtype=np.float32))
+    assert torch.equal(col[:, 13], a[:, 7].float() + bias[13].float())
+    assert torch.equal(col[:, 12], bias[12].float().expand(24))
+    assert torch.equal(torch.from_numpy(oracle.linear(a.numpy(), b.numpy())),
+                       torch.from_numpy(oracle.matmul(a.numpy(), b.numpy())))
+
+
+def test_add_matmul_softmax_pins(oracle):
+    # the reference test's own comparison (test/python/torch-mlir/test_add_matmul_softmax.py:32-60: three 32x32
+    # fp32 randn, rtol 1e-5, atol 1e-6) plus what the mathematics fixes: rows sum to 1, y = -x gives the uniform
+    # distribution, a shift of every score of a row (z with equal columns added) changes nothing
+    g = torch.Generator().manual_seed(22)
+    x, y, z = (torch.randn(32, 32, generator=g) for _ in range(3))
+    got = torch.from_numpy(oracle.add_matmul_softmax(x.numpy(), y.numpy(), z.numpy()))
+    want = torch.softmax(torch.matmul(x + y, z), dim=-1)
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(got.sum(-1), torch.ones(32), atol=1e-6)
+    uniform = torch.from_numpy(oracle.add_matmul_softmax(x.numpy(), (-x).numpy(), z.numpy()))
+    assert torch.allclose(uniform, torch.full((32, 32), 1 / 32), atol=1e-7)
+    shifted = z + torch.randn(32, 1, generator=g)                    # adds (x + y)[m,:] . c to every score of row m
+    got2 = torch.from_numpy(oracle.add_matmul_softmax(x.numpy(), y.numpy(), shifted.numpy()))
+    assert torch.allclose(got2, got, rtol=1e-4, atol=1e-6)
+    xh, yh, zh = x.half(), y.half(), z.half()
+    goth = torch.from_numpy(oracle.add_matmul_softmax(xh.numpy(), yh.numpy(), zh.numpy()))
+    wanth = torch.softmax((xh + yh).double() @ zh.double(), dim=-1)
+    assert (goth.double() - wanth).abs().max() <= 1e-3
