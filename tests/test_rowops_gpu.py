@@ -146,6 +146,7 @@ def test_norm_config_shape(hexmi, oracle):
 # walking several row groups with the next group's loads in flight); row counts chosen so that workgroups walk
 # unequal numbers of groups.
 WALK_SHAPES = [(torch.float16, 32772, 512), (torch.float16, 16388, 1024), (torch.float32, 8204, 1024),
+               (torch.float32, 16400, 1024),       # softmax over >= 16384 rows: one workgroup per CU in the walk
                (torch.float16, 4100, 4096), (torch.bfloat16, 2051, 8192), (torch.float32, 1030, 8192)]
 
 
