@@ -49,7 +49,11 @@ __device__ __forceinline__ float unary(float x) {
 }
 
 constexpr int kEwThreads = 256;
-constexpr int kEwChunks = 4;                         // 16-byte chunks per thread
+// 16-byte chunks per thread (and loads in flight per thread). A/B on one box, GELU / SiLU fp16 [8192,4096]: two chunks
+// 0.705 / 0.718 of the HBM figure, four 0.675 / 0.690, eight 0.686 / 0.715; 128-, 512- and 1024-thread workgroups
+// were no better with either.
+constexpr int kEwChunks = 2;
+constexpr int kBinChunks = 2;                        // binary operators: chunks per operand and thread
 
 template <typename T, int OP>
 __global__ __launch_bounds__(kEwThreads)
@@ -98,7 +102,7 @@ template <typename T, int OP>
 __global__ __launch_bounds__(kEwThreads)
 void binary_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ y, int64_t n) {
   constexpr int N = Chunk<T>::N;
-  constexpr int CH = kEwChunks / 2;                  // two operands: the same number of loads in flight
+  constexpr int CH = kBinChunks;
   const int64_t chunks = n / N;
   const int64_t c0 = (int64_t)blockIdx.x * (kEwThreads * CH) + threadIdx.x;
   Chunk<T> ia[CH], ib[CH];
@@ -284,7 +288,7 @@ int launch_binary(const void* av, const void* bv, void* yv, int64_t n, hipStream
   constexpr int N = 16 / sizeof(T);
   if (aligned_to(a, 16) && aligned_to(b, 16) && aligned_to(y, 16) && n >= N) {
     const int64_t chunks = n / N;
-    const int64_t per_block = kEwThreads * (kEwChunks / 2);
+    const int64_t per_block = kEwThreads * kBinChunks;
     const int64_t blocks = (chunks + per_block - 1) / per_block;
     if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
     hipLaunchKernelGGL((binary_kernel<T, OP>), dim3((unsigned)blocks), dim3(kEwThreads), 0, s, a, b, y, n);
