@@ -17,6 +17,8 @@ replayed REPLAYS times, each replay timed on its own; `ms_per_step` is the media
 HBM-bound entries also carry a `hot` figure (one buffer set, served by the 256 MB Infinity Cache where it fits):
 the rotated one is the HBM claim. `--workload mfma_peak` times a registers-only MFMA stream (zeros and U(-1,1)
 operands, both instruction shapes, about a second each): the data-dependent ceiling of the matrix cores on this box.
+`--workload issue_slots` (vector instructions that fit between a wave's MFMAs) and `--workload lds_patterns` (cycles
+per LDS read for the GEMM's fragment address patterns) are two more calibrations of the same kind.
 """
 import argparse
 import json
@@ -704,6 +706,89 @@ def run_peak(torch, hexmi, args):
     print(json.dumps(line), flush=True)
 
 
+def _time_launch(torch, fn, repeats=5):
+    """Median and minimum of `repeats` single launches (ms), HIP events on torch's current stream."""
+    fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(repeats):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ts.append(e0.elapsed_time(e1))
+    ts.sort()
+    return ts[len(ts) // 2], ts[0]
+
+
+def _calibration_line(args, workload, description, kernel, rows, key):
+    return {"metric": "GEMM/attn TFLOP/s + softmax/norm GB/s, % of MI355X roofline, 1 GPU", "value": None,
+            "unit": "cycles", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None,
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": workload, "description": description},
+            "roofline": {"bound": "mfma", "achieved": None, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": None,
+                         "traffic": None, "kernel": kernel},
+            key: rows}
+
+
+def run_issue_slots(torch, hexmi, args):
+    """--workload issue_slots: time per MFMA of a registers-only stream with 0..8 vector instructions after each
+    MFMA (hexmi_issue_slots; zero operands, so the clock is the 2.4 GHz the cycle figures assume)."""
+    from hexmi import _lib
+    lib = _lib.lib()
+    sink = torch.empty(lib.hexmi_num_cus() * 512, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    kinds = ["v_pk_add_f16", "v_fma_f32", "v_exp_f32"]
+    rows = []
+    for waves in (1, 2):
+        for shape in (1, 0):
+            per_iter = 4 if shape == 0 else 16
+            iters = 40000 if shape == 0 else 10000
+            for kind in (0, 2) if shape == 1 else (0, 1, 2):
+                for per in (0, 1, 2, 3, 4, 5, 6, 8):
+                    fn = lambda: _lib.check(lib.hexmi_issue_slots(shape, kind, per, iters, waves, sink.data_ptr(), st),
+                                            "hexmi_issue_slots")
+                    med, best = _time_launch(torch, fn)
+                    ns = med * 1e6 / (iters * per_iter * waves)
+                    rows.append({"mfma": "32x32x16" if shape == 0 else "16x16x32", "waves_per_simd": waves,
+                                 "instruction": kinds[kind], "per_mfma": per, "ns_per_mfma": round(ns, 2),
+                                 "cycles_per_mfma_at_2.4GHz": round(ns * 2.4, 1), "launch_ms": round(med, 3),
+                                 "launch_ms_min": round(best, 3)})
+                    print("# %s, %d waves/SIMD, %d x %s per MFMA: %.1f cycles per MFMA" % (
+                        rows[-1]["mfma"], waves, per, kinds[kind], ns * 2.4), file=sys.stderr, flush=True)
+    print(json.dumps(_calibration_line(args, "issue_slots", "vector instructions between the MFMAs of one wave: time "
+                                       "per MFMA per SIMD; a calibration, not a product kernel", "issue_slots_kernel",
+                                       rows, "issue_slots")), flush=True)
+
+
+def run_lds_patterns(torch, hexmi, args):
+    """--workload lds_patterns: cycles per wave-wide 16-byte LDS read for the tiled GEMM's fragment-read address
+    patterns, the LDS saturated by 16 waves per compute unit (hexmi_lds_read_pattern)."""
+    from hexmi import _lib
+    lib = _lib.lib()
+    sink = torch.empty(lib.hexmi_num_cus() * 1024, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    names = ["linear (lane * 16)", "fp16 rows, chunk 4*step + g, swizzle (row>>1)&7 (fp16 kernels)",
+             "fp16 rows, chunk 2*g + step, swizzle (row>>1)&7", "fp16 rows, chunk 2*g + step, swizzle of the int8-weight kernel",
+             "int8 rows, swizzle (row>>2)&3", "int8 rows, swizzle (row>>1)&3 (in use)", "fp16 rows, chunk 4*step + g, no swizzle"]
+    iters = 20000
+    # clock: the same launch shape on the linear pattern moves 1 KiB per read; the figure is quoted in ns and in
+    # cycles of the 2.4 GHz the chip holds on a load this light
+    rows = []
+    for pat, name in enumerate(names):
+        fn = lambda: _lib.check(lib.hexmi_lds_read_pattern(pat, iters, sink.data_ptr(), st), "hexmi_lds_read_pattern")
+        med, best = _time_launch(torch, fn)
+        ns = med * 1e6 / (iters * 8 * 16)                # per wave-wide read of one compute unit
+        rows.append({"pattern": pat, "description": name, "ns_per_read": round(ns, 3),
+                     "cycles_per_read_at_2.4GHz": round(ns * 2.4, 2), "bytes_per_cycle_per_cu": round(1024 / (ns * 2.4), 1),
+                     "launch_ms": round(med, 3), "launch_ms_min": round(best, 3)})
+        print("# pattern %d (%s): %.2f cycles per read" % (pat, name, ns * 2.4), file=sys.stderr, flush=True)
+    print(json.dumps(_calibration_line(args, "lds_patterns", "wave-wide 16-byte LDS reads with the tiled GEMM's "
+                                       "fragment address patterns; a calibration, not a product kernel",
+                                       "lds_pattern_kernel", rows, "lds_patterns")), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -730,6 +815,10 @@ def main():
 
     if args.workload == "mfma_peak":
         return run_peak(torch, hexmi, args)
+    if args.workload == "issue_slots":
+        return run_issue_slots(torch, hexmi, args)
+    if args.workload == "lds_patterns":
+        return run_lds_patterns(torch, hexmi, args)
 
     wls = make_workloads()
     primary = wls[ALIASES.get(args.workload, args.workload)]

@@ -3,6 +3,8 @@
 // operands of the caller's choice. The rate depends on the data: the chip is power-limited, all-zero operands
 // toggle nothing and hold the top clock, random operands do not. Roofline fractions of the MFMA-bound kernels are
 // priced against the published peak; this figure says how much of that peak any kernel could reach on such data.
+#include <type_traits>
+
 #include "hexmi_common.h"
 
 namespace hexmi {
@@ -69,6 +71,107 @@ void mfma_peak_kernel(const T* __restrict__ operands, int iters, float* __restri
   sink[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = total;
 }
 
+
+// ---- issue slots --------------------------------------------------------------------------------------------
+// How much vector work fits under a wave's own MFMAs: per MFMA (independent accumulators, zero operands, so the chip
+// holds its top clock) VPM vector instructions of one kind follow in the same instruction stream. A SIMD issues one
+// instruction at a time, so the time per MFMA is the larger of the matrix pipe's (16 or 32 cycles) and the issue time
+// of everything in between.
+template <bool BIG, int KIND, int VPM>
+__global__ __launch_bounds__(512)
+void issue_slots_kernel(int iters, float* __restrict__ sink) {
+  const f16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, b = a;
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = 0.001f * (float)(threadIdx.x + i);
+  constexpr int NM = BIG ? 4 : 16;                 // 64 accumulator registers either way
+  typedef typename std::conditional<BIG, f32x16, f32x4v>::type Acc;
+  Acc acc[NM];
+#pragma unroll
+  for (int m = 0; m < NM; ++m)
+#pragma unroll
+    for (int r = 0; r < (BIG ? 16 : 4); ++r) acc[m][r] = 0.0f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      if constexpr (BIG) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[m]) : "v"(a), "v"(b));
+      else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[m]) : "v"(a), "v"(b));
+#pragma unroll
+      for (int n = 0; n < VPM; ++n) {
+        const int idx = (m * VPM + n) % 8;         // eight independent chains
+        if constexpr (KIND == 0) asm volatile("v_pk_add_f16 %0, %0, %0" : "+v"(v[idx]));
+        else if constexpr (KIND == 1) asm volatile("v_fma_f32 %0, %0, %0, %0" : "+v"(v[idx]));
+        else asm volatile("v_exp_f32 %0, %0" : "+v"(v[idx]));
+      }
+    }
+  }
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the MFMAs are assembly: wait states before reading acc
+  float total = 0.0f;
+#pragma unroll
+  for (int m = 0; m < NM; ++m) total += acc[m][0];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) total += v[i];
+  sink[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = total;
+}
+
+template <bool BIG, int KIND>
+int launch_issue_slots(int per_mfma, dim3 grid, dim3 block, hipStream_t st, int iters, float* sink) {
+#define HEXMI_SLOTS(V) case V: hipLaunchKernelGGL((issue_slots_kernel<BIG, KIND, V>), grid, block, 0, st, iters, sink); break;
+  switch (per_mfma) {
+    HEXMI_SLOTS(0) HEXMI_SLOTS(1) HEXMI_SLOTS(2) HEXMI_SLOTS(3) HEXMI_SLOTS(4) HEXMI_SLOTS(5) HEXMI_SLOTS(6) HEXMI_SLOTS(8)
+    default: return HEXMI_EINVAL;
+  }
+#undef HEXMI_SLOTS
+  return launch_status();
+}
+
+// ---- LDS read patterns --------------------------------------------------------------------------------------
+// Cycles per wave-wide ds_read_b128 for the fragment-read address patterns of the tiled GEMM, with 16 waves per
+// compute unit issuing nothing else (the LDS saturated). Eight reads (four 16-row tiles x two K steps) per round.
+// 0 lane*16 (linear)                    3 the same read with swizzle ((r>>1)&1) | ((r&1)<<1) | (r&4)
+// 1 fp16 rows of 128 bytes, lane group g reads chunk 4*step + g, chunks XOR-swizzled by (row >> 1) & 7
+// 2 the same rows read as chunk 2*g + step (what int8 B imposes on A), same swizzle
+// 4 int8 rows of 64 bytes, lane group g reads chunk g, swizzle (row >> 2) & 3      5 the same, swizzle (row >> 1) & 3
+// 6 pattern 1 without a swizzle
+__device__ __forceinline__ int lds_pattern_addr(int pattern, int lane, int t) {
+  const int r16 = lane % 16, g = lane / 16, step = t / 4;
+  const int row = (t % 4) * 16 + r16;
+  switch (pattern) {
+    case 0: return t * 1024 + lane * 16;
+    case 1: return row * 128 + (((4 * step + g) ^ ((row >> 1) & 7)) * 16);
+    case 2: return row * 128 + (((2 * g + step) ^ ((row >> 1) & 7)) * 16);
+    case 3: return row * 128 + (((2 * g + step) ^ (((row >> 1) & 1) | ((row & 1) << 1) | (row & 4))) * 16);
+    case 4: return (t * 16 + r16) * 64 + ((g ^ (((t * 16 + r16) >> 2) & 3)) * 16);
+    case 5: return (t * 16 + r16) * 64 + ((g ^ (((t * 16 + r16) >> 1) & 3)) * 16);
+    default: return row * 128 + (4 * step + g) * 16;
+  }
+}
+
+constexpr int kLdsPatternBytes = 32768;             // four waves' worth of 8 KiB tiles
+
+__global__ __launch_bounds__(1024)
+void lds_pattern_kernel(int pattern, int iters, float* __restrict__ sink) {
+  __shared__ __attribute__((aligned(16))) uint32_t tile[kLdsPatternBytes / 4];
+  for (int i = threadIdx.x; i < kLdsPatternBytes / 4; i += blockDim.x) reinterpret_cast<volatile uint32_t*>(tile)[i] = i;
+  __syncthreads();
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int base = (int)(uintptr_t)((__attribute__((address_space(3))) void*)tile) + (wave % 4) * 8192;
+  int addr[8];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) addr[t] = base + lds_pattern_addr(pattern, lane, t);
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      u32x4 v;
+      asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(4)" : "=v"(v) : "v"(addr[t]) : "memory");
+      acc ^= v;                                   // may see the register before the read lands: only the time matters
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+  sink[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = (float)(acc[0] ^ acc[1] ^ acc[2] ^ acc[3]);
+}
+
 }  // namespace
 }  // namespace hexmi
 
@@ -98,5 +201,34 @@ extern "C" int hexmi_mfma_peak(int shape, int dtype, const void* operands, int64
   else if (dtype == HEXMI_BF16) { if (shape == 0) HEXMI_PEAK(bf16, true); else HEXMI_PEAK(bf16, false); }
   else return HEXMI_ENOTSUP;
 #undef HEXMI_PEAK
+  return launch_status();
+}
+
+extern "C" int hexmi_issue_slots(int shape, int kind, int per_mfma, int64_t iters, int waves_per_simd, float* sink,
+                                 hexmi_stream_t stream) {
+  if ((shape != 0 && shape != 1) || kind < 0 || kind > 2 || waves_per_simd < 1 || waves_per_simd > 2 || iters < 0 ||
+      iters > 0x7fffffff || !sink)
+    return HEXMI_EINVAL;
+  const int cus = hexmi_num_cus();
+  if (cus <= 0) return HEXMI_ELAUNCH;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid((unsigned)cus), block(256u * waves_per_simd);
+  begin_call();
+  if (shape == 0) {
+    if (kind == 0) return launch_issue_slots<true, 0>(per_mfma, grid, block, st, (int)iters, sink);
+    if (kind == 1) return launch_issue_slots<true, 1>(per_mfma, grid, block, st, (int)iters, sink);
+    return launch_issue_slots<true, 2>(per_mfma, grid, block, st, (int)iters, sink);
+  }
+  if (kind == 0) return launch_issue_slots<false, 0>(per_mfma, grid, block, st, (int)iters, sink);
+  if (kind == 1) return launch_issue_slots<false, 1>(per_mfma, grid, block, st, (int)iters, sink);
+  return launch_issue_slots<false, 2>(per_mfma, grid, block, st, (int)iters, sink);
+}
+
+extern "C" int hexmi_lds_read_pattern(int pattern, int64_t iters, float* sink, hexmi_stream_t stream) {
+  if (pattern < 0 || pattern > 6 || iters < 0 || iters > 0x7fffffff || !sink) return HEXMI_EINVAL;
+  const int cus = hexmi_num_cus();
+  if (cus <= 0) return HEXMI_ELAUNCH;
+  begin_call();
+  hipLaunchKernelGGL(lds_pattern_kernel, dim3((unsigned)cus), dim3(1024), 0, as_stream(stream), pattern, (int)iters, sink);
   return launch_status();
 }

@@ -447,6 +447,12 @@ void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __r
 // the L2 request count halves, and one barrier serves 64 elements of K instead of 32.
 constexpr int BK2 = 64;
 __device__ __forceinline__ int swz_k2(int row) { return (row >> 1) & 7; }      // row pitch 128 B: 16 rows, 16 slots
+// The int8-B kernel reads the same rows with another lane-to-chunk assignment (lane group g takes chunk 2g + step
+// instead of 4*step + g); with swz_k2 those reads take twice the cycles in the LDS (measured: 8.3 against 4.6 per
+// wave-wide 16-byte read with the LDS saturated). Of the 4096 XOR-linear maps of the row bits this is one of the
+// single-bit ones that run both at full rate.
+__device__ __forceinline__ int swz_k2i(int row) { return ((row >> 1) & 1) | ((row & 1) << 1) | (row & 4); }
+template <bool ALT> __device__ __forceinline__ int swz_k2_sel(int row) { return ALT ? swz_k2i(row) : swz_k2(row); }
 // N-contiguous tiles: 32 lanes of a transposing read touch 8 rows (k%4, k/8%2) x 32 bytes of one column block;
 // the XOR spreads them over the eight 32-byte slots of 256 bytes of banks. A row's chunks stay whole 128-byte lines.
 __device__ __forceinline__ int swz_n2(int k) { return ((k & 3) | (((k >> 3) & 1) << 2)) << 1; }
@@ -454,7 +460,7 @@ __device__ __forceinline__ int swz_n2(int k) { return ((k & 3) | (((k >> 3) & 1)
 // Copies are copy_to_lds() buffer loads: rows and column chunks outside the matrix are clamped by the loaders,
 // per-lane offsets stay below 2^31 (checked by the launcher).
 
-template <typename T, int ROWS>
+template <typename T, int ROWS, bool ALT = false>
 struct KMajorLoader2 {
   static constexpr int NI = ROWS / 32;              // 8 rows per wave-wide copy, four waves
   int voff[NI];
@@ -465,7 +471,7 @@ struct KMajorLoader2 {
     for (int j = 0; j < NI; ++j) {
       const int inst = j * 4 + wave;
       const int row = inst * 8 + lane / 8;
-      const int c = (lane % 8) ^ swz_k2(row);
+      const int c = (lane % 8) ^ swz_k2_sel<ALT>(row);
       int grow = row0 + row;
       grow = grow < row_max ? grow : row_max;
       voff[j] = (int)(((int64_t)(grow - row0) * ld + c * kChunk) * (int64_t)sizeof(T));
@@ -502,10 +508,10 @@ struct NMajorLoader2 {
   }
 };
 
-template <typename T>
+template <typename T, bool ALT = false>
 __device__ __forceinline__ typename Mfma<T>::Frag read_kmajor2(const T* lds, int row, int chunk) {
   typedef typename Mfma<T>::Frag Frag;
-  return *reinterpret_cast<const Frag*>(lds + row * BK2 + ((chunk ^ swz_k2(row)) * kChunk));
+  return *reinterpret_cast<const Frag*>(lds + row * BK2 + ((chunk ^ swz_k2_sel<ALT>(row)) * kChunk));
 }
 
 // ds_read_tr16_b64: 16 lanes hand in the addresses of a [4 k x 16 columns] block (lane i: row i/4, columns
@@ -530,7 +536,8 @@ __device__ __forceinline__ typename Mfma<T>::Frag read_nmajor2(const T* lds, int
 
 // Weight-only quantised B: int8 [N,K] rows, 64 bytes per row and slab (four 16-byte chunks, 16 rows per copy),
 // kept as int8 in LDS and widened to fp16 in registers, one fragment (8 values of one row) at a time.
-__device__ __forceinline__ int swz_k8(int row) { return (row >> 2) & 3; }      // row pitch 64 B
+// row pitch 64 B. (row >> 2) & 3 also gives every 16 lanes sixteen different slots, but reads at half the rate.
+__device__ __forceinline__ int swz_k8(int row) { return (row >> 1) & 3; }
 template <int ROWS>
 struct I8RowLoader2 {
   static constexpr int NI = ROWS / 64;              // 16 rows per wave-wide copy, four waves
@@ -655,7 +662,7 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
     }
   }
 
-  KMajorLoader2<T, BM> load_a;
+  KMajorLoader2<T, BM, B_I8> load_a;
   load_a.init(lda, m0, M - 1, wave, lane);
   KMajorLoader2<T, BN> load_bk;
   NMajorLoader2<T, BN> load_bn;
@@ -683,7 +690,7 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
   // fragments of step ks (32 elements of K): lane holds row/column lane%16 of a tile, K group lane/16 (8 elements)
   auto read_a = [&](const T* src, int ks, int i) __attribute__((always_inline)) {
     // int8 B fixes the K slots of a step as k = 16*(lane/16) + 8*step + 0..7 (see read_i8row)
-    return read_kmajor2<T>(src, (wm * TM + i) * 16 + lane % 16, B_I8 ? 2 * (lane / 16) + ks : ks * 4 + lane / 16);
+    return read_kmajor2<T, B_I8>(src, (wm * TM + i) * 16 + lane % 16, B_I8 ? 2 * (lane / 16) + ks : ks * 4 + lane / 16);
   };
   auto read_b = [&](const BT* src, int ks, int j) __attribute__((always_inline)) {
     if constexpr (B_I8) return Frag{};              // int8 B is read raw (read_b8) and widened later

@@ -53,6 +53,8 @@ SIGNATURES = {
     "hexmi_rope": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _f64, _int, _ptr]),
     "hexmi_mfma_peak_flops": (_f64, [_int, _int, _i64]),
     "hexmi_mfma_peak": (_int, [_int, _int, _ptr, _i64, _int, _ptr, _ptr]),
+    "hexmi_issue_slots": (_int, [_int, _int, _int, _i64, _int, _ptr, _ptr]),
+    "hexmi_lds_read_pattern": (_int, [_int, _i64, _ptr, _ptr]),
     "hexmi_attention": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _ptr]),
 }
 

@@ -334,6 +334,30 @@ double hexmi_mfma_peak_flops(int shape, int waves_per_simd, int64_t iters);
 int hexmi_mfma_peak(int shape, int dtype, const void *operands, int64_t iters,
                     int waves_per_simd, float *sink, hexmi_stream_t stream);
 
+/* Two more measurement aids without a counterpart in the reference, both one
+ * workgroup per compute unit, sink as above (hexmi_lds_read_pattern: 1024
+ * floats per compute unit).
+ *
+ * hexmi_issue_slots: per MFMA of a registers-only stream (shape as above, fp16,
+ * zero operands, 64 accumulator registers) per_mfma vector instructions of one
+ * kind follow in the same wave: kind 0 = v_pk_add_f16, 1 = v_fma_f32,
+ * 2 = v_exp_f32; per_mfma in {0,1,2,3,4,5,6,8}. The time per MFMA says how much
+ * vector work a kernel can place between its MFMAs before the SIMD's
+ * instruction issue, not the matrix pipe, sets the pace. The launch runs
+ * iters * (4 for shape 0, 16 for shape 1) MFMAs per wave.
+ *
+ * hexmi_lds_read_pattern: 16 waves per compute unit issue only wave-wide
+ * 16-byte LDS reads (iters * 8 per wave) with the lane-to-address pattern of
+ * one of the tiled GEMM's fragment reads: 0 linear; 1 fp16 rows of 128 bytes
+ * read as chunk 4*step + lane/16, swizzle (row>>1)&7; 2 the same rows read as
+ * chunk 2*(lane/16) + step; 3 pattern 2 with the swizzle the int8-weight
+ * kernel uses; 4 int8 rows of 64 bytes, swizzle (row>>2)&3; 5 the same with
+ * (row>>1)&3 (in use); 6 pattern 1 unswizzled. */
+int hexmi_issue_slots(int shape, int kind, int per_mfma, int64_t iters,
+                      int waves_per_simd, float *sink, hexmi_stream_t stream);
+int hexmi_lds_read_pattern(int pattern, int64_t iters, float *sink,
+                           hexmi_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
