@@ -226,18 +226,24 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
 // CU, each owning an equal contiguous range of at most 48 output channels, so the weights cross HBM once, in
 // contiguous 256-byte row segments. K is walked in chunks of 256. The raw int8 weight chunk [48][256] and the
 // activation chunk [MB*16][256] fp16 are copied global -> LDS (global_load_lds, no registers) by different
-// waves: waves 12..15 copy weights, four chunks ahead (five stages; this is the HBM stream, it needs the depth),
-// waves 0..3*MB-1 copy activations, two chunks ahead (three stages; L2 hits). A wave's outstanding-copy counter
-// only sees its own copies, so each role waits with its own count and the workgroup barrier publishes both.
-// Wave w < 3*MB also owns the 16 x 16 output tile (row block w/3, channel tile w%3) for the whole K loop, so
-// there is no cross-wave reduction: it reads its fragments back from LDS (16-byte chunks XOR-swizzled by row
-// through the copy's source addresses, conflict-free), converts the int8 bytes in registers and keeps one
-// accumulator. Every copying wave issues exactly three copies per chunk (repeats of real ones fill the slots and
-// rewrite the same bytes).
+// waves: waves 12..15 copy weights, four chunks ahead (five stages: three or four measured the same, seven and
+// nine 5-10 % slower), waves 0..11 copy activations, two chunks ahead (three stages; L2 hits). A wave's
+// outstanding-copy counter only sees its own copies, so each role waits with its own count and the workgroup
+// barrier publishes both.
+// Compute wave w < 12 owns channel tile w % 3 and the quarter w / 3 of every chunk (64 of its 256 k) for ALL row
+// blocks: it converts its 16 x 64 int8 weights to fp16 once per chunk (20 vector instructions) and multiplies them
+// into MB accumulators (2 * MB MFMAs). A SIMD issues one instruction at a time and a 16x16x32 MFMA hides only two
+// vector instructions, so the conversions per MFMA set the pace: with one 16 x 16 tile per wave (every row-block
+// wave converting the same weights, 10 instructions per MFMA) the kernel took 18.4 us at M = 64, N = 11008, K = 4096,
+// this way 15.0 (22.6 -> 18.7 with the weights coming from HBM). Fragments are read back from LDS in 16-byte chunks
+// XOR-swizzled by row through the copies' source addresses (conflict-free). The four K quarters of a tile are
+// summed through LDS after the K loop, in a fixed order. Every copying wave issues exactly three copies per chunk
+// (repeats of real ones fill the slots and rewrite the same bytes).
 constexpr int kMidKC = 256;                                 // K per chunk
 constexpr int kMidCh = 48;                                  // channels per workgroup (three tiles of 16)
 constexpr int kMidSlots = 3;                                // copies per copying wave per chunk
 constexpr int kMidAStages = 3, kMidWStages = 5;
+constexpr int kMidCompute = 12;                             // compute waves: three channel tiles x four K quarters
 constexpr int kMidWWave0 = 12;                              // first of the four weight-copy waves
 
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
@@ -250,18 +256,15 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   __shared__ __attribute__((aligned(16))) f16 a_s0[MB * 16 * kMidKC];
   __shared__ __attribute__((aligned(16))) f16 a_s1[MB * 16 * kMidKC];
   __shared__ __attribute__((aligned(16))) f16 a_s2[MB * 16 * kMidKC];
-  __shared__ __attribute__((aligned(16))) int8_t w_s0[kMidCh * kMidKC];
-  __shared__ __attribute__((aligned(16))) int8_t w_s1[kMidCh * kMidKC];
-  __shared__ __attribute__((aligned(16))) int8_t w_s2[kMidCh * kMidKC];
-  __shared__ __attribute__((aligned(16))) int8_t w_s3[kMidCh * kMidKC];
-  __shared__ __attribute__((aligned(16))) int8_t w_s4[kMidCh * kMidKC];
+  constexpr int WS = kMidWStages;
+  __shared__ __attribute__((aligned(16))) int8_t w_s[WS][kMidCh * kMidKC];
 
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int r16 = lane % 16, kg = lane / 16;
   const int n_begin = blockIdx.x * chan_per_wg;
   const int n_end = n_begin + chan_per_wg < N ? n_begin + chan_per_wg : N;
   const int n_chunks = K / kMidKC;
-  const bool computes = wave < 3 * MB;                      // also copies activations
+  const bool computes = wave < kMidCompute;                 // also copies activations
   const bool copies_w = wave >= kMidWWave0;
 
   // ---- copy slots. Activation copy i (0 .. 8*MB-1) moves rows 2i, 2i+1 (512 bytes each); weight copy t (0 .. 11)
@@ -273,7 +276,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     slot_src[j] = nullptr;
     slot_dst[j] = 0;
     if (computes) {
-      const int i = (j * 3 * MB + wave) % (8 * MB);
+      const int i = (j * kMidCompute + wave) % (8 * MB);
       const int row = 2 * i + lane / 32;
       const int c = lane % 32;                              // 16-byte position inside the row's 512 bytes
       const int src_c = (c & 16) | ((c ^ row) & 15);        // the chunk that belongs at this position
@@ -290,9 +293,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     }
   }
   auto a_stage = [&](int i) __attribute__((always_inline)) { return i == 0 ? a_s0 : (i == 1 ? a_s1 : a_s2); };
-  auto w_stage = [&](int i) __attribute__((always_inline)) {
-    return i == 0 ? w_s0 : (i == 1 ? w_s1 : (i == 2 ? w_s2 : (i == 3 ? w_s3 : w_s4)));
-  };
+  auto w_stage = [&](int i) __attribute__((always_inline)) { return w_s[i]; };
   // chunk indices past the end repeat the last chunk (copied, never read): every chunk issues the same copies
   auto issue_a = [&](int chunk, f16* dst) __attribute__((always_inline)) {
     const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
@@ -309,22 +310,26 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
                                        HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, 0);
   };
 
-  // ---- fragment side: wave < 3*MB owns row block mb, channel tile nt
-  const int mb = wave / 3, nt = wave % 3;
-  int w_off[4], a_off[4][2];
+  // ---- fragment side: compute wave w owns channel tile nt = w % 3 and the quarter kq = w / 3 of every chunk
+  //      (64 of its 256 k), for all MB row blocks
+  const int nt = wave % 3, kq = wave / 3;
+  int w_off, a_off[MB][2];
   {
-    const int wrow = nt * 16 + r16, arow = mb * 16 + r16;
+    const int wrow = nt * 16 + r16;
+    w_off = wrow * kMidKC + (((kq * 4 + kg) ^ wrow) & 15) * 16;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      w_off[ks] = wrow * kMidKC + (((ks * 4 + kg) ^ wrow) & 15) * 16;
+    for (int rb = 0; rb < MB; ++rb) {
+      const int arow = rb * 16 + r16;
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int c = ks * 8 + kg * 2 + h;
-        a_off[ks][h] = arow * kMidKC * 2 + ((c & 16) | ((c ^ arow) & 15)) * 16;
+        const int c = kq * 8 + kg * 2 + h;
+        a_off[rb][h] = arow * kMidKC * 2 + ((c & 16) | ((c ^ arow) & 15)) * 16;
       }
     }
   }
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[MB];
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
   // The fragment reads are written as inline assembly: the compiler cannot tell which stage an in-flight
   // global_load_lds writes and would make every LDS read wait for all of them (vmcnt(0)), which undoes the
   // pipelining. The waits this kernel needs are the explicit ones around the barrier.
@@ -332,29 +337,52 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   auto multiply = [&](const f16* a_src, const int8_t* w_src) __attribute__((always_inline)) {
     const unsigned a_base = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(a_src);
     const unsigned w_base = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(w_src);
-    u32x4 raw[4], a0[4], a1[4];
-    asm volatile(
-        "ds_read_b128 %0, %12\n\tds_read_b128 %1, %13\n\tds_read_b128 %2, %14\n\tds_read_b128 %3, %15\n\t"
-        "ds_read_b128 %4, %16\n\tds_read_b128 %5, %17\n\tds_read_b128 %6, %18\n\tds_read_b128 %7, %19\n\t"
-        "ds_read_b128 %8, %20\n\tds_read_b128 %9, %21\n\tds_read_b128 %10, %22\n\tds_read_b128 %11, %23\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(raw[0]), "=&v"(raw[1]), "=&v"(raw[2]), "=&v"(raw[3]), "=&v"(a0[0]), "=&v"(a0[1]), "=&v"(a0[2]),
-          "=&v"(a0[3]), "=&v"(a1[0]), "=&v"(a1[1]), "=&v"(a1[2]), "=&v"(a1[3])
-        : "v"(w_base + w_off[0]), "v"(w_base + w_off[1]), "v"(w_base + w_off[2]), "v"(w_base + w_off[3]),
-          "v"(a_base + a_off[0][0]), "v"(a_base + a_off[1][0]), "v"(a_base + a_off[2][0]), "v"(a_base + a_off[3][0]),
-          "v"(a_base + a_off[0][1]), "v"(a_base + a_off[1][1]), "v"(a_base + a_off[2][1]), "v"(a_base + a_off[3][1])
-        : "memory");
+    u32x4 raw, a0[MB], a1[MB];
+    if constexpr (MB == 4) {
+      asm volatile(
+          "ds_read_b128 %0, %9\n\tds_read_b128 %1, %10\n\tds_read_b128 %2, %11\n\tds_read_b128 %3, %12\n\t"
+          "ds_read_b128 %4, %13\n\tds_read_b128 %5, %14\n\tds_read_b128 %6, %15\n\tds_read_b128 %7, %16\n\t"
+          "ds_read_b128 %8, %17\n\ts_waitcnt lgkmcnt(0)"
+          : "=&v"(raw), "=&v"(a0[0]), "=&v"(a1[0]), "=&v"(a0[1]), "=&v"(a1[1]), "=&v"(a0[2]), "=&v"(a1[2]), "=&v"(a0[3]),
+            "=&v"(a1[3])
+          : "v"(w_base + w_off), "v"(a_base + a_off[0][0]), "v"(a_base + a_off[0][1]), "v"(a_base + a_off[1][0]),
+            "v"(a_base + a_off[1][1]), "v"(a_base + a_off[2][0]), "v"(a_base + a_off[2][1]), "v"(a_base + a_off[3][0]),
+            "v"(a_base + a_off[3][1])
+          : "memory");
+    } else if constexpr (MB == 3) {
+      asm volatile(
+          "ds_read_b128 %0, %7\n\tds_read_b128 %1, %8\n\tds_read_b128 %2, %9\n\tds_read_b128 %3, %10\n\t"
+          "ds_read_b128 %4, %11\n\tds_read_b128 %5, %12\n\tds_read_b128 %6, %13\n\ts_waitcnt lgkmcnt(0)"
+          : "=&v"(raw), "=&v"(a0[0]), "=&v"(a1[0]), "=&v"(a0[1]), "=&v"(a1[1]), "=&v"(a0[2]), "=&v"(a1[2])
+          : "v"(w_base + w_off), "v"(a_base + a_off[0][0]), "v"(a_base + a_off[0][1]), "v"(a_base + a_off[1][0]),
+            "v"(a_base + a_off[1][1]), "v"(a_base + a_off[2][0]), "v"(a_base + a_off[2][1])
+          : "memory");
+    } else if constexpr (MB == 2) {
+      asm volatile(
+          "ds_read_b128 %0, %5\n\tds_read_b128 %1, %6\n\tds_read_b128 %2, %7\n\tds_read_b128 %3, %8\n\t"
+          "ds_read_b128 %4, %9\n\ts_waitcnt lgkmcnt(0)"
+          : "=&v"(raw), "=&v"(a0[0]), "=&v"(a1[0]), "=&v"(a0[1]), "=&v"(a1[1])
+          : "v"(w_base + w_off), "v"(a_base + a_off[0][0]), "v"(a_base + a_off[0][1]), "v"(a_base + a_off[1][0]),
+            "v"(a_base + a_off[1][1])
+          : "memory");
+    } else {
+      asm volatile(
+          "ds_read_b128 %0, %3\n\tds_read_b128 %1, %4\n\tds_read_b128 %2, %5\n\ts_waitcnt lgkmcnt(0)"
+          : "=&v"(raw), "=&v"(a0[0]), "=&v"(a1[0])
+          : "v"(w_base + w_off), "v"(a_base + a_off[0][0]), "v"(a_base + a_off[0][1])
+          : "memory");
+    }
+    f16x8 w0, w1;
+    cvt16(raw, w0, w1);                                     // converted once, used for every row block
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      f16x8 w0, w1;
-      cvt16(raw[ks], w0, w1);
+    for (int rb = 0; rb < MB; ++rb) {
       // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, __builtin_bit_cast(f16x8, a0[ks]), acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, __builtin_bit_cast(f16x8, a1[ks]), acc, 0, 0, 0);
+      acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, __builtin_bit_cast(f16x8, a0[rb]), acc[rb], 0, 0, 0);
+      acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, __builtin_bit_cast(f16x8, a1[rb]), acc[rb], 0, 0, 0);
     }
   };
   // s_waitcnt immediates (gfx9 encoding), LDS counter untouched: copies of the newer chunks may stay in flight
-  constexpr int kNewerA = (kMidAStages - 2) * kMidSlots, kNewerW = (kMidWStages - 2) * kMidSlots;
+  constexpr int kNewerA = (kMidAStages - 2) * kMidSlots, kNewerW = (WS - 2) * kMidSlots;
   constexpr int kWaitA = (kNewerA & 0xF) | ((kNewerA >> 4) << 14) | (0x7 << 4) | (0xF << 8);
   constexpr int kWaitW = (kNewerW & 0xF) | ((kNewerW >> 4) << 14) | (0x7 << 4) | (0xF << 8);
 
@@ -374,14 +402,12 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     issue_a(0, a_s0);
     issue_a(1, a_s1);
   } else if (copies_w) {
-    issue_w(0, w_s0);
-    issue_w(1, w_s1);
-    issue_w(2, w_s2);
-    issue_w(3, w_s3);
+#pragma unroll
+    for (int i = 0; i < WS - 1; ++i) issue_w(i, w_s[i]);
   }
 #pragma unroll
   for (int e = 0; e < 4; ++e) asm volatile("" : "+v"(sc[e]));
-  constexpr int kPeriod = kMidAStages * kMidWStages;        // stage assignment repeats every 15 chunks
+  constexpr int kPeriod = WS % kMidAStages == 0 ? WS : kMidAStages * WS;   // the stage assignment repeats
   for (int base = 0; base < n_chunks; base += kPeriod) {
 #pragma unroll
     for (int u = 0; u < kPeriod; ++u) {
@@ -394,22 +420,41 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
         __builtin_amdgcn_s_barrier();
         if (computes) {
           issue_a(chunk + 2, a_stage((u + 2) % kMidAStages));
-          multiply(a_stage(u % kMidAStages), w_stage(u % kMidWStages));
+          multiply(a_stage(u % kMidAStages), w_stage(u % WS));
         } else if (copies_w) {
-          issue_w(chunk + 4, w_stage((u + 4) % kMidWStages));
+          issue_w(chunk + WS - 1, w_stage((u + WS - 1) % WS));
         }
       }
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // trailing copies land before the LDS is released
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // trailing copies land before the stages are reused
+  __syncthreads();
 
-  if (computes) {
-    const int gm = mb * 16 + r16;
-    const int gn = n_begin + nt * 16 + kg * 4;
-    if (gm < M) {
+  // the four K quarters of a tile are summed through the first two activation stages (quarters 1 and 2 in the
+  // first, quarter 3 in the second: MB KiB per wave), in the fixed order 0 + 1 + 2 + 3
+  float* red0 = reinterpret_cast<float*>(a_s0);
+  float* red1 = reinterpret_cast<float*>(a_s1);
+  static_assert(2 * 3 * MB * 1024 <= MB * 16 * kMidKC * 2, "two quarters of partial tiles fit one activation stage");
+  if (computes && kq > 0) {
+    float* dst = kq < 3 ? red0 + ((kq - 1) * 3 + nt) * MB * 256 : red1 + nt * MB * 256;
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (gn + e < n_end) C[(int64_t)gm * N + gn + e] = (f16)(acc[e] * (float)sc[e]);
+    for (int rb = 0; rb < MB; ++rb) *reinterpret_cast<f32x4*>(dst + (rb * 64 + lane) * 4) = acc[rb];
+  }
+  __syncthreads();
+  if (computes && kq == 0) {
+    const int gn = n_begin + nt * 16 + kg * 4;
+#pragma unroll
+    for (int rb = 0; rb < MB; ++rb) {
+      f32x4 sum = acc[rb];
+      sum += *reinterpret_cast<const f32x4*>(red0 + (nt * MB * 64 + rb * 64 + lane) * 4);
+      sum += *reinterpret_cast<const f32x4*>(red0 + ((3 + nt) * MB * 64 + rb * 64 + lane) * 4);
+      sum += *reinterpret_cast<const f32x4*>(red1 + (nt * MB * 64 + rb * 64 + lane) * 4);
+      const int gm = rb * 16 + r16;
+      if (gm < M) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (gn + e < n_end) C[(int64_t)gm * N + gn + e] = (f16)(sum[e] * (float)sc[e]);
+      }
     }
   }
 }
