@@ -113,7 +113,8 @@ void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const
   }
 }
 
-// Up to 16 activation rows, K <= 4096: persistent workgroups of 16 waves, one per compute unit. The per-CU rate
+// Up to 16 activation rows, K <= 4096 (used for M <= 8, and for M <= 16 on pre-packed weights; 9 .. 16 rows of
+// plain weights go through the chunked kernel further down): persistent workgroups of 16 waves, one per compute unit. The per-CU rate
 // of the 16-row strided weight reads is what bounds this shape, so the output channels are dealt in equal
 // contiguous ranges over exactly as many workgroups as there are CUs (N = 11008 on 256 CUs: 43 channels each,
 // walked as tiles of 16, 16 and 11 channels; the lanes of a short tile re-read its last row and drop the result).
@@ -222,29 +223,42 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
   }
 }
 
-// 16 < M <= 64 (MB = 2..4 blocks of 16 activation rows), K % 256 == 0: one persistent workgroup of 16 waves per
+// 16 < M <= 128 (MB = 2..8 blocks of 16 activation rows), K % 256 == 0: one persistent workgroup of 16 waves per
 // CU, each owning an equal contiguous range of at most 48 output channels, so the weights cross HBM once, in
-// contiguous 256-byte row segments. K is walked in chunks of 256. The raw int8 weight chunk [48][256] and the
-// activation chunk [MB*16][256] fp16 are copied global -> LDS (global_load_lds, no registers) by different
-// waves: waves 12..15 copy weights, four chunks ahead (five stages: three or four measured the same, seven and
-// nine 5-10 % slower), waves 0..11 copy activations, two chunks ahead (three stages; L2 hits). A wave's
-// outstanding-copy counter only sees its own copies, so each role waits with its own count and the workgroup
-// barrier publishes both.
-// Compute wave w < 12 owns channel tile w % 3 and the quarter w / 3 of every chunk (64 of its 256 k) for ALL row
-// blocks: it converts its 16 x 64 int8 weights to fp16 once per chunk (20 vector instructions) and multiplies them
-// into MB accumulators (2 * MB MFMAs). A SIMD issues one instruction at a time and a 16x16x32 MFMA hides only two
-// vector instructions, so the conversions per MFMA set the pace: with one 16 x 16 tile per wave (every row-block
-// wave converting the same weights, 10 instructions per MFMA) the kernel took 18.4 us at M = 64, N = 11008, K = 4096,
-// this way 15.0 (22.6 -> 18.7 with the weights coming from HBM). Fragments are read back from LDS in 16-byte chunks
-// XOR-swizzled by row through the copies' source addresses (conflict-free). The four K quarters of a tile are
-// summed through LDS after the K loop, in a fixed order. Every copying wave issues exactly three copies per chunk
-// (repeats of real ones fill the slots and rewrite the same bytes).
-constexpr int kMidKC = 256;                                 // K per chunk
+// contiguous row segments. K is walked in chunks of KC = 256 (MB <= 4) or 128 (MB = 8): an activation chunk is at
+// most 32 KiB. The raw int8 weight chunk [48][KC] and the activation chunk [MB*16][KC] fp16 are copied
+// global -> LDS (global_load_lds, no registers) by different waves: waves 12..15 copy weights, four chunks ahead
+// (five stages: three or four measured the same, seven and nine 5-10 % slower), waves 0..11 copy activations, two
+// chunks ahead (three stages; L2 hits). A wave's outstanding-copy counter only sees its own copies, so each role
+// waits with its own count and the workgroup barrier publishes both.
+// Compute wave w < 12 owns channel tile w % 3 and, of every chunk, one unit of 64 k for one group of row blocks
+// (four K units and all row blocks at KC = 256; two units and two groups of four row blocks at KC = 128). It converts
+// its 16 x 64 int8 weights to fp16 once per chunk (20 vector instructions) and multiplies them into its RB
+// accumulators (2 * RB MFMAs). A SIMD issues one instruction at a time and a 16x16x32 MFMA hides only two vector
+// instructions, so the conversions per MFMA set the pace: with one 16 x 16 tile per wave (every row-block wave
+// converting the same weights, 10 instructions per MFMA) the kernel took 18.4 us at M = 64, N = 11008, K = 4096,
+// this way 15.0 (22.6 -> 21.1 with the weights coming from HBM). Fragments are read back from LDS in 16-byte chunks
+// permuted inside their row through the copies' source addresses (conflict-free). The K units of a tile are summed
+// through LDS after the K loop, in a fixed order.
+// With every CU fetching all of A the kernel moves M * 8 KiB per CU through L2: 29 us at M = 128 (the 128 x 128
+// tile kernel, 86 tiles: 34), but 47 us at M = 256 with 64-k chunks (tile kernel: 37), so it stops at 128 rows.
 constexpr int kMidCh = 48;                                  // channels per workgroup (three tiles of 16)
-constexpr int kMidSlots = 3;                                // copies per copying wave per chunk
 constexpr int kMidAStages = 3, kMidWStages = 5;
-constexpr int kMidCompute = 12;                             // compute waves: three channel tiles x four K quarters
+constexpr int kMidCompute = 12;                             // compute waves: three channel tiles x four (unit, group)
 constexpr int kMidWWave0 = 12;                              // first of the four weight-copy waves
+constexpr int kMidMaxM = 128;
+constexpr int mid_kc(int mb) { return mb <= 4 ? 256 : 128; }
+
+// position of 16-byte chunk c inside its row of CH chunks (an involution in c for a given row); rows of 256 and
+// 512 bytes start at the same banks, so the row number itself spreads the chunks
+template <int CH> __device__ __forceinline__ int mid_a_pos(int c, int row) {
+  if constexpr (CH == 32) return (c & 16) | ((c ^ row) & 15);
+  else return (c ^ row) & 15;
+}
+template <int CH> __device__ __forceinline__ int mid_w_pos(int c, int row) {
+  if constexpr (CH == 16) return (c ^ row) & 15;
+  else return (c ^ (row >> 1)) & 7;                         // 128-byte rows read as chunk 4u + g
+}
 
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -253,203 +267,212 @@ template <int MB>
 __global__ __launch_bounds__(1024)
 void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
                       f16* __restrict__ C, int M, int N, int K, int chan_per_wg) {
-  __shared__ __attribute__((aligned(16))) f16 a_s0[MB * 16 * kMidKC];
-  __shared__ __attribute__((aligned(16))) f16 a_s1[MB * 16 * kMidKC];
-  __shared__ __attribute__((aligned(16))) f16 a_s2[MB * 16 * kMidKC];
+  constexpr int KC = mid_kc(MB);
+  constexpr int KU = KC / 64;                               // 64-k units per chunk
+  constexpr int RG = 4 / KU;                                // row-block groups
+  constexpr int RB = MB / RG;                               // row blocks per compute wave
+  static_assert(MB % RG == 0 && RB >= 1 && RB <= 4, "row blocks split evenly over the groups");
+  constexpr int ACH = KC / 8, WCH = KC / 16;                // 16-byte chunks per activation / weight row
+  constexpr int NAC = MB * KC / 32, NWC = kMidCh * KC / 1024;   // 1 KiB copies per chunk
+  constexpr int ASL = (NAC + kMidCompute - 1) / kMidCompute, WSL = (NWC + 3) / 4;   // copy slots per wave
+  constexpr int SL = ASL > WSL ? ASL : WSL;
   constexpr int WS = kMidWStages;
-  __shared__ __attribute__((aligned(16))) int8_t w_s[WS][kMidCh * kMidKC];
+  __shared__ __attribute__((aligned(16))) f16 a_s[kMidAStages][MB * 16 * KC];
+  __shared__ __attribute__((aligned(16))) int8_t w_s[WS][kMidCh * KC];
 
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int r16 = lane % 16, kg = lane / 16;
   const int n_begin = blockIdx.x * chan_per_wg;
   const int n_end = n_begin + chan_per_wg < N ? n_begin + chan_per_wg : N;
-  const int n_chunks = K / kMidKC;
+  const int n_chunks = K / KC;
   const bool computes = wave < kMidCompute;                 // also copies activations
   const bool copies_w = wave >= kMidWWave0;
 
-  // ---- copy slots. Activation copy i (0 .. 8*MB-1) moves rows 2i, 2i+1 (512 bytes each); weight copy t (0 .. 11)
-  //      moves rows 4t .. 4t+3 (256 bytes each). Lane positions are permuted inside a row (see the fragment side).
-  const char* slot_src[kMidSlots];                          // source of this lane for chunk 0
-  int slot_dst[kMidSlots];                                  // byte offset of the copy inside its stage
+  // ---- copy slots: every copy moves 1 KiB (1024 / row bytes whole rows); lane positions are permuted inside a row
+  //      (see the fragment side). Slots past the last real copy repeat one (same bytes, rewritten).
+  const char* slot_src[SL];                                 // source of this lane for chunk 0
+  int slot_dst[SL];                                         // byte offset of the copy inside its stage
 #pragma unroll
-  for (int j = 0; j < kMidSlots; ++j) {
+  for (int j = 0; j < SL; ++j) {
     slot_src[j] = nullptr;
     slot_dst[j] = 0;
-    if (computes) {
-      const int i = (j * kMidCompute + wave) % (8 * MB);
-      const int row = 2 * i + lane / 32;
-      const int c = lane % 32;                              // 16-byte position inside the row's 512 bytes
-      const int src_c = (c & 16) | ((c ^ row) & 15);        // the chunk that belongs at this position
+    if (computes && j < ASL) {
+      const int i = (j * kMidCompute + wave) % NAC;
+      const int row = i * (64 / ACH) + lane / ACH;          // 64 chunks per copy
+      const int src_c = mid_a_pos<ACH>(lane % ACH, row);    // the chunk that belongs at this position
       slot_src[j] = reinterpret_cast<const char*>(A + (int64_t)(row < M ? row : M - 1) * K) + src_c * 16;
       slot_dst[j] = i * 1024;
-    } else if (copies_w) {
-      const int t = j * 4 + (wave - kMidWWave0);
-      const int row = 4 * t + lane / 16;
-      const int c = lane % 16;
-      const int src_c = (c ^ row) & 15;
+    } else if (copies_w && j < WSL) {
+      const int t = (j * 4 + (wave - kMidWWave0)) % NWC;
+      const int row = t * (64 / WCH) + lane / WCH;
+      const int src_c = mid_w_pos<WCH>(lane % WCH, row);
       const int n = n_begin + row < n_end ? n_begin + row : n_end - 1;
       slot_src[j] = reinterpret_cast<const char*>(W + (int64_t)n * K) + src_c * 16;
       slot_dst[j] = t * 1024;
     }
   }
-  auto a_stage = [&](int i) __attribute__((always_inline)) { return i == 0 ? a_s0 : (i == 1 ? a_s1 : a_s2); };
-  auto w_stage = [&](int i) __attribute__((always_inline)) { return w_s[i]; };
   // chunk indices past the end repeat the last chunk (copied, never read): every chunk issues the same copies
   auto issue_a = [&](int chunk, f16* dst) __attribute__((always_inline)) {
     const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
 #pragma unroll
-    for (int j = 0; j < kMidSlots; ++j)
-      __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * kMidKC * 2),
+    for (int j = 0; j < ASL; ++j)
+      __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * KC * 2),
                                        HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, 0);
   };
   auto issue_w = [&](int chunk, int8_t* dst) __attribute__((always_inline)) {
     const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
 #pragma unroll
-    for (int j = 0; j < kMidSlots; ++j)
-      __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * kMidKC),
+    for (int j = 0; j < WSL; ++j)
+      __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * KC),
                                        HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, 0);
   };
 
-  // ---- fragment side: compute wave w owns channel tile nt = w % 3 and the quarter kq = w / 3 of every chunk
-  //      (64 of its 256 k), for all MB row blocks
-  const int nt = wave % 3, kq = wave / 3;
-  int w_off, a_off[MB][2];
+  // ---- fragment side: compute wave w owns channel tile nt = w % 3, K unit ku and row-block group rg
+  const int nt = wave % 3, ku = (wave / 3) % KU, rg = (wave / 3) / KU;
+  // A chunk's position depends on the row only through its low four bits, so row block rb of the group is a
+  // constant 16 * KC * 2 * rb bytes further: an immediate offset of the read, not a register.
+  int w_off, a_off[2];
   {
     const int wrow = nt * 16 + r16;
-    w_off = wrow * kMidKC + (((kq * 4 + kg) ^ wrow) & 15) * 16;
+    w_off = wrow * KC + mid_w_pos<WCH>(ku * 4 + kg, wrow) * 16;
+    const int arow = rg * RB * 16 + r16;
 #pragma unroll
-    for (int rb = 0; rb < MB; ++rb) {
-      const int arow = rb * 16 + r16;
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int c = kq * 8 + kg * 2 + h;
-        a_off[rb][h] = arow * kMidKC * 2 + ((c & 16) | ((c ^ arow) & 15)) * 16;
-      }
-    }
+    for (int h = 0; h < 2; ++h) a_off[h] = arow * KC * 2 + mid_a_pos<ACH>(ku * 8 + kg * 2 + h, arow) * 16;
   }
-  f32x4 acc[MB];
+  static_assert((RB - 1) * 16 * KC * 2 < 65536, "row-block offsets fit the read's immediate");
+  f32x4 acc[RB];
 #pragma unroll
-  for (int rb = 0; rb < MB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
   // The fragment reads are written as inline assembly: the compiler cannot tell which stage an in-flight
   // global_load_lds writes and would make every LDS read wait for all of them (vmcnt(0)), which undoes the
   // pipelining. The waits this kernel needs are the explicit ones around the barrier.
-  // One statement holds the reads and the wait for them, so no register of the result can be touched early.
-  auto multiply = [&](const f16* a_src, const int8_t* w_src) __attribute__((always_inline)) {
+  // Fragments are double-buffered in registers: the reads of chunk u+1 are issued before the arithmetic of chunk u
+  // and waited for at the top of the next round, so the LDS latency passes under the conversions and MFMAs. The wait
+  // statement names every fragment register as modified: nothing that uses one can be scheduled above it.
+  struct Frags { u32x4 raw, a0[RB], a1[RB]; };
+  auto read_frags = [&](Frags& f, const f16* a_src, const int8_t* w_src) __attribute__((always_inline)) {
     const unsigned a_base = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(a_src);
     const unsigned w_base = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(w_src);
-    u32x4 raw, a0[MB], a1[MB];
-    if constexpr (MB == 4) {
-      asm volatile(
-          "ds_read_b128 %0, %9\n\tds_read_b128 %1, %10\n\tds_read_b128 %2, %11\n\tds_read_b128 %3, %12\n\t"
-          "ds_read_b128 %4, %13\n\tds_read_b128 %5, %14\n\tds_read_b128 %6, %15\n\tds_read_b128 %7, %16\n\t"
-          "ds_read_b128 %8, %17\n\ts_waitcnt lgkmcnt(0)"
-          : "=&v"(raw), "=&v"(a0[0]), "=&v"(a1[0]), "=&v"(a0[1]), "=&v"(a1[1]), "=&v"(a0[2]), "=&v"(a1[2]), "=&v"(a0[3]),
-            "=&v"(a1[3])
-          : "v"(w_base + w_off), "v"(a_base + a_off[0][0]), "v"(a_base + a_off[0][1]), "v"(a_base + a_off[1][0]),
-            "v"(a_base + a_off[1][1]), "v"(a_base + a_off[2][0]), "v"(a_base + a_off[2][1]), "v"(a_base + a_off[3][0]),
-            "v"(a_base + a_off[3][1])
-          : "memory");
-    } else if constexpr (MB == 3) {
-      asm volatile(
-          "ds_read_b128 %0, %7\n\tds_read_b128 %1, %8\n\tds_read_b128 %2, %9\n\tds_read_b128 %3, %10\n\t"
-          "ds_read_b128 %4, %11\n\tds_read_b128 %5, %12\n\tds_read_b128 %6, %13\n\ts_waitcnt lgkmcnt(0)"
-          : "=&v"(raw), "=&v"(a0[0]), "=&v"(a1[0]), "=&v"(a0[1]), "=&v"(a1[1]), "=&v"(a0[2]), "=&v"(a1[2])
-          : "v"(w_base + w_off), "v"(a_base + a_off[0][0]), "v"(a_base + a_off[0][1]), "v"(a_base + a_off[1][0]),
-            "v"(a_base + a_off[1][1]), "v"(a_base + a_off[2][0]), "v"(a_base + a_off[2][1])
-          : "memory");
-    } else if constexpr (MB == 2) {
-      asm volatile(
-          "ds_read_b128 %0, %5\n\tds_read_b128 %1, %6\n\tds_read_b128 %2, %7\n\tds_read_b128 %3, %8\n\t"
-          "ds_read_b128 %4, %9\n\ts_waitcnt lgkmcnt(0)"
-          : "=&v"(raw), "=&v"(a0[0]), "=&v"(a1[0]), "=&v"(a0[1]), "=&v"(a1[1])
-          : "v"(w_base + w_off), "v"(a_base + a_off[0][0]), "v"(a_base + a_off[0][1]), "v"(a_base + a_off[1][0]),
-            "v"(a_base + a_off[1][1])
-          : "memory");
-    } else {
-      asm volatile(
-          "ds_read_b128 %0, %3\n\tds_read_b128 %1, %4\n\tds_read_b128 %2, %5\n\ts_waitcnt lgkmcnt(0)"
-          : "=&v"(raw), "=&v"(a0[0]), "=&v"(a1[0])
-          : "v"(w_base + w_off), "v"(a_base + a_off[0][0]), "v"(a_base + a_off[0][1])
-          : "memory");
-    }
-    f16x8 w0, w1;
-    cvt16(raw, w0, w1);                                     // converted once, used for every row block
+    asm volatile("ds_read_b128 %0, %1" : "=&v"(f.raw) : "v"(w_base + w_off) : "memory");
+    const unsigned a_at0 = a_base + a_off[0], a_at1 = a_base + a_off[1];
 #pragma unroll
-    for (int rb = 0; rb < MB; ++rb) {
-      // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
-      acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, __builtin_bit_cast(f16x8, a0[rb]), acc[rb], 0, 0, 0);
-      acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, __builtin_bit_cast(f16x8, a1[rb]), acc[rb], 0, 0, 0);
+    for (int rb = 0; rb < RB; ++rb) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(f.a0[rb]) : "v"(a_at0), "n"(rb * 16 * KC * 2) : "memory");
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(f.a1[rb]) : "v"(a_at1), "n"(rb * 16 * KC * 2) : "memory");
     }
   };
+  auto wait_frags = [&](Frags& f) __attribute__((always_inline)) {
+    if constexpr (RB == 4)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.raw), "+v"(f.a0[0]), "+v"(f.a1[0]), "+v"(f.a0[1]), "+v"(f.a1[1]),
+                   "+v"(f.a0[2]), "+v"(f.a1[2]), "+v"(f.a0[3]), "+v"(f.a1[3]) :: "memory");
+    else if constexpr (RB == 3)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.raw), "+v"(f.a0[0]), "+v"(f.a1[0]), "+v"(f.a0[1]), "+v"(f.a1[1]),
+                   "+v"(f.a0[2]), "+v"(f.a1[2]) :: "memory");
+    else if constexpr (RB == 2)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.raw), "+v"(f.a0[0]), "+v"(f.a1[0]), "+v"(f.a0[1]), "+v"(f.a1[1]) :: "memory");
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.raw), "+v"(f.a0[0]), "+v"(f.a1[0]) :: "memory");
+  };
+  auto multiply = [&](const Frags& f) __attribute__((always_inline)) {
+    f16x8 w0, w1;
+    cvt16(f.raw, w0, w1);                                   // converted once, used for every row block
+    // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+      acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, __builtin_bit_cast(f16x8, f.a0[rb]), acc[rb], 0, 0, 0);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+      acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, __builtin_bit_cast(f16x8, f.a1[rb]), acc[rb], 0, 0, 0);
+  };
   // s_waitcnt immediates (gfx9 encoding), LDS counter untouched: copies of the newer chunks may stay in flight
-  constexpr int kNewerA = (kMidAStages - 2) * kMidSlots, kNewerW = (WS - 2) * kMidSlots;
+  constexpr int kNewerA = (kMidAStages - 2) * ASL, kNewerW = (WS - 2) * WSL;
   constexpr int kWaitA = (kNewerA & 0xF) | ((kNewerA >> 4) << 14) | (0x7 << 4) | (0xF << 8);
   constexpr int kWaitW = (kNewerW & 0xF) | ((kNewerW >> 4) << 14) | (0x7 << 4) | (0xF << 8);
 
-  // Channel scales of this lane's four outputs, requested before anything else: they come from HBM and would
-  // otherwise be waited for at the very end. The empty asm statements are uses on every path, which keeps the
-  // loads here instead of next to the stores.
-  f16 sc[4] = {(f16)0, (f16)0, (f16)0, (f16)0};
+  // prologue: activations of chunks 0, 1; weights of chunks 0 .. 3
   if (computes) {
+    issue_a(0, a_s[0]);
+    issue_a(1, a_s[1]);
+  } else if (copies_w) {
+#pragma unroll
+    for (int i = 0; i < WS - 1; ++i) issue_w(i, w_s[i]);
+  }
+  // Round u: chunk u+1 has landed for every wave after the barrier (each role waited for its own copies of it) and
+  // every wave has the fragments of chunk u in registers, so the stages of chunk u are free: the copies of chunk
+  // u+3 (activations) and u+WS (weights) go there. Then the fragments of chunk u+1 are requested and chunk u is
+  // multiplied. Round -1 (before the loop) fetches the fragments of chunk 0.
+  constexpr int kWaitA0 = (ASL & 0xF) | ((ASL >> 4) << 14) | (0x7 << 4) | (0xF << 8);                      // chunk 0 landed
+  constexpr int kWaitW0 = (((WS - 2) * WSL) & 0xF) | ((((WS - 2) * WSL) >> 4) << 14) | (0x7 << 4) | (0xF << 8);
+  if (computes) __builtin_amdgcn_s_waitcnt(kWaitA0);
+  else if (copies_w) __builtin_amdgcn_s_waitcnt(kWaitW0);
+  __builtin_amdgcn_s_barrier();
+  Frags fa, fb;
+  if (computes) {
+    issue_a(2, a_s[2]);
+    read_frags(fa, a_s[0], w_s[0]);
+  } else if (copies_w) {
+    issue_w(WS - 1, w_s[WS - 1]);
+  }
+  constexpr int kBase = WS % kMidAStages == 0 ? WS : kMidAStages * WS;
+  constexpr int kPeriod = kBase % 2 == 0 ? kBase : 2 * kBase;   // stage and register-buffer assignment repeat
+  // Registers with a read in flight must never be moved: the round's body is straight-line code (the loop is left
+  // with a break, not skipped round by round), the last round requests nothing, and the one pending buffer that
+  // crosses the loop's back edge is waited for first.
+  for (int base = 0; base < n_chunks; base += kPeriod) {
+#pragma unroll
+    for (int u = 0; u < kPeriod; ++u) {
+      const int chunk = base + u;
+      if (chunk >= n_chunks) break;
+      Frags& cur = u % 2 == 0 ? fa : fb;
+      Frags& nxt = u % 2 == 0 ? fb : fa;
+      if (computes) {
+        wait_frags(cur);                                    // fragments of this chunk are in registers
+        __builtin_amdgcn_s_waitcnt(kWaitA);                 // own copies of chunk + 1 have landed
+      } else if (copies_w) {
+        __builtin_amdgcn_s_waitcnt(kWaitW);
+      }
+      // A bare s_barrier: __syncthreads() would add a wait for every outstanding copy and undo the pipelining.
+      __builtin_amdgcn_s_barrier();
+      if (computes) {
+        issue_a(chunk + 3, a_s[u % kMidAStages]);
+        if (chunk + 1 < n_chunks) read_frags(nxt, a_s[(u + 1) % kMidAStages], w_s[(u + 1) % WS]);
+        multiply(cur);
+        if (u == kPeriod - 1 && chunk + 1 < n_chunks) wait_frags(nxt);
+      } else if (copies_w) {
+        issue_w(chunk + WS, w_s[u % WS]);
+      }
+    }
+  }
+  // channel scales of this lane's four outputs: requested here, their latency passes under the sum of the K units
+  f16 sc[4] = {(f16)0, (f16)0, (f16)0, (f16)0};
+  if (computes && ku == 0) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int gn = n_begin + nt * 16 + kg * 4 + e;
       sc[e] = scales[gn < n_end ? gn : n_end - 1];
     }
   }
-  // prologue: activations of chunks 0, 1; weights of chunks 0 .. 3
-  if (computes) {
-    issue_a(0, a_s0);
-    issue_a(1, a_s1);
-  } else if (copies_w) {
-#pragma unroll
-    for (int i = 0; i < WS - 1; ++i) issue_w(i, w_s[i]);
-  }
-#pragma unroll
-  for (int e = 0; e < 4; ++e) asm volatile("" : "+v"(sc[e]));
-  constexpr int kPeriod = WS % kMidAStages == 0 ? WS : kMidAStages * WS;   // the stage assignment repeats
-  for (int base = 0; base < n_chunks; base += kPeriod) {
-#pragma unroll
-    for (int u = 0; u < kPeriod; ++u) {
-      if (base + u < n_chunks) {
-        const int chunk = base + u;
-        if (computes) __builtin_amdgcn_s_waitcnt(kWaitA);
-        else if (copies_w) __builtin_amdgcn_s_waitcnt(kWaitW);
-        // chunk landed for every wave; the stages of chunk-1 are free. A bare s_barrier: __syncthreads() would add
-        // a wait for every outstanding copy and undo the pipelining.
-        __builtin_amdgcn_s_barrier();
-        if (computes) {
-          issue_a(chunk + 2, a_stage((u + 2) % kMidAStages));
-          multiply(a_stage(u % kMidAStages), w_stage(u % WS));
-        } else if (copies_w) {
-          issue_w(chunk + WS - 1, w_stage((u + WS - 1) % WS));
-        }
-      }
-    }
-  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // trailing copies land before the stages are reused
   __syncthreads();
 
-  // the four K quarters of a tile are summed through the first two activation stages (quarters 1 and 2 in the
-  // first, quarter 3 in the second: MB KiB per wave), in the fixed order 0 + 1 + 2 + 3
-  float* red0 = reinterpret_cast<float*>(a_s0);
-  float* red1 = reinterpret_cast<float*>(a_s1);
-  static_assert(2 * 3 * MB * 1024 <= MB * 16 * kMidKC * 2, "two quarters of partial tiles fit one activation stage");
-  if (computes && kq > 0) {
-    float* dst = kq < 3 ? red0 + ((kq - 1) * 3 + nt) * MB * 256 : red1 + nt * MB * 256;
+  // the K units of a tile are summed through the activation stages (RB KiB per wave), in the fixed order 0 + 1 + ...
+  float* red = reinterpret_cast<float*>(&a_s[0][0]);
+  static_assert((KU - 1) * 3 * MB * 1024 <= kMidAStages * MB * 16 * KC * 2, "the partial tiles fit the activation stages");
+  if (computes && ku > 0) {
+    float* dst = red + (((ku - 1) * 3 + nt) * RG + rg) * RB * 256;
 #pragma unroll
-    for (int rb = 0; rb < MB; ++rb) *reinterpret_cast<f32x4*>(dst + (rb * 64 + lane) * 4) = acc[rb];
+    for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(dst + (rb * 64 + lane) * 4) = acc[rb];
   }
-  __syncthreads();
-  if (computes && kq == 0) {
+  if constexpr (KU > 1) __syncthreads();
+  if (computes && ku == 0) {
     const int gn = n_begin + nt * 16 + kg * 4;
 #pragma unroll
-    for (int rb = 0; rb < MB; ++rb) {
+    for (int rb = 0; rb < RB; ++rb) {
       f32x4 sum = acc[rb];
-      sum += *reinterpret_cast<const f32x4*>(red0 + (nt * MB * 64 + rb * 64 + lane) * 4);
-      sum += *reinterpret_cast<const f32x4*>(red0 + ((3 + nt) * MB * 64 + rb * 64 + lane) * 4);
-      sum += *reinterpret_cast<const f32x4*>(red1 + (nt * MB * 64 + rb * 64 + lane) * 4);
-      const int gm = rb * 16 + r16;
+#pragma unroll
+      for (int q = 1; q < KU; ++q)
+        sum += *reinterpret_cast<const f32x4*>(red + ((((q - 1) * 3 + nt) * RG + rg) * RB * 64 + rb * 64 + lane) * 4);
+      const int gm = (rg * RB + rb) * 16 + r16;
       if (gm < M) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -651,7 +674,9 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
 #undef HEXMI_GEMV
     return launch_status();
   }
-  if (M <= 16 && K % (kPWaves * 64) == 0 && K / (kPWaves * 64) <= kPSteps) {
+  // up to 8 rows; 9 .. 16 rows stream faster through the chunked kernel below (12.6 against 13.8 us at M = 16,
+  // N = 11008, K = 4096 with the weights from HBM; 12.5 against 12.1 at M = 4)
+  if (M <= 8 && K % (kPWaves * 64) == 0 && K / (kPWaves * 64) <= kPSteps) {
     const int cus = hexmi_num_cus();
     if (cus <= 0) return HEXMI_ELAUNCH;
     int chan_per_wg = (int)((N + cus - 1) / cus);
@@ -661,7 +686,7 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
                        chan_per_wg);
     return launch_status();
   }
-  if (M <= 64 && K % kMidKC == 0 && N <= 0x7fffffff) {
+  if (M <= kMidMaxM && K % 256 == 0 && N <= 0x7fffffff) {
     const int cus = hexmi_num_cus();
     if (cus <= 0) return HEXMI_ELAUNCH;
     int chan_per_wg = (int)((N + cus - 1) / cus);
@@ -670,7 +695,8 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     const int grid = (int)((N + chan_per_wg - 1) / chan_per_wg);
 #define HEXMI_MID(MB) \
   hipLaunchKernelGGL(w8a16_mid_kernel<MB>, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg)
-    if (M <= 16) HEXMI_MID(1); else if (M <= 32) HEXMI_MID(2); else if (M <= 48) HEXMI_MID(3); else HEXMI_MID(4);
+    if (M <= 16) HEXMI_MID(1); else if (M <= 32) HEXMI_MID(2); else if (M <= 48) HEXMI_MID(3); else if (M <= 64) HEXMI_MID(4);
+    else HEXMI_MID(8);
 #undef HEXMI_MID
     return launch_status();
   }
