@@ -183,7 +183,7 @@ int hexmi_pack_w8(int64_t N, int64_t K, const int8_t *W, int8_t *Wp,
 /* hexmi_gemm_w8a16 on weights packed by hexmi_pack_w8: every weight load of a
  * wave is a contiguous KiB already in MFMA fragment order. K % 1024 == 0 and
  * K <= 4096. Meant for M <= 16 (decode batches); larger M runs 16 rows per
- * launch. For 3 <= M <= 16 hexmi_gemm_w8a16 runs the same kernel and the results
+ * launch. For 3 <= M <= 8 hexmi_gemm_w8a16 runs the same kernel and the results
  * agree bit for bit; for other M its kernels sum in another order and the
  * results agree to one fp16 unit in the last place. */
 int hexmi_gemm_w8a16_packed(int64_t M, int64_t N, int64_t K, const void *A,
