@@ -488,18 +488,22 @@ class MfmaPeak(Workload):
 
     def __init__(self, shape, dtype_name, data, waves=2):
         self.shape, self.dtype, self.data, self.waves = shape, dtype_name, data, waves
-        self.name = "mfma_peak_%s_%s_%s" % ("32x32x16" if shape == 0 else "16x16x32", dtype_name, data)
-        self.desc = ("v_mfma_f32_%s_%s only, %d waves per SIMD, operands %s, accumulators in registers"
-                     % ("32x32x16" if shape == 0 else "16x16x32", dtype_name, waves,
-                        "all zero" if data == "zeros" else "U(-1,1)"))
-        self.iters = 20000 if shape == 0 else 20000
+        tag = ("32x32x16", "16x16x32", "16x16x32_tile8x8")[shape]
+        if shape == 2:
+            self.waves = waves = 1
+        self.name = "mfma_peak_%s_%s_%s" % (tag, dtype_name, data)
+        self.desc = ("v_mfma_f32_%s_%s only, %d waves per SIMD, operands %s, accumulators in registers%s"
+                     % (tag[:8], dtype_name, waves, "all zero" if data == "zeros" else "U(-1,1)",
+                        ", 8 A x 8 B fragments walked as a GEMM tile (one operand changes per instruction)" if shape == 2 else ""))
+        self.iters = 5000 if shape == 2 else 20000
 
     def setup(self, torch, hexmi):
         from hexmi import _lib
         self.lib, self._lib = _lib.lib(), _lib
         dt = torch.float16 if self.dtype == "f16" else torch.bfloat16
         g = torch.Generator().manual_seed(0)
-        ops = torch.zeros(1024) if self.data == "zeros" else 2 * torch.rand(1024, generator=g) - 1
+        n_ops = 8192 if self.shape == 2 else 1024
+        ops = torch.zeros(n_ops) if self.data == "zeros" else 2 * torch.rand(n_ops, generator=g) - 1
         self.ops = ops.to(dt).cuda()
         self.sink = torch.empty(self.lib.hexmi_num_cus() * 256 * self.waves, device="cuda")
         self.work = int(self.lib.hexmi_mfma_peak_flops(self.shape, self.waves, self.iters))
@@ -537,7 +541,8 @@ def make_workloads():
 
 
 def peak_workloads():
-    return [MfmaPeak(shape, dt, data) for dt in ("f16", "bf16") for shape in (0, 1) for data in ("zeros", "uniform")]
+    return ([MfmaPeak(shape, dt, data) for dt in ("f16", "bf16") for shape in (0, 1) for data in ("zeros", "uniform")]
+            + [MfmaPeak(2, dt, "uniform") for dt in ("f16", "bf16")])
 
 
 ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "softmax_f32_4096x1024",

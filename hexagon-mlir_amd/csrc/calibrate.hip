@@ -72,6 +72,40 @@ void mfma_peak_kernel(const T* __restrict__ operands, int iters, float* __restri
 }
 
 
+// The same stream with the operands of a GEMM tile: 8 x 8 accumulator tiles of 16x16x32 per wave (one wave per SIMD,
+// 256 accumulator registers), accumulator (i, j) fed by A fragment i and B fragment j, walked row by row, so one
+// operand changes with every instruction and the other with every eighth, as in gemm.hip. operands: 16 KiB, A
+// fragment i of lane l at byte 1024*i + 16*l, B fragment j at byte 8192 + 1024*j + 16*l.
+template <typename T>
+__global__ __launch_bounds__(256)
+void mfma_tile_kernel(const T* __restrict__ operands, int iters, float* __restrict__ sink) {
+  typedef typename Peak<T>::Frag Frag;
+  const int lane = threadIdx.x % kWave;
+  Frag a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = *reinterpret_cast<const Frag*>(operands + (i * 64 + lane) * 8);
+    b[i] = *reinterpret_cast<const Frag*>(operands + 4096 + (i * 64 + lane) * 8);
+  }
+  f32x4v acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i][j] = Peak<T>::small(b[j], a[i], acc[i][j]);
+  }
+  float total = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) total += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+  sink[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = total;
+}
+
 // ---- issue slots --------------------------------------------------------------------------------------------
 // How much vector work fits under a wave's own MFMAs: per MFMA (independent accumulators, zero operands, so the chip
 // holds its top clock) VPM vector instructions of one kind follow in the same instruction stream. A SIMD issues one
@@ -179,15 +213,18 @@ using namespace hexmi;
 
 extern "C" double hexmi_mfma_peak_flops(int shape, int waves_per_simd, int64_t iters) {
   const int cus = hexmi_num_cus();
-  if (cus <= 0 || (shape != 0 && shape != 1) || waves_per_simd < 1 || waves_per_simd > 2 || iters < 0) return 0.0;
+  if (cus <= 0 || shape < 0 || shape > 2 || waves_per_simd < 1 || waves_per_simd > (shape == 2 ? 1 : 2) || iters < 0)
+    return 0.0;
   const double per_wave_iter = shape == 0 ? (double)kUnroll * kBigChains * (2.0 * 32 * 32 * 16)
-                                          : (double)kUnroll * kSmallChains * (2.0 * 16 * 16 * 32);
+                               : shape == 1 ? (double)kUnroll * kSmallChains * (2.0 * 16 * 16 * 32)
+                                            : 64.0 * (2.0 * 16 * 16 * 32);
   return per_wave_iter * (double)iters * 4.0 * waves_per_simd * cus;
 }
 
 extern "C" int hexmi_mfma_peak(int shape, int dtype, const void* operands, int64_t iters, int waves_per_simd,
                                float* sink, hexmi_stream_t stream) {
-  if ((shape != 0 && shape != 1) || waves_per_simd < 1 || waves_per_simd > 2 || iters < 0 || iters > 0x7fffffff)
+  if (shape < 0 || shape > 2 || waves_per_simd < 1 || waves_per_simd > (shape == 2 ? 1 : 2) || iters < 0 ||
+      iters > 0x7fffffff)
     return HEXMI_EINVAL;
   if (!operands || !sink || !aligned_to(operands, 16)) return HEXMI_EINVAL;
   const int cus = hexmi_num_cus();
@@ -195,6 +232,15 @@ extern "C" int hexmi_mfma_peak(int shape, int dtype, const void* operands, int64
   hipStream_t st = as_stream(stream);
   const dim3 grid((unsigned)cus), block(256u * waves_per_simd);
   begin_call();
+  if (shape == 2) {
+    if (dtype == HEXMI_F16)
+      hipLaunchKernelGGL(mfma_tile_kernel<f16>, grid, block, 0, st, static_cast<const f16*>(operands), (int)iters, sink);
+    else if (dtype == HEXMI_BF16)
+      hipLaunchKernelGGL(mfma_tile_kernel<bf16>, grid, block, 0, st, static_cast<const bf16*>(operands), (int)iters, sink);
+    else
+      return HEXMI_ENOTSUP;
+    return launch_status();
+  }
 #define HEXMI_PEAK(T, BIG) \
   hipLaunchKernelGGL((mfma_peak_kernel<T, BIG>), grid, block, 0, st, static_cast<const T*>(operands), (int)iters, sink)
   if (dtype == HEXMI_F16) { if (shape == 0) HEXMI_PEAK(f16, true); else HEXMI_PEAK(f16, false); }

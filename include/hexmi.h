@@ -329,6 +329,12 @@ int hexmi_rope(const void *x, void *y, int64_t batch, int64_t seq,
  * byte 16*l and its B fragment at byte 1024 + 16*l, every wave the same);
  * waves_per_simd: 1 or 2; one workgroup per compute unit; sink: one float per
  * thread (hexmi_num_cus() * 256 * waves_per_simd), written once at the end.
+ * shape 2 = v_mfma_f32_16x16x32 with the operand traffic of a GEMM tile: 8 x 8
+ * accumulator tiles per wave, tile (i, j) fed by A fragment i and B fragment j
+ * (operands: 16 KiB, A fragment i of lane l at byte 1024*i + 16*l, B fragment j
+ * at byte 8192 + 1024*j + 16*l), one operand changing with every instruction;
+ * waves_per_simd 1 only. The data-dependent rate is lower than with the same
+ * two fragments throughout.
  * hexmi_mfma_peak_flops is the FLOP count of such a launch on this device. */
 double hexmi_mfma_peak_flops(int shape, int waves_per_simd, int64_t iters);
 int hexmi_mfma_peak(int shape, int dtype, const void *operands, int64_t iters,
