@@ -1,6 +1,7 @@
-"""Check the compiled GEMM kernels for reads of an accumulator too soon after an inline-assembly MFMA.
+"""Check the compiled kernels for reads of an accumulator too soon after an inline-assembly MFMA.
 
-    python hexagon-mlir_amd/check_mfma_hazards.py            # compiles csrc/gemm.hip to gfx950 assembly and scans it
+    python hexagon-mlir_amd/check_mfma_hazards.py            # compiles csrc/gemm.hip and csrc/calibrate.hip to gfx950
+                                                             # assembly and scans it
 
 The 16x16x32 MFMAs of the paired-slab GEMM are `asm volatile` (the accumulator is tied to the destination), so the
 compiler's hazard recogniser does not see them and inserts no wait states between such an MFMA and a later read of
@@ -57,15 +58,19 @@ def scan(asm_path):
     return bad
 
 
+SOURCES = ("gemm.hip", "calibrate.hip")      # the files with MFMAs written as inline assembly
+
+
 def main():
-    src = os.path.join(_build.CSRC, "gemm.hip")
+    bad = {}
     with tempfile.TemporaryDirectory() as tmp:
-        out = os.path.join(tmp, "gemm.s")
-        cmd = [_build.HIPCC] + _build.FLAGS + ["--cuda-device-only", "-S", src, "-o", out]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            sys.exit("hipcc failed:\n" + r.stderr)
-        bad = scan(out)
+        for name in SOURCES:
+            out = os.path.join(tmp, name[:-4] + ".s")
+            cmd = [_build.HIPCC] + _build.FLAGS + ["--cuda-device-only", "-S", os.path.join(_build.CSRC, name), "-o", out]
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                sys.exit("hipcc failed:\n" + r.stderr)
+            bad.update(scan(out))
     for k, v in bad.items():
         print("%s: %d accumulator reads too close to an assembly MFMA, first: %d wait states before `%s`"
               % (k, len(v), v[0][0], v[0][1]))
