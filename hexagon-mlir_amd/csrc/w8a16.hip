@@ -242,6 +242,7 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
 // through LDS after the K loop, in a fixed order.
 // With every CU fetching all of A the kernel moves M * 8 KiB per CU through L2: 29 us at M = 128 (the 128 x 128
 // tile kernel, 86 tiles: 34), but 47 us at M = 256 with 64-k chunks (tile kernel: 37), so it stops at 128 rows.
+constexpr int kMidWeightPolicy = 2;                         // nt: weights are read once (12.4 against 13.0 us at M = 16)
 constexpr int kMidCh = 48;                                  // channels per workgroup (three tiles of 16)
 constexpr int kMidAStages = 3, kMidWStages = 5;
 constexpr int kMidCompute = 12;                             // compute waves: three channel tiles x four (unit, group)
@@ -324,7 +325,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
 #pragma unroll
     for (int j = 0; j < WSL; ++j)
       __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * KC),
-                                       HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, 0);
+                                       HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, kMidWeightPolicy);
   };
 
   // ---- fragment side: compute wave w owns channel tile nt = w % 3, K unit ku and row-block group rg
