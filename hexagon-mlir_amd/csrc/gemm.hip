@@ -902,7 +902,9 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
         const int row = r0 + lane / CP, c = lane % CP;
         const u32x4 v = *reinterpret_cast<const u32x4*>(cs + row * PITCH + ((c ^ swz(row)) * kChunk));
         const int grow = m0 + wm * TM * 16 + row, gcol = n0 + wn * TN * 16 + c * kChunk;
-        if (grow < M && gcol < N) *reinterpret_cast<u32x4*>(C + (int64_t)grow * ldc + gcol) = v;
+        // non-temporal: C is not read again, and the operand panels other tiles still need stay in the caches
+        // (bf16 8192^3: 0.617 -> 0.632 of peak, A/B on one box; 4096^3 unchanged)
+        if (grow < M && gcol < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)grow * ldc + gcol));
       }
       return;
     }
