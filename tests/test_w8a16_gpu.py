@@ -68,8 +68,8 @@ def test_scale_selection_and_indexing(hexmi, oracle):
     assert c1[1, 37] == w[37, 7] and c1[:, :37].abs().sum() == 0 and c1[:, 38:].abs().sum() == 0
 
 
-@pytest.mark.parametrize("M", [1, 2, 15, 16, 17, 33, 64, 100])
-@pytest.mark.parametrize("N,K", [(96, 512), (1000, 256), (16, 64), (11, 4096)])
+@pytest.mark.parametrize("M", [1, 2, 15, 16, 17, 33, 64, 100, 129, 200, 256])
+@pytest.mark.parametrize("N,K", [(96, 512), (1000, 256), (16, 64), (11, 4096), (200, 7936)])
 def test_w8a16_parity(hexmi, oracle, M, N, K):
     a, w, s = _inputs(M, N, K, seed=3)
     got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
