@@ -42,7 +42,7 @@ struct MaskTileLoader {
     const char* base = reinterpret_cast<const char*>(mask_wg);
     int key = key0 + (col0 ^ ((j & 1) * 32));
     key = key + 8 <= Skv ? key : Skv - 8;
-    copy_to_lds(base, (rowoff[j] + key) * (int)sizeof(T), lds + j * 512);
+    copy_to_lds<T, 2>(base, (rowoff[j] + key) * (int)sizeof(T), lds + j * 512);      // the mask is read once
   }
   __device__ __forceinline__ void issue(const T* __restrict__ mask_wg, int key0, int Skv, T* lds) const {
 #pragma unroll

@@ -144,12 +144,13 @@ int fill_zero_2d(void* C, int64_t rows, int64_t cols, int64_t ld, int elem_size,
 // registers, built by scalar arithmetic) plus a per-lane 32-bit byte offset, and the LDS destination (lds + lane*16
 // bytes) is a scalar, so a copy costs no vector arithmetic. voff must stay below 2^31; the descriptor's own range
 // check is left wide open, callers clamp what must not be read.
-template <typename T>
+// POLICY: the cache-policy bits of the load (0 = default, 2 = non-temporal: data that is read once).
+template <typename T, int POLICY = 0>
 __device__ __forceinline__ void copy_to_lds(const char* base, int voff, T* lds) {
 #if defined(__HIP_DEVICE_COMPILE__)        // the descriptor type exists in the device pass only
   const __amdgpu_buffer_rsrc_t rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, 0x7fffffff, 0x00020000);
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(lds), 16, voff, 0, 0, 0);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(lds), 16, voff, 0, 0, POLICY);
 #endif
 }
 
