@@ -106,3 +106,11 @@ def test_block_sum_workspace_query_needs_no_device():
     assert lib.hexmi_block_sum_workspace(0, 16, _lib.F32) == 0
     assert lib.hexmi_block_sum_ws(None, None, -1, 4, _lib.F32, None, 0, None) == _lib.EINVAL
     assert "capacity" in _lib.strerror(_lib.ETOOBIG)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stderr + r.stdout)
