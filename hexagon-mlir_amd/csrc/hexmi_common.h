@@ -98,19 +98,17 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // ---- int8 -> fp16 (weight-only quantisation) --------------------------------
-// int8 -> fp16 is exact: byte b = w ^ 0x80 placed in the low mantissa bits of 0x6400 is the fp16 number
-// 1024 + b, and subtracting 1152 leaves w.
-// 4 int8 (one dword) -> 4 fp16 in two dwords, exact.
+// 4 int8 (one dword) -> 4 fp16 in two dwords, exact (|w| <= 128 has at most eight significant bits): one
+// v_cvt_f16_i16 per weight, its source the sign-extended byte picked by the instruction's operand selector and its
+// destination one half of the result register. (One instruction fewer per dword than building 1024 + (w ^ 0x80) with
+// byte permutes and subtracting 1152 in packed fp16: 0.157 -> 0.164 of the HBM figure at M = 256, +1 % at M = 1.)
 __device__ __forceinline__ void cvt4(uint32_t w, uint32_t& lo, uint32_t& hi) {
-  const uint32_t b = w ^ 0x80808080u;                         // bytes now w + 128 in [1, 255]
-  // v_perm_b32 byte selectors: 0..3 pick bytes of the second source, 4..7 of the first.
-  uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, b, 0x07010700u);   // {0x64, b1, 0x64, b0}
-  uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, b, 0x07030702u);   // {0x64, b3, 0x64, b2}
-  const f16x2 bias = {(f16)1152.0f, (f16)1152.0f};
-  f16x2 h0 = *reinterpret_cast<f16x2*>(&p0) - bias;
-  f16x2 h1 = *reinterpret_cast<f16x2*>(&p1) - bias;
-  lo = *reinterpret_cast<uint32_t*>(&h0);
-  hi = *reinterpret_cast<uint32_t*>(&h1);
+  asm("v_cvt_f16_i16_sdwa %0, sext(%2) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0\n\t"
+      "v_cvt_f16_i16_sdwa %0, sext(%2) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1\n\t"
+      "v_cvt_f16_i16_sdwa %1, sext(%2) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_2\n\t"
+      "v_cvt_f16_i16_sdwa %1, sext(%2) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3"
+      : "=&v"(lo), "=&v"(hi)
+      : "v"(w));
 }
 
 // 16 int8 -> two 8-element fp16 fragments (bytes 0..7 and 8..15).

@@ -4,8 +4,7 @@
 // The weight matrix is the only large operand (N*K bytes) and every weight is used once per 16 activation rows,
 // so weights never touch LDS: each lane fetches 16 consecutive int8 of one output channel straight from HBM
 // (16-byte loads, a 16-channel tile reads 64 contiguous bytes per channel per instruction), converts them to
-// fp16 in registers and feeds two MFMAs. int8 -> fp16 is exact: byte b = w ^ 0x80 placed in the low mantissa
-// bits of 0x6400 is the fp16 number 1024 + b, and subtracting 1152 leaves w.
+// fp16 in registers (exact: one v_cvt_f16_i16 per weight on the sign-extended byte) and feeds two MFMAs.
 //
 // The per-channel scale multiplies the finished fp32 sum (it is constant over k), which differs from
 // "dequantise, then multiply" only by fp32 rounding; hexmi_dequant_w8 exposes the element-wise dequantisation.
@@ -233,10 +232,10 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
 // waits with its own count and the workgroup barrier publishes both.
 // Compute wave w < 12 owns channel tile w % 3 and, of every chunk, one unit of 64 k for one group of row blocks
 // (four K units and all row blocks at KC = 256; two units and two groups of four row blocks at KC = 128). It converts
-// its 16 x 64 int8 weights to fp16 once per chunk (20 vector instructions) and multiplies them into its RB
+// its 16 x 64 int8 weights to fp16 once per chunk (16 vector instructions) and multiplies them into its RB
 // accumulators (2 * RB MFMAs). A SIMD issues one instruction at a time and a 16x16x32 MFMA hides only two vector
 // instructions, so the conversions per MFMA set the pace: with one 16 x 16 tile per wave (every row-block wave
-// converting the same weights, 10 instructions per MFMA) the kernel took 18.4 us at M = 64, N = 11008, K = 4096,
+// converting the same weights, 8 to 10 instructions per MFMA) the kernel took 18.4 us at M = 64, N = 11008, K = 4096,
 // this way 15.0 (22.6 -> 21.1 with the weights coming from HBM). Fragments are read back from LDS in 16-byte chunks
 // permuted inside their row through the copies' source addresses (conflict-free). The K units of a tile are summed
 // through LDS after the K loop, in a fixed order.
