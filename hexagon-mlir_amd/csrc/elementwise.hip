@@ -191,10 +191,13 @@ void block_sum_kernel(const T* __restrict__ x, TOut* __restrict__ out, int64_t b
 //   y[2i] = x[2i] cos - x[2i+1] sin,   y[2i+1] = x[2i] sin + x[2i+1] cos.
 // A workgroup owns one sequence position; a thread owns one 16-byte chunk of the feature vector, computes the
 // sines and cosines of its pairs once (in double: the angle m*freq is accurate to fp32 for any m) and walks all
-// (batch, head) rows with them.
+// (batch, head) rows with them. The frequencies of a thread's pairs are a geometric sequence: one double-precision
+// exp2 for the first, then a multiplication by pair_ratio = theta^(-2/feat) for each further pair (the set-up of a
+// thread, four double exp2 and four sine / cosine pairs, was more vector work than its eight rows).
 template <typename T>
 __global__ __launch_bounds__(256)
-void rope_kernel(const T* __restrict__ x, T* __restrict__ y, int batch, int seq, int heads, int feat, double log2_theta) {
+void rope_kernel(const T* __restrict__ x, T* __restrict__ y, int batch, int seq, int heads, int feat, double log2_theta,
+                 double pair_ratio) {
   constexpr int N = Chunk<T>::N;                     // elements per chunk (even)
   const int chunks = feat / N;                       // chunks per feature vector (feat % N == 0 on this path)
   const int rows_per_pass = 256 / chunks;            // (batch, head) rows handled side by side
@@ -203,10 +206,11 @@ void rope_kernel(const T* __restrict__ x, T* __restrict__ y, int batch, int seq,
   const int r0 = threadIdx.x / chunks;
   if (r0 >= rows_per_pass) return;
   float cs[N / 2], sn[N / 2];
+  // even feature index i2 = ch * N + 2 * p (the reference's `steps`): freq = theta^(-i2 / feat)
+  double freq = exp2(-((double)(ch * N) / (double)feat) * log2_theta);
 #pragma unroll
   for (int p = 0; p < N / 2; ++p) {
-    const int i2 = ch * N + 2 * p;                   // even feature index = the reference's `steps`
-    const double freq = exp2(-((double)i2 / (double)feat) * log2_theta);
+    if (p > 0) freq *= pair_ratio;
     // the angle m*freq in double, reduced to one turn in double (so it is accurate to fp32 for any m), then the
     // fp32 sine and cosine of the reduced angle: a double-precision sincos per pair costs as much as the kernel's
     // whole memory time
@@ -218,11 +222,18 @@ void rope_kernel(const T* __restrict__ x, T* __restrict__ y, int batch, int seq,
     cs[p] = c;
     sn[p] = s;
   }
-  const int64_t rows = (int64_t)batch * heads;
-  // one row in flight per thread: with the next row's load issued ahead the kernel measured 5 % slower
-  for (int64_t r = r0 + (int64_t)blockIdx.y * rows_per_pass; r < rows; r += (int64_t)rows_per_pass * gridDim.y) {
-    const int64_t b = r / heads, h = r % heads;
-    const int64_t off = (((b * seq + m) * heads) + h) * feat + ch * N;
+  const int rows = batch * heads;                    // < 2^31: checked by the launcher
+  // one row in flight per thread: with the next row's load issued ahead the kernel measured 5 % slower.
+  // (batch, head) of the row advance with it: a division per row was a third of the loop's instructions
+  const int step = rows_per_pass * (int)gridDim.y, step_b = step / heads, step_h = step % heads;
+  int r = r0 + (int)blockIdx.y * rows_per_pass;
+  int b = r / heads, h = r % heads;
+  for (; r < rows; r += step, b += step_b, h += step_h) {
+    if (h >= heads) {
+      h -= heads;
+      ++b;
+    }
+    const int64_t off = ((((int64_t)b * seq + m) * heads) + h) * feat + ch * N;
     const Chunk<T> in = load_chunk(x + off);
     Chunk<T> out;
 #pragma unroll
@@ -348,14 +359,14 @@ int launch_rope(const void* xv, void* yv, int64_t batch, int64_t seq, int64_t he
   T* y = static_cast<T*>(yv);
   constexpr int N = 16 / sizeof(T);
   const double log2_theta = log2(theta);
-  if (aligned_to(x, 16) && aligned_to(y, 16) && feat % N == 0 && feat / N <= 256) {
+  if (aligned_to(x, 16) && aligned_to(y, 16) && feat % N == 0 && feat / N <= 256 && batch * heads < 0x40000000) {
     // enough workgroups to fill the chip when the sequence is short: split the (batch, head) rows over grid.y
     const int64_t passes = (batch * heads + 256 / (feat / N) - 1) / (256 / (feat / N));
     int64_t split = (2048 + seq - 1) / seq;
     split = split < passes ? split : passes;
     split = split < 65535 ? split : 65535;
     hipLaunchKernelGGL((rope_kernel<T>), dim3((unsigned)seq, (unsigned)split), dim3(256), 0, s, x, y, (int)batch,
-                       (int)seq, (int)heads, (int)feat, log2_theta);
+                       (int)seq, (int)heads, (int)feat, log2_theta, exp2(-2.0 * log2_theta / (double)feat));
   } else {
     const int64_t pairs = batch * seq * heads * (feat / 2);
     const int64_t blocks = (pairs + 255) / 256;
