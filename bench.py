@@ -18,7 +18,8 @@ HBM-bound entries also carry a `hot` figure (one buffer set, served by the 256 M
 the rotated one is the HBM claim. `--workload mfma_peak` times a registers-only MFMA stream (zeros and U(-1,1)
 operands, both instruction shapes, about a second each): the data-dependent ceiling of the matrix cores on this box.
 `--workload issue_slots` (vector instructions that fit between a wave's MFMAs) and `--workload lds_patterns` (cycles
-per LDS read for the GEMM's fragment address patterns) are two more calibrations of the same kind.
+per LDS read for the GEMM's fragment address patterns) are two more calibrations of the same kind. `--operands zeros` runs a GEMM or attention workload on all-zero inputs
+(same instructions, same traffic): against the random-operand time it shows what the data costs in power.
 """
 import argparse
 import json
@@ -171,6 +172,18 @@ class LayerNorm(Norms):
     desc = "LayerNorm fp16 [8192,4096]"
 
 
+# --operands zeros: the matrix-core workloads (GEMM, attention) run on all-zero inputs, through the same
+# instructions and the same memory traffic. Not a throughput claim: the difference to the random-operand time is what
+# the data costs in power, and the line says so in its "data" field.
+ZERO_OPERANDS = False
+
+
+def _zero_operands(buffers, names):
+    if ZERO_OPERANDS:
+        for n in names:
+            buffers[n].zero_()
+
+
 class Gemm(Workload):
     bound, kernel = "mfma", "gemm_kernel_k64"
 
@@ -191,6 +204,7 @@ class Gemm(Workload):
         self.work = gemm_flops(self.size, self.size, self.size)
         self.sets = _sets(torch, self.host, 0, rotate=False)
         self.sets[0]["out"] = torch.empty(self.size, self.size, dtype=dt, device="cuda")
+        _zero_operands(self.sets[0], ("a", "b"))
         if self.packed:
             self.sets[0]["b"] = hexmi.pack_weight(self.sets[0]["b"])
 
@@ -268,6 +282,7 @@ class Attention(Workload):
         t = {k: v for k, v in self.host.items() if k != "sm_scale"}
         self.sets = _sets(torch, t, 0, rotate=False)
         self.sets[0]["out"] = torch.empty_like(self.sets[0]["q"])
+        _zero_operands(self.sets[0], ("q", "k", "v"))
 
     def step(self, i):
         s = self.sets[0]
@@ -804,7 +819,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time direct launches instead of a HIP graph replay")
     ap.add_argument("--only", default="", help="comma-separated suite entries to measure (default: all)")
+    ap.add_argument("--operands", choices=("random", "zeros"), default="random",
+                    help="zeros: GEMM / attention workloads on all-zero inputs (what the data costs in power)")
     args = ap.parse_args()
+    global ZERO_OPERANDS
+    ZERO_OPERANDS = args.operands == "zeros"
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
@@ -837,7 +856,8 @@ def main():
         "value": roof["achieved"], "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(m["ms"], 5), "ms_per_step_min": round(m["min"], 5), "ms_per_step_max": round(m["max"], 5),
         "timed_replays": m["replays"], "wall_ms_per_step": round(m["wall"], 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": primary.dtype, "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": primary.dtype,
+        "data": "synthetic, ALL-ZERO operands (power calibration, not a throughput claim)" if ZERO_OPERANDS else "synthetic",
         "config": {"workload": primary.name, "description": primary.desc,
                    "buffers": "%d rotated sets" % len(primary.sets),
                    "launch": "hip graph replay" if m["graph"] else "direct",
