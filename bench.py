@@ -20,6 +20,8 @@ operands, both instruction shapes, about a second each): the data-dependent ceil
 `--workload issue_slots` (vector instructions that fit between a wave's MFMAs) and `--workload lds_patterns` (cycles
 per LDS read for the GEMM's fragment address patterns) are two more calibrations of the same kind. `--operands zeros` runs a GEMM or attention workload on all-zero inputs
 (same instructions, same traffic): against the random-operand time it shows what the data costs in power.
+`--workload vendor` times the GEMM and attention configurations through this library and through torch.matmul /
+F.scaled_dot_product_attention on the same box (a comparison; hexmi calls neither).
 """
 import argparse
 import json
@@ -782,6 +784,54 @@ def run_issue_slots(torch, hexmi, args):
                                        rows, "issue_slots")), flush=True)
 
 
+class _Lambda:
+    """A step function with the attributes measure() looks at."""
+    sets = None
+
+    def __init__(self, fn):
+        self.step = lambda i: fn()
+
+
+def run_vendor(torch, hexmi, args):
+    """--workload vendor: the GEMM and causal-attention configurations through this library and through the
+    libraries PyTorch-ROCm ships (torch.matmul -> hipBLASLt / rocBLAS, F.scaled_dot_product_attention), same box, same
+    buffers, same HIP-graph protocol, alternating. A comparison, not a product path: nothing in hexmi calls them."""
+    import torch.nn.functional as F
+    from hexmi.workloads import gemm_inputs, gemm_flops, attention_inputs, attention_flops
+    rows = []
+
+    def pair(name, flops, ours, theirs, their_name, steps):
+        for who, fn in (("hexmi", ours), (their_name, theirs), ("hexmi", ours), (their_name, theirs)):
+            m = measure(torch, _Lambda(fn), steps, args.warmup, not args.no_graph)
+            rows.append({"config": name, "library": who, "ms": round(m["ms"], 5), "ms_min": round(m["min"], 5),
+                         "tflops": round(flops / (m["ms"] * 1e-3) / 1e12, 1),
+                         "frac": round(flops / (m["ms"] * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+            print("# %-34s %-28s %.4f ms  frac %.3f" % (name, who, rows[-1]["ms"], rows[-1]["frac"]), file=sys.stderr)
+
+    for size, dt, tag in ((4096, torch.float16, "f16"), (8192, torch.bfloat16, "bf16")):
+        host = gemm_inputs(size, size, size, dt)
+        a, b = host["a"].cuda(), host["b"].cuda()
+        out = torch.empty(size, size, dtype=dt, device="cuda")
+        steps = args.steps if size <= 4096 else max(5, args.steps // 5)
+        pair("gemm_%s_%d" % (tag, size), gemm_flops(size, size, size), lambda: hexmi.matmul(a, b, out=out),
+             lambda: torch.matmul(a, b, out=out), "torch.matmul", steps)
+        del a, b, out
+    for shape in ((4, 32, 4096, 128), (1, 32, 16384, 128)):
+        host = attention_inputs(*shape)
+        q, k, v = host["q"].cuda(), host["k"].cuda(), host["v"].cuda()
+        out = torch.empty_like(q)
+        scale = host["sm_scale"]
+        steps = args.steps if shape[2] <= 4096 else max(5, args.steps // 5)
+        pair("attn_causal_f16_%dx%dx%dx%d" % shape, attention_flops(*shape, causal=True),
+             lambda: hexmi.flash_attention(q, k, v, scale, True, out=out),
+             lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale),
+             "F.scaled_dot_product_attention", steps)
+        del q, k, v, out
+    print(json.dumps(_calibration_line(args, "vendor", "hexmi and the libraries PyTorch-ROCm ships on the same "
+                                       "configurations, same box, alternating; fractions of 2.5 PFLOP/s",
+                                       "gemm_kernel_k64 / flash_fwd_kernel", rows, "vendor")))
+
+
 def run_lds_patterns(torch, hexmi, args):
     """--workload lds_patterns: cycles per wave-wide 16-byte LDS read for the tiled GEMM's fragment-read address
     patterns, the LDS saturated by 16 waves per compute unit (hexmi_lds_read_pattern)."""
@@ -843,6 +893,8 @@ def main():
         return run_issue_slots(torch, hexmi, args)
     if args.workload == "lds_patterns":
         return run_lds_patterns(torch, hexmi, args)
+    if args.workload == "vendor":
+        return run_vendor(torch, hexmi, args)
 
     wls = make_workloads()
     primary = wls[ALIASES.get(args.workload, args.workload)]
