@@ -789,7 +789,7 @@ class _Lambda:
     sets = None
 
     def __init__(self, fn):
-        self.step = lambda i: fn()
+        self.step = (lambda i: fn()) if fn is not None else None
 
 
 def run_vendor(torch, hexmi, args):
@@ -827,8 +827,37 @@ def run_vendor(torch, hexmi, args):
              lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale),
              "F.scaled_dot_product_attention", steps)
         del q, k, v, out
+    # the row kernels against torch's own, on buffer sets rotated over 1 GiB (the Infinity Cache cannot serve them)
+    from hexmi.workloads import (softmax_inputs, norm_inputs, softmax_bytes, rms_norm_bytes, layer_norm_bytes)
+
+    def pair_hbm(name, nbytes, ours, theirs, their_name, n_sets):
+        for who, fn in (("hexmi", ours), (their_name, theirs), ("hexmi", ours), (their_name, theirs)):
+            wl = _Lambda(None)
+            wl.step = lambda i, fn=fn: fn(i % n_sets)
+            m = measure(torch, wl, args.steps, args.warmup, not args.no_graph)
+            rows.append({"config": name, "library": who, "ms": round(m["ms"], 5), "ms_min": round(m["min"], 5),
+                         "gbs": round(nbytes / (m["ms"] * 1e-3) / 1e9, 1),
+                         "frac": round(nbytes / (m["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+            print("# %-34s %-28s %.4f ms  frac %.3f" % (name, who, rows[-1]["ms"], rows[-1]["frac"]), file=sys.stderr)
+
+    host = softmax_inputs()
+    xs = [host["x"].cuda() for _ in range(32)]
+    outs = [torch.empty_like(x) for x in xs]
+    pair_hbm("softmax_f32_4096x1024", softmax_bytes(4096, 1024), lambda j: hexmi.softmax(xs[j], out=outs[j]),
+             lambda j: torch.softmax(xs[j], dim=-1), "torch.softmax", 32)
+    del xs, outs
+    host = norm_inputs()
+    xs = [host["x"].cuda() for _ in range(8)]
+    outs = [torch.empty_like(x) for x in xs]
+    w, b = host["weight"].cuda(), host["bias"].cuda()
+    pair_hbm("rms_norm_f16_8192x4096", rms_norm_bytes(8192, 4096), lambda j: hexmi.rms_norm(xs[j], w, 1e-5, out=outs[j]),
+             lambda j: F.rms_norm(xs[j], (4096,), w, 1e-5), "F.rms_norm", 8)
+    pair_hbm("layer_norm_f16_8192x4096", layer_norm_bytes(8192, 4096),
+             lambda j: hexmi.layer_norm(xs[j], w, b, 1e-5, out=outs[j]),
+             lambda j: F.layer_norm(xs[j], (4096,), w, b, 1e-5), "F.layer_norm", 8)
+    del xs, outs
     print(json.dumps(_calibration_line(args, "vendor", "hexmi and the libraries PyTorch-ROCm ships on the same "
-                                       "configurations, same box, alternating; fractions of 2.5 PFLOP/s",
+                                       "configurations, same box, alternating; fractions of 2.5 PFLOP/s (of 8 TB/s for the row kernels)",
                                        "gemm_kernel_k64 / flash_fwd_kernel", rows, "vendor")))
 
 

@@ -394,7 +394,7 @@ def pack_w8(w_int8):
 
 
 def w8a16_matmul_packed(a, w_packed, scales, out=None):
-    """`w8a16_matmul` on weights packed by `pack_w8` (N = len(scales)). Same result bit for bit for 3 <= M <= 16
+    """`w8a16_matmul` on weights packed by `pack_w8` (N = len(scales)). Same result bit for bit for 3 <= M <= 8
     (the same kernel); for other M `w8a16_matmul` uses kernels that sum in another order (one fp16 ulp)."""
     if a.dtype != torch.float16 or w_packed.dtype != torch.int8 or scales.dtype != torch.float16:
         raise TypeError("hexmi.w8a16_matmul_packed: expected fp16 activations, packed int8 weights, fp16 scales")
