@@ -790,8 +790,13 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
 #pragma unroll
       for (int jj = 0; jj < TN / 2; ++jj) {
         if (live) {
-          Mfma16<T>::run(bf[ks][2 * jj], af[ks][row], acc[row][2 * jj]);
-          Mfma16<T>::run(bf[ks][2 * jj + 1], af[ks][row], acc[row][2 * jj + 1]);
+          // odd rounds walk the row of tiles backwards: the round boundary then changes one MFMA operand, not both.
+          // The kernel runs at the power limit and operand bits that do not toggle are power: +0.6 % at bf16 8192^3
+          // and +0.5 % at fp16 4096^3, six alternating runs each on one box, every run of the new order ahead of
+          // every run of the old one at 8192^3. (Which of the two operands a round holds fixed makes no difference.)
+          const int c0 = (row & 1) ? TN - 1 - 2 * jj : 2 * jj, c1 = (row & 1) ? c0 - 1 : c0 + 1;
+          Mfma16<T>::run(bf[ks][c0], af[ks][row], acc[row][c0]);
+          Mfma16<T>::run(bf[ks][c1], af[ks][row], acc[row][c1]);
         }
         HEXMI_FENCE;
         // side instructions of slot jj of round q
