@@ -761,13 +761,13 @@ def run_issue_slots(torch, hexmi, args):
     lib = _lib.lib()
     sink = torch.empty(lib.hexmi_num_cus() * 512, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
-    kinds = ["v_pk_add_f16", "v_fma_f32", "v_exp_f32"]
+    kinds = ["v_pk_add_f16", "v_fma_f32", "v_exp_f32", "v_fma_mix_f32", "v_cvt_f32_f16"]
     rows = []
     for waves in (1, 2):
         for shape in (1, 0):
             per_iter = 4 if shape == 0 else 16
             iters = 40000 if shape == 0 else 10000
-            for kind in (0, 2) if shape == 1 else (0, 1, 2):
+            for kind in (0, 2) if shape == 1 else (0, 1, 2, 3, 4):
                 for per in (0, 1, 2, 3, 4, 5, 6, 8):
                     fn = lambda: _lib.check(lib.hexmi_issue_slots(shape, kind, per, iters, waves, sink.data_ptr(), st),
                                             "hexmi_issue_slots")

@@ -135,7 +135,9 @@ void issue_slots_kernel(int iters, float* __restrict__ sink) {
         const int idx = (m * VPM + n) % 8;         // eight independent chains
         if constexpr (KIND == 0) asm volatile("v_pk_add_f16 %0, %0, %0" : "+v"(v[idx]));
         else if constexpr (KIND == 1) asm volatile("v_fma_f32 %0, %0, %0, %0" : "+v"(v[idx]));
-        else asm volatile("v_exp_f32 %0, %0" : "+v"(v[idx]));
+        else if constexpr (KIND == 2) asm volatile("v_exp_f32 %0, %0" : "+v"(v[idx]));
+        else if constexpr (KIND == 3) asm volatile("v_fma_mix_f32 %0, %0, %0, %0 op_sel_hi:[1,0,0]" : "+v"(v[idx]));
+        else asm volatile("v_cvt_f32_f16 %0, %0" : "+v"(v[idx]));
       }
     }
   }
@@ -252,7 +254,7 @@ extern "C" int hexmi_mfma_peak(int shape, int dtype, const void* operands, int64
 
 extern "C" int hexmi_issue_slots(int shape, int kind, int per_mfma, int64_t iters, int waves_per_simd, float* sink,
                                  hexmi_stream_t stream) {
-  if ((shape != 0 && shape != 1) || kind < 0 || kind > 2 || waves_per_simd < 1 || waves_per_simd > 2 || iters < 0 ||
+  if ((shape != 0 && shape != 1) || kind < 0 || kind > 4 || waves_per_simd < 1 || waves_per_simd > 2 || iters < 0 ||
       iters > 0x7fffffff || !sink)
     return HEXMI_EINVAL;
   const int cus = hexmi_num_cus();
@@ -263,11 +265,15 @@ extern "C" int hexmi_issue_slots(int shape, int kind, int per_mfma, int64_t iter
   if (shape == 0) {
     if (kind == 0) return launch_issue_slots<true, 0>(per_mfma, grid, block, st, (int)iters, sink);
     if (kind == 1) return launch_issue_slots<true, 1>(per_mfma, grid, block, st, (int)iters, sink);
-    return launch_issue_slots<true, 2>(per_mfma, grid, block, st, (int)iters, sink);
+    if (kind == 2) return launch_issue_slots<true, 2>(per_mfma, grid, block, st, (int)iters, sink);
+    if (kind == 3) return launch_issue_slots<true, 3>(per_mfma, grid, block, st, (int)iters, sink);
+    return launch_issue_slots<true, 4>(per_mfma, grid, block, st, (int)iters, sink);
   }
   if (kind == 0) return launch_issue_slots<false, 0>(per_mfma, grid, block, st, (int)iters, sink);
   if (kind == 1) return launch_issue_slots<false, 1>(per_mfma, grid, block, st, (int)iters, sink);
-  return launch_issue_slots<false, 2>(per_mfma, grid, block, st, (int)iters, sink);
+  if (kind == 2) return launch_issue_slots<false, 2>(per_mfma, grid, block, st, (int)iters, sink);
+  if (kind == 3) return launch_issue_slots<false, 3>(per_mfma, grid, block, st, (int)iters, sink);
+  return launch_issue_slots<false, 4>(per_mfma, grid, block, st, (int)iters, sink);
 }
 
 extern "C" int hexmi_lds_read_pattern(int pattern, int64_t iters, float* sink, hexmi_stream_t stream) {

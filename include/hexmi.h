@@ -347,7 +347,8 @@ int hexmi_mfma_peak(int shape, int dtype, const void *operands, int64_t iters,
  * hexmi_issue_slots: per MFMA of a registers-only stream (shape as above, fp16,
  * zero operands, 64 accumulator registers) per_mfma vector instructions of one
  * kind follow in the same wave: kind 0 = v_pk_add_f16, 1 = v_fma_f32,
- * 2 = v_exp_f32; per_mfma in {0,1,2,3,4,5,6,8}. The time per MFMA says how much
+ * 2 = v_exp_f32, 3 = v_fma_mix_f32 (one fp16 source), 4 = v_cvt_f32_f16;
+ * per_mfma in {0,1,2,3,4,5,6,8}. The time per MFMA says how much
  * vector work a kernel can place between its MFMAs before the SIMD's
  * instruction issue, not the matrix pipe, sets the pace. The launch runs
  * iters * (4 for shape 0, 16 for shape 1) MFMAs per wave.

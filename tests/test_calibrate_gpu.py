@@ -30,7 +30,7 @@ def test_argument_checks():
     sink = torch.empty(lib.hexmi_num_cus() * 1024, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
     assert lib.hexmi_issue_slots(2, 0, 0, 10, 1, sink.data_ptr(), st) == _lib.EINVAL       # shape
-    assert lib.hexmi_issue_slots(0, 3, 0, 10, 1, sink.data_ptr(), st) == _lib.EINVAL       # kind
+    assert lib.hexmi_issue_slots(0, 5, 0, 10, 1, sink.data_ptr(), st) == _lib.EINVAL       # kind
     assert lib.hexmi_issue_slots(0, 0, 7, 10, 1, sink.data_ptr(), st) == _lib.EINVAL       # per_mfma not offered
     assert lib.hexmi_issue_slots(0, 0, 0, 10, 3, sink.data_ptr(), st) == _lib.EINVAL       # waves per SIMD
     assert lib.hexmi_issue_slots(0, 0, 0, 10, 1, None, st) == _lib.EINVAL
@@ -62,7 +62,7 @@ def test_issue_slots_vector_work_beyond_the_shadow_costs_time():
     assert t[2] < 1.3 * t[0]
     assert t[8] > 1.7 * t[0]
     for shape in (0, 1):
-        for kind in (0, 1, 2):
+        for kind in (0, 1, 2, 3, 4):
             _lib.check(lib.hexmi_issue_slots(shape, kind, 5, 100, 2, sink.data_ptr(), st), "hexmi_issue_slots")
     torch.cuda.synchronize()
 
