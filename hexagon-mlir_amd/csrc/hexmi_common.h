@@ -55,10 +55,14 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float a, float
 // (quad permutes for lane^1 and lane^2; the half-row and row mirrors stand in for lane^4 and lane^8 because the
 // partial results are already uniform inside groups of 4 and 8), then v_permlane16_swap / v_permlane32_swap
 // for the exchanges between rows. Every lane ends with the full result.
+// (Every lane has a valid source under these permutations, so the value for lanes without one is never used; it is
+// given as 0 with the bound-control bit set, the form the compiler folds into the add or max that consumes the
+// exchange - v_add_f32_dpp, one instruction per step - where "keep the own value" leaves a copy, the exchange and
+// the add: three.)
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
   const int i = __builtin_bit_cast(int, v);
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xF, 0xF, false));
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, i, CTRL, 0xF, 0xF, true));
 }
 // {a, b} with a = value of the partner row (16 lanes) / half (32 lanes) and b = own, in some order that is the
 // same for both partners up to exchange: callers combine them with a commutative operation.
