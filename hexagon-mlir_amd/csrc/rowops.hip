@@ -71,6 +71,12 @@ __device__ __forceinline__ void fresh(Vec16<T>& r) {
 // ulp) and one Newton step, five instructions. The correctly rounded square root followed by the correctly rounded
 // division, which every thread of a row would execute, is forty: a fifth of all the vector instructions of a
 // LayerNorm row group. The result is within an ulp of theirs.
+// 1 / x the same way (v_rcp_f32 and one Newton step, three instructions for the correctly rounded division's ten),
+// for the sum of a softmax row: 1 <= x <= the row length.
+__device__ __forceinline__ float rcp_newton(float x) {
+  const float y = __builtin_amdgcn_rcpf(x);
+  return fmaf(fmaf(-x, y, 1.0f), y, y);
+}
 __device__ __forceinline__ float rsqrt_newton(float x) {
   const float y = __builtin_amdgcn_rsqf(x);
   const float e = fmaf(-(x * y), y, 1.0f);              // 1 - x y^2
@@ -205,7 +211,7 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
 #pragma unroll
         for (int i = 0; i < N; ++i) { v[c][i] = __expf(v[c][i] - m); s += v[c][i]; }
       s = block_reduce<false, WAVES>(s, red_b[slot][row_in_block], wave_in_row);
-      const float inv = 1.0f / s;
+      const float inv = rcp_newton(s);
 #pragma unroll
       for (int c = 0; c < CHUNKS; ++c) {
         const int col = (c * THREADS + t) * N;
