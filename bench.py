@@ -224,20 +224,28 @@ class Gemm(Workload):
 
 
 class W8A16(Workload):
-    bound, dtype, kernel = "hbm", "f16", "w8a16_kernel"
+    bound, dtype = "hbm", "f16"
+    # the kernel rocprofv3 names for each measured shape (the library picks by M, N, K)
+    KERNELS = {(1, 11008): "w8a16_gemv_kernel", (16, 11008): "w8a16_mid_kernel", (64, 11008): "w8a16_mid_kernel",
+               (256, 11008): "gemm_kernel_k64", (1, 4096): "w8a16_gemv_any_kernel", (16, 4096): "w8a16_mid_kernel",
+               (64, 4096): "w8a16_split_kernel", (256, 4096): "w8a16_split_kernel"}
 
-    def __init__(self, M):
-        self.M = M
-        self.name = "w8a16_m%d" % M
-        self.desc = "W8A16 A fp16 [%d,4096] N(0,1), W int8 [11008,4096], per-channel fp16 scales, fp32 accumulate" % M
+    def __init__(self, M, N=11008, K=4096):
+        self.M, self.N, self.K = M, N, K
+        # N = 11008, K = 4096 is the measured configuration (a gate / up projection); N = 4096, K = 11008 is the down
+        # projection of the same model: the same 45 MB of weights walked the other way
+        self.name = ("w8a16_m%d" if N == 11008 else "w8a16_down_m%d") % M
+        self.kernel = self.KERNELS.get((M, N), "w8a16")
+        self.desc = ("W8A16 A fp16 [%d,%d] N(0,1), W int8 [%d,%d], per-channel fp16 scales, fp32 accumulate"
+                     % (M, K, N, K))
 
     def setup(self, torch, hexmi):
         from hexmi.workloads import w8a16_inputs, w8a16_bytes
-        self.hexmi, self.host = hexmi, w8a16_inputs(self.M)
-        self.work = w8a16_bytes(self.M, 11008, 4096)
+        self.hexmi, self.host = hexmi, w8a16_inputs(self.M, self.N, self.K)
+        self.work = w8a16_bytes(self.M, self.N, self.K)
         self.sets = _sets(torch, self.host, self.work)
         for s in self.sets:
-            s["out"] = torch.empty(self.M, 11008, dtype=torch.float16, device="cuda")
+            s["out"] = torch.empty(self.M, self.N, dtype=torch.float16, device="cuda")
 
     def step(self, i):
         s = self.sets[i % len(self.sets)]
@@ -551,6 +559,7 @@ def make_workloads():
     return {w.name: w for w in (
         Norms(), Softmax(), Softmax(65536, 1024), RmsNorm(), LayerNorm(), Gemm(4096, "f16"), Gemm(8192, "bf16"),
         Gemm(8192, "bf16", packed=True), Gemm(4096, "f32"), W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256),
+        W8A16(1, 4096, 11008), W8A16(16, 4096, 11008), W8A16(64, 4096, 11008), W8A16(256, 4096, 11008),
         Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), AttentionF32(4, 32, 2048, 64),
         MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
         Elementwise("sum"), LinearFused(), AddMatmulSoftmax(32, 32, 32, "f32"), AddMatmulSoftmax(512, 512, 64, "f16"),
@@ -569,7 +578,8 @@ ALIASES = {"copy": "copy_64MiB", "norms": "norms_f16_8192x4096", "softmax": "sof
            "attn_f32": "attn_causal_f32_4x32x2048x64", "gelu": "gelu_f16_8192x4096", "silu": "silu_f16_8192x4096",
            "rope": "rope_f16_4x4096x32x128", "sum": "block_sum_f32_8192x4096", "rms_norm": "rms_norm_f16_8192x4096",
            "layer_norm": "layer_norm_f16_8192x4096", "w8a16_m1": "w8a16_m1", "w8a16_m16": "w8a16_m16",
-           "w8a16_m64": "w8a16_m64", "w8a16_m256": "w8a16_m256",
+           "w8a16_m64": "w8a16_m64", "w8a16_m256": "w8a16_m256", "w8a16_down_m1": "w8a16_down_m1",
+           "w8a16_down_m16": "w8a16_down_m16", "w8a16_down_m64": "w8a16_down_m64", "w8a16_down_m256": "w8a16_down_m256",
            "linear": "linear_bias_residual_f16_8192x768x3072", "ams": "add_matmul_softmax_f32_32x32x32",
            "ams_mid": "add_matmul_softmax_f16_512x512x64"}
 
@@ -628,7 +638,7 @@ def measure_hot(torch, wl, steps, warmup, use_graph):
 
 PROFILE_KEYS = {"norms_f16_8192x4096": "norms", "softmax_f32_4096x1024": "softmax", "gemm_f16_4096": "gemm",
                 "gemm_bf16_8192": "gemm_bf16", "gemm_f32_4096": "gemm_f32", "w8a16_m1": "w8a16_m1", "w8a16_m16": "w8a16_m16",
-                "w8a16_m256": "w8a16_m256", "attn_causal_f16_4x32x4096x128": "attn",
+                "w8a16_m64": "w8a16_m64", "w8a16_m256": "w8a16_m256", "attn_causal_f16_4x32x4096x128": "attn",
                 "attn_causal_f16_1x32x16384x128": "attn_long", "attn_masked_f16_32x2048x128": "attn_masked", "attn_causal_f32_4x32x2048x64": "attn_f32"}
 
 
@@ -667,7 +677,7 @@ def entry_for(torch, wl, m, hot, cores, with_cpu):
     if hot is not None:
         entry["hot"] = {"ms": round(hot["ms"], 5), "frac": report(wl, hot["ms"])["frac"],
                         "note": "one buffer set: Infinity-Cache resident where it fits, not an HBM figure"}
-    if wl.name == "w8a16_m256":
+    if wl.name in ("w8a16_m256", "w8a16_down_m256"):
         # 23 GFLOP: this shape is matrix-bound, not weight-stream-bound; both fractions are reported
         flop = 2.0 * 256 * 11008 * 4096
         entry["mfma_frac"] = round(flop / (m["ms"] * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)

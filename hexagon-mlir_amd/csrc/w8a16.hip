@@ -569,6 +569,65 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
   }
 }
 
+// The same decode kernel for any K that is a multiple of 16 (up to NJ KiB per row): lane i takes the 16-byte pieces
+// i, i + 64, ... of the row, the last round masked where the row has ended (zero weights). One channel per wave, eight
+// waves per workgroup; the activation rows are staged in LDS once per workgroup and read back piece by piece, so the
+// registers hold the row's weight loads (all in flight at once) and little else.
+template <int MR, int NJ>
+__global__ __launch_bounds__(512)
+void w8a16_gemv_any_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
+                           f16* __restrict__ C, int M, int N, int K) {
+  constexpr int NW = 8;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n = blockIdx.x * NW + wave;                     // may lie past N in the last workgroup: loads clamp
+  const f16 sc = scales[n < N ? n : N - 1];
+  const int pieces = K / 16;                                // 16-byte pieces of a weight row
+  u32x4 wv[NJ];
+  {
+    const int8_t* wrow = W + (int64_t)(n < N ? n : N - 1) * K;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int pc = j * 64 + lane;
+      wv[j] = u32x4{0u, 0u, 0u, 0u};
+      if (pc < pieces) wv[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + pc * 16));
+    }
+  }
+  __shared__ __attribute__((aligned(16))) f16 a_lds[MR][NJ * 1024];
+  for (int m = 0; m < MR; ++m) {
+    const f16* arow = A + (int64_t)(m < M ? m : 0) * K;
+    for (int c = threadIdx.x; c < K / 8; c += NW * 64)
+      *reinterpret_cast<f16x8*>(&a_lds[m][c * 8]) = *reinterpret_cast<const f16x8*>(arow + c * 8);
+  }
+  __syncthreads();
+  float acc[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const int pc = j * 64 + lane;
+    if (j * 64 < pieces) {                                  // wave-uniform: rounds past the row do nothing
+      f16x8 w0, w1;
+      cvt16(wv[j], w0, w1);
+      const int at = (pc < pieces ? pc : 0) * 16;           // masked lanes hold zero weights; any valid address
+#pragma unroll
+      for (int m = 0; m < MR; ++m) {
+        const f16x8 a0 = *reinterpret_cast<const f16x8*>(&a_lds[m][at]);
+        const f16x8 a1 = *reinterpret_cast<const f16x8*>(&a_lds[m][at + 8]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc[m] = __builtin_amdgcn_fdot2(f16x2{w0[2 * e], w0[2 * e + 1]}, f16x2{a0[2 * e], a0[2 * e + 1]}, acc[m], false);
+          acc[m] = __builtin_amdgcn_fdot2(f16x2{w1[2 * e], w1[2 * e + 1]}, f16x2{a1[2 * e], a1[2 * e + 1]}, acc[m], false);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    const float tot = wave_sum(acc[m]);
+    if (lane == 0 && n < N && m < M) C[(int64_t)m * N + n] = (f16)(tot * (float)sc);
+  }
+}
+
 // One-time re-layout of int8 weights [N, K] into fragment-major order for the small-M kernels (the analogue of
 // the reference's constant-weight block linearisation, qcom_hexagon_backend/lib/Transforms/
 // PreprocessWeightsForHMXPass.cpp:39-117): tiles of 16 channels x 64 k, tile (t, s) at byte
@@ -652,6 +711,24 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
   f16* c = static_cast<f16*>(C);
   begin_call();
   if (K == 0) return fill_zero_2d(C, M, N, N, 2, st);      // an empty sum
+  if (M <= 2 && K % 16 == 0 && K <= 16384 && K != 1024 && K != 2048 && K != 4096 && K != 8192 && aligned_to(A, 16) &&
+      aligned_to(W, 16)) {
+    // any other row length: the masked form of the same kernel, instantiated per KiB of row
+    const unsigned blocks = (unsigned)((N + 7) / 8);
+    const int nj = (int)((K + 1023) / 1024);
+#define HEXMI_GEMV_ANY(MR, NJ) hipLaunchKernelGGL((w8a16_gemv_any_kernel<MR, NJ>), dim3(blocks), dim3(512), 0, st, a, W, s, c, (int)M, (int)N, (int)K)
+#define HEXMI_GEMV_ANY_NJ(MR) switch (nj) { \
+    case 1: HEXMI_GEMV_ANY(MR, 1); break; case 2: HEXMI_GEMV_ANY(MR, 2); break; case 3: HEXMI_GEMV_ANY(MR, 3); break; \
+    case 4: HEXMI_GEMV_ANY(MR, 4); break; case 5: HEXMI_GEMV_ANY(MR, 5); break; case 6: HEXMI_GEMV_ANY(MR, 6); break; \
+    case 7: HEXMI_GEMV_ANY(MR, 7); break; case 8: HEXMI_GEMV_ANY(MR, 8); break; case 9: HEXMI_GEMV_ANY(MR, 9); break; \
+    case 10: HEXMI_GEMV_ANY(MR, 10); break; case 11: HEXMI_GEMV_ANY(MR, 11); break; case 12: HEXMI_GEMV_ANY(MR, 12); break; \
+    case 13: HEXMI_GEMV_ANY(MR, 13); break; case 14: HEXMI_GEMV_ANY(MR, 14); break; case 15: HEXMI_GEMV_ANY(MR, 15); break; \
+    default: HEXMI_GEMV_ANY(MR, 16); break; }
+    if (M == 1) { HEXMI_GEMV_ANY_NJ(1) } else { HEXMI_GEMV_ANY_NJ(2) }
+#undef HEXMI_GEMV_ANY_NJ
+#undef HEXMI_GEMV_ANY
+    return launch_status();
+  }
   // the fast kernels read 16 bytes of a weight row per lane in 64-wide K steps; other shapes take the generic one
   if (K % 64 != 0 || !aligned_to(A, 16) || !aligned_to(W, 16)) {
     constexpr int MR = 4;
@@ -711,6 +788,66 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
   }
   return rc;
 }
+
+namespace {
+// Shapes the (channel range x K part) kernel takes ahead of the kernels of hexmi_gemm_w8a16, from timings of both over
+// N in 1024 .. 28672 and K in 2048 .. 14336 on 256 CUs. Those kernels give every workgroup all of K and up to 48
+// channels (M <= 128) or a 128 x 128 tile (M > 128): they fall behind when that leaves CUs idle or oversubscribed
+// (N > 48 channels per CU; fewer tiles than half the CUs) and when K is long (every workgroup pulls M x K of
+// activations through L2).
+bool prefer_split(int64_t M, int64_t N, int64_t K, int cus) {
+  if (M < 32 || M > 256) return false;
+  if (M <= 128) return N > 48 * (int64_t)cus || (K >= 8192 && M >= 64);
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  return tiles * 2 <= cus;
+}
+}  // namespace
+
+extern "C" int64_t hexmi_gemm_w8a16_workspace(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const int cus = hexmi_num_cus();
+  if (cus <= 0 || !prefer_split(M, N, K, cus)) return 0;
+  return w8a16_split_workspace(M, N, K, cus);
+}
+
+extern "C" int hexmi_gemm_w8a16_ws(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
+                                   void* C, void* workspace, int64_t workspace_bytes, hexmi_stream_t stream) {
+  if (M < 0 || N < 0 || K < 0 || workspace_bytes < 0) return HEXMI_EINVAL;
+  if (M == 0 || N == 0) return HEXMI_OK;
+  if (!C || (K > 0 && (!A || !W || !scales))) return HEXMI_EINVAL;
+  const int cus = hexmi_num_cus();
+  if (cus > 0 && K > 0 && prefer_split(M, N, K, cus) && (workspace || w8a16_split_workspace(M, N, K, cus) == 0)) {
+    const int64_t need = w8a16_split_workspace(M, N, K, cus);
+    if (need > 0 && workspace_bytes < need) return HEXMI_EINVAL;
+    hipStream_t st = as_stream(stream);
+    begin_call();
+    int rc = HEXMI_OK;
+    if (need > 0) {
+      // the flags the K parts raise start at zero in every call: the workspace carries nothing from one call to the next
+      rc = w8a16_split_clear(workspace, w8a16_split_header(M, N, K, cus), st);
+      if (rc != HEXMI_OK) return rc;
+    }
+    if (w8a16_split(M, N, K, static_cast<const f16*>(A), W, static_cast<const f16*>(scales), static_cast<f16*>(C),
+                    workspace, workspace_bytes, cus, st, &rc))
+      return rc;
+  }
+  return hexmi_gemm_w8a16(M, N, K, A, W, scales, C, stream);
+}
+
+#ifdef HEXMI_TUNE
+// measurement hook (not built into the library): the split kernel with a forced decomposition
+extern "C" int hexmi_w8_tune(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
+                             void* C, void* ws, int64_t ws_bytes, int parts, int cols, int clear,
+                             hexmi_stream_t stream) {
+  hipStream_t st = as_stream(stream);
+  int rc = HEXMI_OK;
+  if (clear) rc = w8a16_split_clear(ws, 4096, st);
+  if (!w8a16_split(M, N, K, static_cast<const f16*>(A), W, static_cast<const f16*>(scales), static_cast<f16*>(C), ws,
+                   ws_bytes, hexmi_num_cus(), st, &rc, parts, cols))
+    return HEXMI_ENOTSUP;
+  return rc;
+}
+#endif
 
 extern "C" int hexmi_pack_w8(int64_t N, int64_t K, const int8_t* W, int8_t* Wp, hexmi_stream_t stream) {
   if (N < 0 || K < 0) return HEXMI_EINVAL;

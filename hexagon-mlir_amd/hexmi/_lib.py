@@ -39,6 +39,8 @@ SIGNATURES = {
     "hexmi_add_matmul_softmax": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _ptr]),
     "hexmi_transpose16": (_int, [_i64, _i64, _ptr, _i64, _ptr, _i64, _ptr]),
     "hexmi_gemm_w8a16": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "hexmi_gemm_w8a16_workspace": (_i64, [_i64, _i64, _i64]),
+    "hexmi_gemm_w8a16_ws": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "hexmi_pack_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr]),
     "hexmi_gemm_w8a16_packed": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_dequant_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),

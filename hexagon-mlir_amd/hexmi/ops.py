@@ -139,12 +139,26 @@ def _add_matmul_softmax_impl(x, y, z, out):
                    "hexmi_add_matmul_softmax")
 
 
+_W8_WORKSPACES = {}          # (device index, stream) -> uint8 tensor, grown on demand
+
+
 def _w8a16_impl(a, w, scales, out):
     M, K = a.shape
     N = w.shape[0]
     with _on(a.device):
-        _lib.check(_lib.lib().hexmi_gemm_w8a16(M, N, K, _p(a), _p(w), _p(scales), _p(out), _stream()),
-                   "hexmi_gemm_w8a16")
+        # shapes the library sums over several K parts need fp32 scratch for the partial tiles; one buffer per device
+        # and stream is kept and reused (calls on one stream are ordered, so they may share it)
+        need = _lib.lib().hexmi_gemm_w8a16_workspace(M, N, K)
+        ws = None
+        if need:
+            key = (a.device.index, _stream())
+            ws = _W8_WORKSPACES.get(key)
+            if ws is None or ws.numel() < need:
+                ws = torch.empty(need, dtype=torch.uint8, device=a.device)
+                _W8_WORKSPACES[key] = ws
+        _lib.check(_lib.lib().hexmi_gemm_w8a16_ws(M, N, K, _p(a), _p(w), _p(scales), _p(out), _p(ws),
+                                                  ws.numel() if ws is not None else 0, _stream()),
+                   "hexmi_gemm_w8a16_ws")
 
 
 def _pack_impl(w, out):

@@ -163,6 +163,30 @@ int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void *A,
                      const int8_t *W, const void *scales, void *C,
                      hexmi_stream_t stream);
 
+/* hexmi_gemm_w8a16 with a caller-owned scratch buffer, for the shapes whose
+ * kernels of choice split K over several workgroups and add the fp32 partial
+ * tiles up afterwards: 32 <= M <= 256 with more than 48 output channels per
+ * compute unit, with K >= 8192 (M >= 64), or, for M > 128, with fewer 128 x 128
+ * tiles than half the compute units (the down projection N = 4096, K = 11008 of
+ * the model whose up projection is the benchmark shape is one: M = 256 in 40 us
+ * where hexmi_gemm_w8a16 takes 75). hexmi_gemm_w8a16_workspace returns the bytes
+ * that takes for (M, N, K) on the current device, 0 when hexmi_gemm_w8a16's own
+ * kernels are used anyway. workspace may be NULL (then they are used for every
+ * shape the query answers with a size); a workspace smaller than the query's
+ * answer is HEXMI_EINVAL. It must
+ * be 16-byte aligned, needs no initialisation and holds no state between calls;
+ * two calls that overlap in time (different streams) need a workspace each.
+ * Partial tiles are added in a fixed order: results are reproducible bit for
+ * bit, and permuting output channels permutes the columns of C.
+ * The reference's counterpart is the scratch its matmul runtime routine sets up
+ * per call (bin/runtime/src/HexKLAPI.cpp:15-68: VTCM for tiles and the
+ * accumulator read-back). */
+int64_t hexmi_gemm_w8a16_workspace(int64_t M, int64_t N, int64_t K);
+int hexmi_gemm_w8a16_ws(int64_t M, int64_t N, int64_t K, const void *A,
+                        const int8_t *W, const void *scales, void *C,
+                        void *workspace, int64_t workspace_bytes,
+                        hexmi_stream_t stream);
+
 /* out[n,k] (fp32) = float(W[n,k]) * float(scales[n]): the dequantisation the
  * fused kernel applies, exposed so indexing and scale selection can be
  * checked bit-exactly. */

@@ -177,3 +177,106 @@ def test_packed_weights_through_a_tensor_file(hexmi, tmp_path):
     assert back.dtype == torch.int8 and torch.equal(back, wp.cpu())
     got = hexmi.w8a16_matmul_packed(a.cuda(), back.cuda(), s.cuda()).cpu()
     assert torch.equal(got, hexmi.w8a16_matmul_packed(a.cuda(), wp, s.cuda()).cpu())
+
+
+# ---- the (channel range x K part) kernel behind hexmi_gemm_w8a16_ws -------------------------------------------
+
+def _ws_call(hexmi, a, w, s, ws, ws_bytes=None):
+    """hexmi_gemm_w8a16_ws through the C ABI on device tensors; ws may be None."""
+    lib = hexmi.lib()
+    M, K = a.shape
+    N = w.shape[0]
+    c = torch.full((M, N), 7.0, dtype=torch.float16, device="cuda")
+    rc = lib.hexmi_gemm_w8a16_ws(M, N, K, a.data_ptr(), w.data_ptr(), s.data_ptr(), c.data_ptr(),
+                                 ws.data_ptr() if ws is not None else None,
+                                 (ws.numel() if ws is not None else 0) if ws_bytes is None else ws_bytes,
+                                 torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return rc, c
+
+
+# shapes the library gives to that kernel: many channels per CU, a long K, or few 128 x 128 tiles; K parts 1, 2, 8;
+# ragged channel ranges, a last row tile of one row, a last channel range of eight channels
+SPLIT_SHAPES = [(64, 96, 8192), (33, 12300, 128), (256, 1000, 1024), (129, 2000, 384), (200, 8192, 2048),
+                (100, 13000, 256), (80, 264, 16384), (250, 72, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", SPLIT_SHAPES)
+def test_w8a16_split_parity(hexmi, oracle, M, N, K):
+    a, w, s = _inputs(M, N, K, seed=11)
+    ad, wd, sd = a.cuda(), w.cuda(), s.cuda()
+    need = hexmi.lib().hexmi_gemm_w8a16_workspace(M, N, K)
+    # the scratch starts out as garbage: the library must not rely on its contents
+    ws = torch.full((max(need, 16),), 0xA5, dtype=torch.uint8, device="cuda")
+    rc, got = _ws_call(hexmi, ad, wd, sd, ws)
+    assert rc == 0
+    ch = torch.arange(0, N, max(1, N // 160))
+    want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w[ch].contiguous().numpy(), s[ch].contiguous().numpy()))
+    assert close16(got.cpu()[:, ch], want, max_ulp=1, atol=2e-4)
+    assert (got.cpu()[:, ch].float() - want.float()).abs().max() / math.sqrt(K) <= 2e-2
+    # the operator front takes the same path (it keeps a workspace per stream) and gives the same bits, again and again
+    for _ in range(3):
+        assert torch.equal(hexmi.w8a16_matmul(ad, wd, sd), got)
+    # against the kernels of the plain entry point (another summation order; each is within one unit in the last
+    # place of the oracle, so of each other within two; where the value is a cancellation residue of fp32 partial sums
+    # the two orders differ by the rounding of those sums, which grows with K)
+    plain = torch.empty_like(got)
+    assert hexmi.lib().hexmi_gemm_w8a16(M, N, K, ad.data_ptr(), wd.data_ptr(), sd.data_ptr(), plain.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert close16(got.cpu(), plain.cpu(), max_ulp=2, atol=2e-4 * max(1.0, K / 4096))
+    # permuting output channels permutes the columns, bit for bit
+    perm = torch.randperm(N, generator=_gen(12))
+    rc, got_p = _ws_call(hexmi, ad, w[perm].contiguous().cuda(), s[perm].contiguous().cuda(), ws)
+    assert rc == 0 and torch.equal(got_p.cpu(), got.cpu()[:, perm])
+
+
+@pytest.mark.parametrize("M", [64, 128, 256])
+def test_w8a16_down_projection_sizes(hexmi, oracle, M):
+    # the other projection of the benchmark's model: N = 4096, K = 11008 (the oracle on every 29th channel)
+    N, K = 4096, 11008
+    a, w, s = _inputs(M, N, K, seed=13)
+    assert hexmi.lib().hexmi_gemm_w8a16_workspace(M, N, K) > 0
+    got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
+    ch = torch.arange(0, N, 29)
+    want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w[ch].contiguous().numpy(), s[ch].contiguous().numpy()))
+    assert close16(got[:, ch], want, max_ulp=1, atol=2e-4)
+    assert (got[:, ch].float() - want.float()).abs().max() / math.sqrt(K) <= 2e-2
+    perm = torch.randperm(N, generator=_gen(14))
+    got_p = hexmi.w8a16_matmul(a.cuda(), w[perm].contiguous().cuda(), s[perm].contiguous().cuda()).cpu()
+    assert torch.equal(got_p, got[:, perm])
+
+
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("N,K", [(4096, 11008), (100, 80), (37, 16384), (64, 1040), (9, 5120)])
+def test_w8a16_decode_any_row_length(hexmi, oracle, M, N, K):
+    # one or two rows with K % 16 == 0 outside {1024, 2048, 4096, 8192}: the masked form of the decode kernel
+    a, w, s = _inputs(M, N, K, seed=15)
+    got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
+    ch = torch.arange(0, N, max(1, N // 200))
+    want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w[ch].contiguous().numpy(), s[ch].contiguous().numpy()))
+    assert close16(got[:, ch], want, max_ulp=1, atol=2e-4)
+    perm = torch.randperm(N, generator=_gen(16))
+    got_p = hexmi.w8a16_matmul(a.cuda(), w[perm].contiguous().cuda(), s[perm].contiguous().cuda()).cpu()
+    assert torch.equal(got_p, got[:, perm])
+
+
+def test_w8a16_workspace_contract(hexmi):
+    lib = hexmi.lib()
+    # shapes the plain kernels keep: no workspace asked for, and a NULL workspace is fine
+    assert lib.hexmi_gemm_w8a16_workspace(16, 11008, 4096) == 0
+    assert lib.hexmi_gemm_w8a16_workspace(64, 11008, 4096) == 0
+    assert lib.hexmi_gemm_w8a16_workspace(0, 64, 64) == 0
+    M, N, K = 64, 4096, 11008
+    need = lib.hexmi_gemm_w8a16_workspace(M, N, K)
+    assert need > 0
+    a, w, s = _inputs(M, N, K, seed=17)
+    ad, wd, sd = a.cuda(), w.cuda(), s.cuda()
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    rc, with_ws = _ws_call(hexmi, ad, wd, sd, ws)
+    assert rc == 0
+    rc, _ = _ws_call(hexmi, ad, wd, sd, ws, ws_bytes=need - 1)
+    assert rc == hexmi._lib.EINVAL
+    rc, no_ws = _ws_call(hexmi, ad, wd, sd, None)             # the plain kernels
+    assert rc == 0 and close16(no_ws.cpu(), with_ws.cpu(), max_ulp=2, atol=2e-4)
+    rc, _ = _ws_call(hexmi, ad, wd, sd, ws, ws_bytes=-1)
+    assert rc == hexmi._lib.EINVAL
