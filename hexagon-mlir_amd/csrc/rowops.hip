@@ -77,10 +77,13 @@ __device__ __forceinline__ float rcp_newton(float x) {
   const float y = __builtin_amdgcn_rcpf(x);
   return fmaf(fmaf(-x, y, 1.0f), y, y);
 }
+// Outside that range the estimate itself is the answer (x = 0: inf, x = inf: 0, NaN: NaN) and the step, which would
+// multiply 0 by inf, is skipped.
 __device__ __forceinline__ float rsqrt_newton(float x) {
   const float y = __builtin_amdgcn_rsqf(x);
   const float e = fmaf(-(x * y), y, 1.0f);              // 1 - x y^2
-  return fmaf(0.5f * y, e, y);
+  const float r = fmaf(0.5f * y, e, y);
+  return (y > 0.0f && y < INFINITY) ? r : y;
 }
 
 // THREADS threads cooperate on one row (THREADS == 64: a wave per row, several
@@ -365,6 +368,222 @@ void row_kernel_generic(const T* __restrict__ x, T* __restrict__ y, const T* __r
   }
 }
 
+// ---- rows split over several workgroups -------------------------------------------------------------------------
+// A row that one workgroup cannot hold (more than 128 KiB), or a problem of so few rows that one workgroup per row
+// leaves most CUs idle, is cut into parts of part_cols columns. Pass 1 reduces every part on its own, from
+// registers, and leaves its statistics in a workspace; pass 2 merges the statistics of the row's parts, reads its
+// part again (from L2 when the problem is small) and writes the result.
+//   softmax: (m_p, l_p) = (max, sum exp(x - m_p)); merged as in the online form of
+//            test/python/triton/test_online_softmax.py:60-71 (m = max(m_i, m_ij); l = l * exp(m_i - m) + l_ij), which is
+//            associative: m = max_p m_p, l = sum_p l_p exp(m_p - m), summed in a fixed order.
+//   RMSNorm: sum of squares. LayerNorm: (mean_p, M2_p = sum (x - mean_p)^2), merged to mean = sum n_p mean_p / n and
+//            M2 = sum (M2_p + n_p (mean_p - mean)^2): the two-pass variance of the reference kernel
+//            (test/python/triton/test_layer_norm.py:60-72) without a third sweep.
+// A part is CHUNKS 16-byte chunks per thread of a 256-thread workgroup; chunks past the part or the row are masked.
+constexpr int kPartThreads = 256;
+
+template <typename T, int CHUNKS>
+struct PartTile {
+  static constexpr int N = Vec16<T>::N;
+  float v[CHUNKS][N];
+  bool in[CHUNKS];
+  int col[CHUNKS];
+  // loads part `part` of the row at xr; masked slots hold `fill`
+  __device__ __forceinline__ void load(const T* xr, int64_t cols, int64_t part_cols, int64_t part, float fill) {
+    const int64_t c0 = part * part_cols;
+    const int64_t c1 = c0 + part_cols < cols ? c0 + part_cols : cols;
+    Vec16<T> raw[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const int64_t at = c0 + (int64_t)(c * kPartThreads + threadIdx.x) * N;
+      in[c] = at < c1;
+      col[c] = (int)(in[c] ? at - c0 : 0);
+      raw[c] = load16(xr + c0 + col[c]);
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < N; ++i) v[c][i] = in[c] ? to_f32<T>(raw[c].v[i]) : fill;
+  }
+};
+
+template <typename T, int OP, int CHUNKS>
+__global__ __launch_bounds__(kPartThreads)
+void part_stats_kernel(const T* __restrict__ x, float* __restrict__ stats, int64_t cols, int64_t ld_x,
+                       int64_t part_cols, int64_t parts) {
+  constexpr int N = Vec16<T>::N;
+  constexpr int WAVES = kPartThreads / kWave;
+  __shared__ float red_a[WAVES];
+  __shared__ float red_b[WAVES];
+  const int64_t row = blockIdx.x / parts, part = blockIdx.x % parts;
+  const int wave = threadIdx.x / kWave;
+  PartTile<T, CHUNKS> tile;
+  tile.load(x + row * ld_x, cols, part_cols, part, OP == kSoftmax ? -INFINITY : 0.0f);
+  float s0, s1 = 0.0f;
+  if constexpr (OP == kSoftmax) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < N; ++i) m = fmaxf(m, tile.v[c][i]);
+    m = block_reduce<true, WAVES>(m, red_a, wave);
+    float l = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < N; ++i) l += __expf(tile.v[c][i] - m);     // masked slots: exp(-inf) = 0
+    s0 = m;
+    s1 = block_reduce<false, WAVES>(l, red_b, wave);
+    if (m == -INFINITY) s1 = 0.0f;                   // a part of -inf only adds nothing (its own sum would be NaN)
+  } else if constexpr (OP == kRmsNorm) {
+    float q = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < N; ++i) q += tile.v[c][i] * tile.v[c][i];
+    s0 = block_reduce<false, WAVES>(q, red_a, wave);
+  } else {
+    const int64_t c0 = part * part_cols;
+    const float n_p = (float)(c0 + part_cols < cols ? part_cols : cols - c0);
+    float s = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+      for (int i = 0; i < N; ++i) s += tile.v[c][i];
+    const float mean = block_reduce<false, WAVES>(s, red_a, wave) / n_p;
+    float q = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+      if (tile.in[c]) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) { const float d = tile.v[c][i] - mean; q += d * d; }
+      }
+    s0 = mean;
+    s1 = block_reduce<false, WAVES>(q, red_b, wave);
+  }
+  if (threadIdx.x == 0) {
+    stats[blockIdx.x * 2] = s0;
+    stats[blockIdx.x * 2 + 1] = s1;
+  }
+}
+
+template <typename T, int OP, int CHUNKS>
+__global__ __launch_bounds__(kPartThreads)
+void part_apply_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict__ w, const T* __restrict__ b,
+                       float* __restrict__ mean_out, float* __restrict__ rstd_out, const float* __restrict__ stats,
+                       int64_t cols, int64_t ld_x, int64_t ld_y, int64_t part_cols, int64_t parts, float eps) {
+  constexpr int N = Vec16<T>::N;
+  constexpr int WAVES = kPartThreads / kWave;
+  __shared__ float red_a[WAVES];
+  __shared__ float red_b[WAVES];
+  const int64_t row = blockIdx.x / parts, part = blockIdx.x % parts;
+  const int wave = threadIdx.x / kWave;
+  const float* st = stats + row * parts * 2;
+  // the row's own part first (its loads are in flight while the statistics are merged)
+  PartTile<T, CHUNKS> tile;
+  tile.load(x + row * ld_x, cols, part_cols, part, 0.0f);
+  // merge: thread t takes parts t, t + 256, ... in order, then the threads are combined by the block reductions
+  float a = 0.0f, scale = 0.0f;                    // softmax: a = max, scale = 1 / sum; norms: a = mean, scale = rstd
+  if constexpr (OP == kSoftmax) {
+    float m = -INFINITY;
+    for (int64_t i = threadIdx.x; i < parts; i += kPartThreads) m = fmaxf(m, st[i * 2]);
+    m = block_reduce<true, WAVES>(m, red_a, wave);
+    float l = 0.0f;
+    for (int64_t i = threadIdx.x; i < parts; i += kPartThreads) l += st[i * 2 + 1] * __expf(st[i * 2] - m);
+    l = block_reduce<false, WAVES>(l, red_b, wave);
+    a = m;
+    scale = rcp_newton(l);
+  } else if constexpr (OP == kRmsNorm) {
+    float q = 0.0f;
+    for (int64_t i = threadIdx.x; i < parts; i += kPartThreads) q += st[i * 2];
+    q = block_reduce<false, WAVES>(q, red_a, wave);
+    scale = rsqrt_newton(q / (float)cols + eps);
+  } else {
+    auto n_of = [&](int64_t i) { return (float)(i * part_cols + part_cols < cols ? part_cols : cols - i * part_cols); };
+    float s = 0.0f;
+    for (int64_t i = threadIdx.x; i < parts; i += kPartThreads) s += n_of(i) * st[i * 2];
+    const float mean = block_reduce<false, WAVES>(s, red_a, wave) / (float)cols;
+    float q = 0.0f;
+    for (int64_t i = threadIdx.x; i < parts; i += kPartThreads) {
+      const float d = st[i * 2] - mean;
+      q += st[i * 2 + 1] + n_of(i) * d * d;
+    }
+    q = block_reduce<false, WAVES>(q, red_b, wave);
+    a = mean;
+    scale = rsqrt_newton(q / (float)cols + eps);
+    if (part == 0 && threadIdx.x == 0) {
+      if (mean_out) mean_out[row] = mean;
+      if (rstd_out) rstd_out[row] = scale;
+    }
+  }
+  const int64_t c0 = part * part_cols;
+  T* yr = y + row * ld_y + c0;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    if (!tile.in[c]) continue;
+    Vec16<T> o, wv, bv;
+    if (OP != kSoftmax && w) wv = load16(w + c0 + tile.col[c]);
+    if (OP == kLayerNorm && b) bv = load16(b + c0 + tile.col[c]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      float r;
+      if constexpr (OP == kSoftmax) {
+        r = __expf(tile.v[c][i] - a) * scale;
+      } else {
+        r = (tile.v[c][i] - a) * scale;
+        if (w) r *= to_f32<T>(wv.v[i]);
+        if (OP == kLayerNorm && b) r += to_f32<T>(bv.v[i]);
+      }
+      o.v[i] = from_f32<T>(r);
+    }
+    store16_stream(yr + tile.col[c], o);
+  }
+}
+
+// The split of a (rows x cols) problem: part_cols == 0 means the single-pass kernels take it. block_cols > 0 asks for
+// parts of that many columns (rounded up to whole 16-byte chunks, at most 32 KiB); block_cols == 0 leaves the choice
+// to the library: rows of more than 128 KiB, and problems of fewer rows than half the CUs whose rows are at least
+// 32 KiB, in parts of 4 .. 16 KiB so that there are about two workgroups per CU.
+struct RowSplit {
+  int64_t part_cols, parts;
+  int chunks;
+};
+inline RowSplit plan_row_split(int64_t rows, int64_t cols, int64_t block_cols, int elem_size, int cus) {
+  RowSplit r = {0, 0, 0};
+  const int64_t n = 16 / elem_size;                // elements per 16-byte chunk
+  const int64_t unit = kPartThreads * n;           // elements one chunk per thread covers
+  const int64_t row_bytes = cols * elem_size;
+  int64_t part = 0;
+  if (block_cols > 0) {
+    part = (block_cols + n - 1) / n * n;
+    if (part > 8 * unit) part = 8 * unit;
+    if (part >= cols) part = cols;                 // one part: still the two-pass form the caller asked for
+  } else if (row_bytes > (128 << 10) || (rows * 2 < cus && row_bytes >= (32 << 10))) {
+    int64_t bytes = cus > 0 ? row_bytes * rows / (2 * (int64_t)cus) : 0;
+    bytes = bytes < 4096 ? 4096 : (bytes > 16384 ? 16384 : bytes);
+    part = (bytes + 4095) / 4096 * 4096 / elem_size;
+  } else {
+    return r;
+  }
+  r.part_cols = part;
+  r.parts = (cols + part - 1) / part;
+  const int64_t per_thread = (part + unit - 1) / unit;
+  r.chunks = per_thread <= 1 ? 1 : per_thread <= 2 ? 2 : per_thread <= 4 ? 4 : 8;
+  if (rows * r.parts > 0x7fffffff) r = {0, 0, 0};
+  return r;
+}
+
+template <typename T, int OP, int CHUNKS>
+int launch_split(const RowSplit& sp, const T* x, T* y, const T* w, const T* b, float* mean, float* rstd, int64_t rows,
+                 int64_t cols, int64_t ld_x, int64_t ld_y, float eps, float* stats, hipStream_t s) {
+  const dim3 grid((unsigned)(rows * sp.parts));
+  hipLaunchKernelGGL((part_stats_kernel<T, OP, CHUNKS>), grid, dim3(kPartThreads), 0, s, x, stats, cols, ld_x,
+                     sp.part_cols, sp.parts);
+  hipLaunchKernelGGL((part_apply_kernel<T, OP, CHUNKS>), grid, dim3(kPartThreads), 0, s, x, y, w, b, mean, rstd, stats,
+                     cols, ld_x, ld_y, sp.part_cols, sp.parts, eps);
+  return launch_status();
+}
+
 // Grid of a pipelined launch: about 32 KiB of loads in flight per CU (2048 / CHUNKS threads, each with CHUNKS
 // 16-byte loads outstanding) measured fastest on MI355X: more resident workgroups shorten each one's walk and
 // bring the load / reduce / store phases back, fewer leave HBM idle. A problem too small for every workgroup to
@@ -402,7 +621,8 @@ int launch_tile(const T* x, T* y, const T* w, const T* b, float* mean, float* rs
 
 template <typename T, int OP>
 int dispatch_rows(const void* xv, void* yv, const void* wv, const void* bv, float* mean, float* rstd,
-                  int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s) {
+                  int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s,
+                  int64_t block_cols = 0, void* workspace = nullptr, int64_t workspace_bytes = 0) {
   const T* x = static_cast<const T*>(xv);
   T* y = static_cast<T*>(yv);
   const T* w = static_cast<const T*>(wv);
@@ -410,6 +630,19 @@ int dispatch_rows(const void* xv, void* yv, const void* wv, const void* bv, floa
   constexpr int N = 16 / sizeof(T);
   const bool vec_ok = cols % N == 0 && ld_x % N == 0 && ld_y % N == 0 && aligned_to(x, 16) && aligned_to(y, 16) &&
                       (!w || aligned_to(w, 16)) && (!b || aligned_to(b, 16));
+  if (vec_ok && workspace && aligned_to(workspace, 4)) {
+    const RowSplit sp = plan_row_split(rows, cols, block_cols, (int)sizeof(T), hexmi_num_cus());
+    if (sp.part_cols > 0) {
+      if (workspace_bytes < rows * sp.parts * 8) return HEXMI_EINVAL;
+      float* stats = static_cast<float*>(workspace);
+#define HEXMI_SPLIT(C) return launch_split<T, OP, C>(sp, x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, stats, s)
+      if (sp.chunks == 1) HEXMI_SPLIT(1);
+      if (sp.chunks == 2) HEXMI_SPLIT(2);
+      if (sp.chunks == 4) HEXMI_SPLIT(4);
+      HEXMI_SPLIT(8);
+#undef HEXMI_SPLIT
+    }
+  }
   const int64_t chunks = (cols + N - 1) / N;        // 16-byte chunks per row
   // softmax over many rows runs a little faster with half the usual loads in flight (one 256-thread workgroup per
   // CU at 1024 fp32 columns: 0.760 against 0.748 of the HBM figure at [65536,1024], A/B); the norms and small
@@ -437,11 +670,12 @@ int dispatch_rows(const void* xv, void* yv, const void* wv, const void* bv, floa
 
 template <int OP>
 int dispatch_dtype(int dtype, const void* x, void* y, const void* w, const void* b, float* mean, float* rstd,
-                   int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s) {
+                   int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps, hipStream_t s,
+                   int64_t block_cols = 0, void* ws = nullptr, int64_t ws_bytes = 0) {
   switch (dtype) {
-    case HEXMI_F32: return dispatch_rows<float, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s);
-    case HEXMI_F16: return dispatch_rows<f16, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s);
-    case HEXMI_BF16: return dispatch_rows<bf16, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s);
+    case HEXMI_F32: return dispatch_rows<float, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s, block_cols, ws, ws_bytes);
+    case HEXMI_F16: return dispatch_rows<f16, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s, block_cols, ws, ws_bytes);
+    case HEXMI_BF16: return dispatch_rows<bf16, OP>(x, y, w, b, mean, rstd, rows, cols, ld_x, ld_y, eps, s, block_cols, ws, ws_bytes);
     default: return HEXMI_ENOTSUP;
   }
 }
@@ -480,4 +714,47 @@ extern "C" int hexmi_layer_norm(const void* x, const void* weight, const void* b
   begin_call();
   return dispatch_dtype<kLayerNorm>(dtype, x, y, weight, bias, mean, rstd, rows, cols, cols, cols, eps,
                                     as_stream(stream));
+}
+
+// ---- the same operators with leading dimensions, a column-block size and a workspace ------------------------------
+
+extern "C" int64_t hexmi_row_workspace(int64_t rows, int64_t cols, int64_t block_cols, int dtype) {
+  const int esz = dtype_size(dtype);
+  if (rows <= 0 || cols <= 0 || block_cols < 0 || esz < 2) return 0;
+  const RowSplit sp = plan_row_split(rows, cols, block_cols, esz, hexmi_num_cus());
+  return sp.part_cols > 0 ? rows * sp.parts * 8 : 0;
+}
+
+extern "C" int hexmi_softmax_ws(const void* x, void* y, int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y,
+                                int64_t block_cols, int dtype, void* workspace, int64_t workspace_bytes,
+                                hexmi_stream_t stream) {
+  if (rows < 0 || cols < 0 || ld_x < cols || ld_y < cols || block_cols < 0 || workspace_bytes < 0) return HEXMI_EINVAL;
+  if (rows == 0 || cols == 0) return HEXMI_OK;
+  if (!x || !y) return HEXMI_EINVAL;
+  begin_call();
+  return dispatch_dtype<kSoftmax>(dtype, x, y, nullptr, nullptr, nullptr, nullptr, rows, cols, ld_x, ld_y, 0.0f,
+                                  as_stream(stream), block_cols, workspace, workspace_bytes);
+}
+
+extern "C" int hexmi_rms_norm_ws(const void* x, const void* weight, void* y, int64_t rows, int64_t cols, int64_t ld_x,
+                                 int64_t ld_y, float eps, int64_t block_cols, int dtype, void* workspace,
+                                 int64_t workspace_bytes, hexmi_stream_t stream) {
+  if (rows < 0 || cols < 0 || ld_x < cols || ld_y < cols || block_cols < 0 || workspace_bytes < 0) return HEXMI_EINVAL;
+  if (rows == 0 || cols == 0) return HEXMI_OK;
+  if (!x || !y) return HEXMI_EINVAL;
+  begin_call();
+  return dispatch_dtype<kRmsNorm>(dtype, x, y, weight, nullptr, nullptr, nullptr, rows, cols, ld_x, ld_y, eps,
+                                  as_stream(stream), block_cols, workspace, workspace_bytes);
+}
+
+extern "C" int hexmi_layer_norm_ws(const void* x, const void* weight, const void* bias, void* y, float* mean,
+                                   float* rstd, int64_t rows, int64_t cols, int64_t ld_x, int64_t ld_y, float eps,
+                                   int64_t block_cols, int dtype, void* workspace, int64_t workspace_bytes,
+                                   hexmi_stream_t stream) {
+  if (rows < 0 || cols < 0 || ld_x < cols || ld_y < cols || block_cols < 0 || workspace_bytes < 0) return HEXMI_EINVAL;
+  if (rows == 0 || cols == 0) return HEXMI_OK;
+  if (!x || !y) return HEXMI_EINVAL;
+  begin_call();
+  return dispatch_dtype<kLayerNorm>(dtype, x, y, weight, bias, mean, rstd, rows, cols, ld_x, ld_y, eps,
+                                    as_stream(stream), block_cols, workspace, workspace_bytes);
 }

@@ -31,6 +31,11 @@ SIGNATURES = {
     "hexmi_softmax": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _int, _ptr]),
     "hexmi_rms_norm": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _f32, _int, _ptr]),
     "hexmi_layer_norm": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _f32, _int, _ptr]),
+    "hexmi_row_workspace": (_i64, [_i64, _i64, _i64, _int]),
+    "hexmi_softmax_ws": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _i64, _int, _ptr, _i64, _ptr]),
+    "hexmi_rms_norm_ws": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _i64, _int, _ptr, _i64, _ptr]),
+    "hexmi_layer_norm_ws": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _i64, _int, _ptr,
+                                   _i64, _ptr]),
     "hexmi_matmul_f16f16_f32": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_gemm": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _int, _int, _ptr]),
     "hexmi_gemm_ex": (_int, [_i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _i64, _int, _int, _int,

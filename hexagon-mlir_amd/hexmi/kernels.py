@@ -64,10 +64,16 @@ def softmax_kernel(x_ptr, output_ptr, NUM_ROWS, NUM_COLS, BLOCK_SIZE=None):
 
 
 @Kernel
-def online_softmax(x_ptr, output_ptr, NUM_ROWS, NUM_COLS, BLOCK_SIZE=None):
-    """test/python/triton/test_online_softmax.py:31-81: same result as softmax_kernel."""
+def online_softmax(x_ptr, output_ptr, NUM_ROWS, NUM_COLS, BLOCK_ROW_SIZE=None, BLOCK_COL_SIZE=None):
+    """test/python/triton/test_online_softmax.py:31-81: the two-phase softmax over column blocks of BLOCK_COL_SIZE
+    (running max and sum per row, then the normalising sweep). Here every column block of a row is reduced by a
+    workgroup of its own and the (max, sum) pairs are merged with the same recurrence; BLOCK_ROW_SIZE, the rows of a
+    program, has no counterpart (the grid covers all rows)."""
     _check_2d("online_softmax", x_ptr, NUM_ROWS, NUM_COLS)
-    ops.softmax(x_ptr.view(NUM_ROWS, NUM_COLS), out=output_ptr.view(NUM_ROWS, NUM_COLS))
+    block = int(BLOCK_COL_SIZE) if BLOCK_COL_SIZE else NUM_COLS
+    if block <= 0 or NUM_COLS % block != 0:
+        raise ValueError("BLOCK_COL_SIZE must divide NUM_COLS")
+    ops.softmax(x_ptr.view(NUM_ROWS, NUM_COLS), out=output_ptr.view(NUM_ROWS, NUM_COLS), block_cols=block)
 
 
 @Kernel

@@ -86,31 +86,46 @@ _LIBDEF.define("rope(Tensor x, float theta, Tensor(a!) out) -> ()")
 _LIBDEF.define("attention(Tensor q, Tensor k, Tensor v, Tensor? mask, float sm_scale, Tensor(a!) out) -> ()")
 
 
-def _softmax_impl(x, out, rows=None, cols=None):
+def _row_workspace(rows, cols, block_cols, x):
+    """Scratch for the row operators' split form (rows cut into column blocks that several workgroups reduce): the
+    library says how much the shape takes, 0 when its single-pass kernels run anyway."""
+    need = _lib.lib().hexmi_row_workspace(rows, cols, block_cols, _dt(x))
+    return (torch.empty(need, dtype=torch.uint8, device=x.device), need) if need else (None, 0)
+
+
+def _row_geometry(x, out, rows, cols):
+    """(rows, cols, ld_x, ld_out): 2-D tensors whose rows are contiguous may be strided views (ld = row stride);
+    anything else is contiguous with rows and cols given."""
+    if rows is None:
+        rows, cols = x.shape
+        return rows, cols, x.stride(0), out.stride(0)
+    return rows, cols, cols, cols
+
+
+def _softmax_impl(x, out, rows=None, cols=None, block_cols=0):
     """x, out: [rows, cols]; or contiguous tensors of any rank with rows and cols given (no view objects built)."""
-    if rows is None:
-        rows, cols = x.shape
-        ldx, ldo = x.stride(0), out.stride(0)
-    else:
-        ldx = ldo = cols
+    rows, cols, ldx, ldo = _row_geometry(x, out, rows, cols)
     with _on(x.device):
-        _lib.check(_lib.lib().hexmi_softmax(_p(x), _p(out), rows, cols, ldx, ldo, _dt(x), _stream()), "hexmi_softmax")
+        ws, need = _row_workspace(rows, cols, block_cols, x)
+        _lib.check(_lib.lib().hexmi_softmax_ws(_p(x), _p(out), rows, cols, ldx, ldo, block_cols, _dt(x), _p(ws), need,
+                                               _stream()), "hexmi_softmax_ws")
 
 
-def _rms_norm_impl(x, weight, eps, out, rows=None, cols=None):
-    if rows is None:
-        rows, cols = x.shape
+def _rms_norm_impl(x, weight, eps, out, rows=None, cols=None, block_cols=0):
+    rows, cols, ldx, ldo = _row_geometry(x, out, rows, cols)
     with _on(x.device):
-        _lib.check(_lib.lib().hexmi_rms_norm(_p(x), _p(weight), _p(out), rows, cols, eps, _dt(x), _stream()),
-                   "hexmi_rms_norm")
+        ws, need = _row_workspace(rows, cols, block_cols, x)
+        _lib.check(_lib.lib().hexmi_rms_norm_ws(_p(x), _p(weight), _p(out), rows, cols, ldx, ldo, eps, block_cols,
+                                                _dt(x), _p(ws), need, _stream()), "hexmi_rms_norm_ws")
 
 
-def _layer_norm_impl(x, weight, bias, eps, out, mean, rstd, rows=None, cols=None):
-    if rows is None:
-        rows, cols = x.shape
+def _layer_norm_impl(x, weight, bias, eps, out, mean, rstd, rows=None, cols=None, block_cols=0):
+    rows, cols, ldx, ldo = _row_geometry(x, out, rows, cols)
     with _on(x.device):
-        _lib.check(_lib.lib().hexmi_layer_norm(_p(x), _p(weight), _p(bias), _p(out), _p(mean), _p(rstd), rows, cols,
-                                               eps, _dt(x), _stream()), "hexmi_layer_norm")
+        ws, need = _row_workspace(rows, cols, block_cols, x)
+        _lib.check(_lib.lib().hexmi_layer_norm_ws(_p(x), _p(weight), _p(bias), _p(out), _p(mean), _p(rstd), rows, cols,
+                                                  ldx, ldo, eps, block_cols, _dt(x), _p(ws), need, _stream()),
+                   "hexmi_layer_norm_ws")
 
 
 def _matmul_impl(a, b, trans_b, out):
@@ -278,49 +293,66 @@ def _out_like(out, shape, dtype, dev):
 # public operators. They call the implementations above directly: the same code `torch.ops.hexmi.*` runs, without
 # the dispatcher's round trip into Python (several microseconds, more than the shortest kernels here take).
 # --------------------------------------------------------------------------
-def softmax(x, out=None, dim=-1):
+def _row_strided(t):
+    """A 2-D device tensor whose rows are contiguous but not adjacent (a column slice, a padded buffer): the row
+    operators read and write it in place through its row stride, as the reference's kernels take a memref with
+    strides (test/utils/dsp/include/common.h:15-21)."""
+    return (t is not None and t.device.type == "cuda" and t.dim() == 2 and t.stride(1) == 1
+            and t.stride(0) >= t.shape[1] and not t.is_contiguous())
+
+
+def _row_operands(x, out, dev):
+    """(x on the device, tensor to compute into, rows, cols) with rows / cols None when both are 2-D strided views."""
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    if _row_strided(x) or (_row_strided(out) and x.dim() == 2):
+        xd = x if x.device.type == "cuda" and x.dim() == 2 and x.stride(1) == 1 else _stage(x, dev)
+        if out is not None and (tuple(out.shape) != tuple(x.shape) or out.dtype != x.dtype):
+            raise ValueError("hexmi: out must have the shape and dtype of x")
+        od = out if (out is not None and out.device.type == "cuda" and out.stride(1) == 1) else torch.empty_like(xd, memory_format=torch.contiguous_format)
+        return xd, od, None, None
+    return _stage(x, dev), _out_like(out, x.shape, x.dtype, dev), rows, cols
+
+
+def softmax(x, out=None, dim=-1, block_cols=0):
     """Softmax over the last dimension (`F.softmax(x, dim=1)` of
-    test/python/triton/test_softmax.py:93 for 2-D input)."""
+    test/python/triton/test_softmax.py:93 for 2-D input). block_cols > 0: the two-phase (online) form of
+    test/python/triton/test_online_softmax.py:31-81 over column blocks of that size."""
     if dim not in (-1, x.dim() - 1):
         raise ValueError("hexmi.softmax reduces over the last dimension only")
     if x.dim() < 1:
         raise ValueError("hexmi.softmax needs at least 1 dimension")
     dev = _device() if x.device.type != "cuda" else x.device
-    xd = _stage(x, dev)
-    od = _out_like(out, x.shape, x.dtype, dev)
-    cols = x.shape[-1]
-    rows = x.numel() // max(cols, 1)
-    _softmax_impl(xd, od, rows, cols)
+    xd, od, rows, cols = _row_operands(x, out, dev)
+    _softmax_impl(xd, od, rows, cols, int(block_cols))
     return _finish(od, out)
 
 
-def rms_norm(x, weight=None, eps=1e-5, out=None):
+def rms_norm(x, weight=None, eps=1e-5, out=None, block_cols=0):
     """`F.rms_norm(x, (C,), weight, eps)` (test/python/triton/test_rms_norm.py:85-87)."""
     dev = _device() if x.device.type != "cuda" else x.device
     cols = x.shape[-1]
-    rows = x.numel() // max(cols, 1)
     if weight is not None and (weight.shape != (cols,) or weight.dtype != x.dtype):
         raise ValueError("hexmi.rms_norm: weight must be [%d] of %s" % (cols, x.dtype))
-    xd, wd = _stage(x, dev), _stage(weight, dev)
-    od = _out_like(out, x.shape, x.dtype, dev)
-    _rms_norm_impl(xd, wd, float(eps), od, rows, cols)
+    xd, od, rows, c = _row_operands(x, out, dev)
+    _rms_norm_impl(xd, _stage(weight, dev), float(eps), od, rows, c, int(block_cols))
     return _finish(od, out)
 
 
-def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=None):
+def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=None, block_cols=0):
     """`F.layer_norm(x, (C,), weight, bias, eps)` (test/python/triton/test_layer_norm.py:111-113);
     `mean` / `rstd` (fp32, one per row) are filled when given, as the reference kernel does."""
     dev = _device() if x.device.type != "cuda" else x.device
     cols = x.shape[-1]
-    rows = x.numel() // max(cols, 1)
+    nrows = x.numel() // max(cols, 1)
     for name, t in (("weight", weight), ("bias", bias)):
         if t is not None and (t.shape != (cols,) or t.dtype != x.dtype):
             raise ValueError("hexmi.layer_norm: %s must be [%d] of %s" % (name, cols, x.dtype))
-    xd, wd, bd = _stage(x, dev), _stage(weight, dev), _stage(bias, dev)
-    od = _out_like(out, x.shape, x.dtype, dev)
-    md = None if mean is None else _out_like(mean if mean.dtype == torch.float32 else None, (rows,), torch.float32, dev)
-    rd = None if rstd is None else _out_like(rstd if rstd.dtype == torch.float32 else None, (rows,), torch.float32, dev)
-    _layer_norm_impl(xd, wd, bd, float(eps), od, md, rd, rows, cols)
+    xd, od, rows, c = _row_operands(x, out, dev)
+    wd, bd = _stage(weight, dev), _stage(bias, dev)
+    md = None if mean is None else _out_like(mean if mean.dtype == torch.float32 else None, (nrows,), torch.float32, dev)
+    rd = None if rstd is None else _out_like(rstd if rstd.dtype == torch.float32 else None, (nrows,), torch.float32, dev)
+    _layer_norm_impl(xd, wd, bd, float(eps), od, md, rd, rows, c, int(block_cols))
     if mean is not None:
         _finish(md, mean)
     if rstd is not None:

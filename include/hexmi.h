@@ -88,6 +88,47 @@ int hexmi_layer_norm(const void *x, const void *weight, const void *bias,
                      void *y, float *mean, float *rstd, int64_t rows,
                      int64_t cols, float eps, int dtype, hexmi_stream_t stream);
 
+/* The three row operators with the operands a ranked memref carries and the
+ * block size the reference kernels are launched with:
+ *  - ld_x / ld_y: elements between consecutive rows (>= cols), as the strides
+ *    of the reference's MemRefDescriptor (test/utils/dsp/include/common.h:15-21);
+ *  - block_cols: the column block of the kernels' sweeps (BLOCK_SIZE of
+ *    test_rms_norm.py:37-63 and test_layer_norm.py:42-82, BLOCK_COL_SIZE of
+ *    test/python/triton/test_online_softmax.py:31-81). > 0: every block of
+ *    block_cols columns (rounded up to whole 16-byte runs, at most 32 KiB) is
+ *    reduced by a workgroup of its own and the per-block statistics are merged:
+ *    (max, sum) pairs with the online recurrence of test_online_softmax.py:60-71,
+ *    sums of squares, (mean, M2) pairs. 0: the library decides; it splits rows
+ *    longer than 128 KiB and problems of fewer rows than half the compute units
+ *    whose rows are 32 KiB or longer (the reference's own long-row case is
+ *    4 x 65536, test_softmax_scf_multithread.py:19-24; its compiler splits such
+ *    reductions over its threads, lib/Conversion/LinalgToLLVM/
+ *    SplitReduceGenericPass.cpp), everything else runs the single-pass kernels;
+ *  - workspace: fp32 scratch for the per-block statistics of the split form.
+ *    hexmi_row_workspace returns the bytes (rows, cols, block_cols, dtype)
+ *    take, 0 when the single-pass kernels run. workspace may be NULL (single
+ *    pass whatever the shape, up to 128 KiB per row at full speed); one that is
+ *    smaller than the query's answer is HEXMI_EINVAL. No initialisation, no
+ *    state between calls. Rows, leading dims or pointers that are not
+ *    16-byte aligned also run the single-pass kernels.
+ * Same results as hexmi_softmax / hexmi_rms_norm / hexmi_layer_norm up to the
+ * rounding of the merged statistics. */
+int64_t hexmi_row_workspace(int64_t rows, int64_t cols, int64_t block_cols,
+                            int dtype);
+int hexmi_softmax_ws(const void *x, void *y, int64_t rows, int64_t cols,
+                     int64_t ld_x, int64_t ld_y, int64_t block_cols, int dtype,
+                     void *workspace, int64_t workspace_bytes,
+                     hexmi_stream_t stream);
+int hexmi_rms_norm_ws(const void *x, const void *weight, void *y, int64_t rows,
+                      int64_t cols, int64_t ld_x, int64_t ld_y, float eps,
+                      int64_t block_cols, int dtype, void *workspace,
+                      int64_t workspace_bytes, hexmi_stream_t stream);
+int hexmi_layer_norm_ws(const void *x, const void *weight, const void *bias,
+                        void *y, float *mean, float *rstd, int64_t rows,
+                        int64_t cols, int64_t ld_x, int64_t ld_y, float eps,
+                        int64_t block_cols, int dtype, void *workspace,
+                        int64_t workspace_bytes, hexmi_stream_t stream);
+
 /* Dense GEMM ------------------------------------------------------------- */
 
 /* out[n_row, n_col] (fp32) = act[n_row, n_inner] (fp16) * w[n_inner, n_col]

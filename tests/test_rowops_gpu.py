@@ -74,9 +74,13 @@ def test_softmax_host_tensors_in_place(hexmi, oracle):
                                        enableHVXInlining=True, enableSCFLoopUnroll=True,
                                        enableSplitReduceGeneric=True)
     assert torch.allclose(out, torch.from_numpy(oracle.softmax(x.numpy())), atol=1e-5)   # test_softmax.py ATOL_FP32
+    # test_online_softmax.py:84-113: four programs, BLOCK_ROW_SIZE = BLOCK_COL_SIZE = 32, ATOL 1e-5
     out2 = torch.empty_like(x)
-    hexmi.kernels.online_softmax[(4,)](x, out2, NUM_ROWS=128, NUM_COLS=128, BLOCK_SIZE=32)
-    assert torch.equal(out, out2)
+    hexmi.kernels.online_softmax[(4,)](x, out2, NUM_ROWS=128, NUM_COLS=128, BLOCK_ROW_SIZE=32, BLOCK_COL_SIZE=32,
+                                       enableMultiThreading=False, enableVTCMTiling=False,
+                                       enableConvertToHexagonmem=False, enableHexagonmemCopyToDMA=False)
+    assert torch.allclose(out2, torch.from_numpy(oracle.online_softmax_f32(x.numpy(), 32)), rtol=F32_RTOL, atol=1e-9)
+    assert torch.allclose(out2, out, rtol=F32_RTOL, atol=1e-9)
 
 
 def test_softmax_extreme_values(hexmi):
@@ -204,3 +208,146 @@ def test_empty_inputs(hexmi):
     assert hexmi.softmax(torch.empty(0, 16, device="cuda")).shape == (0, 16)
     assert hexmi.rms_norm(torch.empty(0, 16, device="cuda", dtype=torch.float16)).shape == (0, 16)
     assert hexmi.layer_norm(torch.empty(4, 0, device="cuda")).shape == (4, 0)
+
+
+# ---- rows split over several workgroups (the online / split-reduction form) ------------------------------------
+
+# shapes the library splits by itself: few long rows (the reference's 4 x 65536 of
+# test_softmax_scf_multithread.py:19-24) and rows beyond 128 KiB, whole and ragged last parts
+SPLIT_SHAPES = [(torch.float32, 4, 65536), (torch.float16, 4, 65536), (torch.float32, 16, 131072),
+                (torch.float32, 1, 1 << 20), (torch.float16, 3, 40000), (torch.float32, 2, 100004),
+                (torch.bfloat16, 5, 70000), (torch.float32, 300, 40000)]
+
+
+@pytest.mark.parametrize("dtype,rows,cols", SPLIT_SHAPES)
+def test_split_rows_parity(hexmi, oracle, dtype, rows, cols):
+    assert hexmi.lib().hexmi_row_workspace(rows, cols, 0, hexmi.ops._dt(torch.empty(0, dtype=dtype))) > 0
+    g = _gen(21)
+    x = (torch.randn(rows, cols, generator=g) * 2 + 0.25).to(dtype)
+    w = (1 + 0.1 * torch.randn(cols, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(cols, generator=g)).to(dtype)
+    a, tag = to_np(x)
+    wn, _ = to_np(w)
+    bn, _ = to_np(b)
+    xd, wd, bd = x.cuda(), w.cuda(), b.cuda()
+    _check(hexmi.softmax(xd), from_np(oracle.softmax(a, dtype=tag), dtype), dtype, atol16=1e-7, atol32=1e-12)
+    _check(hexmi.rms_norm(xd, wd, 1e-5), from_np(oracle.rms_norm(a, wn, 1e-5, dtype=tag), dtype), dtype)
+    want, mean, rstd = oracle.layer_norm(a, wn, bn, 1e-5, dtype=tag)
+    m = torch.full((rows,), float("nan"), device="cuda")
+    r = torch.full((rows,), float("nan"), device="cuda")
+    got = hexmi.layer_norm(xd, wd, bd, 1e-5, mean=m, rstd=r)
+    _check(got, from_np(want, dtype), dtype, atol16=2e-6, atol32=2e-6)
+    assert torch.allclose(m.cpu(), torch.from_numpy(mean), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(r.cpu(), torch.from_numpy(rstd), rtol=1e-5)
+    # rows sum to one; a shift of the row changes nothing (softmax), nor does it change LayerNorm
+    sm = hexmi.softmax(xd).float().sum(-1).cpu()
+    assert torch.allclose(sm, torch.ones(rows), atol=2e-3 if dtype != torch.float32 else 1e-5)
+
+
+@pytest.mark.parametrize("dtype,rows,cols,block", [(torch.float32, 128, 128, 32), (torch.float32, 37, 520, 24),
+                                                   (torch.float16, 37, 520, 24), (torch.float32, 5, 4096, 1000),
+                                                   (torch.float16, 64, 8192, 2048), (torch.bfloat16, 9, 1024, 1024),
+                                                   (torch.float32, 6, 100000, 100000)])
+def test_forced_column_blocks(hexmi, oracle, dtype, rows, cols, block):
+    g = _gen(22)
+    x = (torch.randn(rows, cols, generator=g) * 3).to(dtype)
+    w = (1 + 0.1 * torch.randn(cols, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(cols, generator=g)).to(dtype)
+    a, tag = to_np(x)
+    wn, _ = to_np(w)
+    bn, _ = to_np(b)
+    xd = x.cuda()
+    got = hexmi.softmax(xd, block_cols=block)
+    _check(got, from_np(oracle.softmax(a, dtype=tag), dtype), dtype, atol16=1e-7, atol32=1e-12)
+    if dtype == torch.float32 and cols % block == 0 and cols <= 8192:
+        # the reference's two-phase algorithm restated with the same block size (its fp32 running sums, so short rows)
+        assert torch.allclose(got.cpu(), torch.from_numpy(oracle.online_softmax_f32(a, block)), rtol=F32_RTOL, atol=1e-12)
+    _check(hexmi.rms_norm(xd, w.cuda(), 1e-5, block_cols=block), from_np(oracle.rms_norm(a, wn, 1e-5, dtype=tag), dtype), dtype)
+    want, mean, rstd = oracle.layer_norm(a, wn, bn, 1e-5, dtype=tag)
+    m = torch.empty(rows, device="cuda")
+    r = torch.empty(rows, device="cuda")
+    got = hexmi.layer_norm(xd, w.cuda(), b.cuda(), 1e-5, mean=m, rstd=r, block_cols=block)
+    _check(got, from_np(want, dtype), dtype, atol16=2e-6, atol32=2e-6)
+    assert torch.allclose(m.cpu(), torch.from_numpy(mean), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(r.cpu(), torch.from_numpy(rstd), rtol=1e-5)
+
+
+def test_split_softmax_rows_of_minus_infinity(hexmi):
+    # whole column blocks of -inf (masked scores): they add nothing; a row of nothing else is NaN, as torch gives
+    x = torch.randn(3, 65536, generator=_gen(23))
+    x[0, :40000] = -float("inf")
+    x[1, 1024:] = -float("inf")
+    x[2, :] = -float("inf")
+    got = hexmi.softmax(x.cuda()).cpu()
+    want = torch.softmax(x.double(), -1).float()
+    assert torch.allclose(got[:2], want[:2], rtol=F32_RTOL, atol=1e-12)
+    assert torch.isnan(got[2]).all() and torch.isnan(want[2]).all()
+
+
+@pytest.mark.parametrize("split", [False, True])
+def test_norms_on_strided_rows(hexmi, oracle, split):
+    # rows inside wider buffers (leading dimension > cols), read and written in place
+    rows, cols, ld = (4, 65536, 65536 + 64) if split else (33, 512, 768)
+    g = _gen(24)
+    x = torch.randn(rows, cols, generator=g).half()
+    w = (1 + 0.1 * torch.randn(cols, generator=g)).half()
+    b = (0.1 * torch.randn(cols, generator=g)).half()
+    big = torch.zeros(rows, ld, dtype=torch.float16, device="cuda")
+    big[:, :cols] = x.cuda()
+    out = torch.full((rows, ld), -1.0, dtype=torch.float16, device="cuda")
+    hexmi.rms_norm(big[:, :cols], w.cuda(), 1e-5, out=out[:, :cols])
+    assert close16(out[:, :cols].cpu(), torch.from_numpy(oracle.rms_norm(x.numpy(), w.numpy(), 1e-5)), 1, 1e-6)
+    assert (out[:, cols:] == -1.0).all()
+    out.fill_(-1.0)
+    m = torch.empty(rows, device="cuda")
+    r = torch.empty(rows, device="cuda")
+    hexmi.layer_norm(big[:, :cols], w.cuda(), b.cuda(), 1e-5, out=out[:, :cols], mean=m, rstd=r)
+    want, mean, rstd = oracle.layer_norm(x.numpy(), w.numpy(), b.numpy(), 1e-5)
+    assert close16(out[:, :cols].cpu(), torch.from_numpy(want), 1, 2e-6)
+    assert (out[:, cols:] == -1.0).all()
+    assert torch.allclose(m.cpu(), torch.from_numpy(mean), rtol=1e-5, atol=1e-6)
+    out.fill_(-1.0)
+    hexmi.softmax(big[:, :cols], out=out[:, :cols])
+    assert close16(out[:, :cols].cpu(), torch.from_numpy(oracle.softmax(x.numpy())), 1, 1e-7)
+    assert (out[:, cols:] == -1.0).all()
+
+
+def test_row_workspace_contract(hexmi):
+    lib = hexmi.lib()
+    F32 = hexmi._lib.F32
+    assert lib.hexmi_row_workspace(4096, 1024, 0, F32) == 0           # single pass
+    assert lib.hexmi_row_workspace(4096, 1024, 256, F32) == 4096 * 4 * 8
+    need = lib.hexmi_row_workspace(4, 65536, 0, F32)
+    assert need > 0 and need % (4 * 8) == 0
+    x = torch.randn(4, 65536, device="cuda")
+    y = torch.empty_like(x)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.hexmi_softmax_ws(x.data_ptr(), y.data_ptr(), 4, 65536, 65536, 65536, 0, F32, ws.data_ptr(), need - 1, st) \
+        == hexmi._lib.EINVAL
+    assert lib.hexmi_softmax_ws(x.data_ptr(), y.data_ptr(), 4, 65536, 65536, 65536, 0, F32, ws.data_ptr(), need, st) == 0
+    y2 = torch.empty_like(x)
+    assert lib.hexmi_softmax_ws(x.data_ptr(), y2.data_ptr(), 4, 65536, 65536, 65536, 0, F32, None, 0, st) == 0
+    torch.cuda.synchronize()
+    assert torch.allclose(y, y2, rtol=F32_RTOL, atol=1e-12)
+    assert lib.hexmi_softmax_ws(x.data_ptr(), y.data_ptr(), 4, 65536, 100, 65536, 0, F32, None, 0, st) == hexmi._lib.EINVAL
+
+
+def test_norm_statistics_at_the_edges_of_the_range(hexmi):
+    # a sum of squares that overflows (rstd = 0), a row of zeros with eps = 0 (rstd = inf): what torch gives
+    import torch.nn.functional as F
+    x = torch.zeros(4, 1024)
+    x[0] = 1e20
+    x[1] = torch.randn(1024, generator=_gen(25))
+    x[3] = 3.0                                                     # constant row: zero variance
+    for eps in (1e-5, 0.0):
+        got = hexmi.rms_norm(x.cuda(), None, eps).cpu()
+        want = F.rms_norm(x, (1024,), None, eps)
+        assert torch.allclose(got, want, rtol=1e-5, atol=1e-7, equal_nan=True)
+        m = torch.empty(4, device="cuda")
+        r = torch.empty(4, device="cuda")
+        got = hexmi.layer_norm(x.cuda(), None, None, eps, mean=m, rstd=r).cpu()
+        want = F.layer_norm(x, (1024,), None, None, eps)
+        assert torch.allclose(got[1:], want[1:], rtol=1e-5, atol=1e-6, equal_nan=True)
+        var = x.double().var(-1, unbiased=False)
+        assert torch.allclose(r.cpu()[1:].double(), 1.0 / torch.sqrt(var + eps)[1:], rtol=1e-5, equal_nan=True)
