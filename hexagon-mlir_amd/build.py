@@ -33,7 +33,7 @@ def _sources():
 
 def _headers_mtime():
     hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
-    hs.append(os.path.join(INCLUDE, "hexmi.h"))
+    hs += [os.path.join(INCLUDE, f) for f in os.listdir(INCLUDE) if f.endswith(".h")]
     return max(os.path.getmtime(h) for h in hs)
 
 

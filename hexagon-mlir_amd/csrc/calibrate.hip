@@ -6,6 +6,7 @@
 #include <type_traits>
 
 #include "hexmi_common.h"
+#include "hexmi_calibrate.h"
 
 namespace hexmi {
 namespace {
@@ -225,10 +226,10 @@ extern "C" double hexmi_mfma_peak_flops(int shape, int waves_per_simd, int64_t i
 
 extern "C" int hexmi_mfma_peak(int shape, int dtype, const void* operands, int64_t iters, int waves_per_simd,
                                float* sink, hexmi_stream_t stream) {
-  if (shape < 0 || shape > 2 || waves_per_simd < 1 || waves_per_simd > (shape == 2 ? 1 : 2) || iters < 0 ||
-      iters > 0x7fffffff)
+  if (shape < 0 || shape > 2 || waves_per_simd < 1 || waves_per_simd > (shape == 2 ? 1 : 2) || iters < 0)
     return HEXMI_EINVAL;
   if (!operands || !sink || !aligned_to(operands, 16)) return HEXMI_EINVAL;
+  if (iters > HEXMI_CALIBRATE_MAX_ITERS) return HEXMI_ETOOBIG;   // one launch holds every CU: keep it to about a minute
   const int cus = hexmi_num_cus();
   if (cus <= 0) return HEXMI_ELAUNCH;
   hipStream_t st = as_stream(stream);
@@ -255,8 +256,9 @@ extern "C" int hexmi_mfma_peak(int shape, int dtype, const void* operands, int64
 extern "C" int hexmi_issue_slots(int shape, int kind, int per_mfma, int64_t iters, int waves_per_simd, float* sink,
                                  hexmi_stream_t stream) {
   if ((shape != 0 && shape != 1) || kind < 0 || kind > 4 || waves_per_simd < 1 || waves_per_simd > 2 || iters < 0 ||
-      iters > 0x7fffffff || !sink)
+      !sink)
     return HEXMI_EINVAL;
+  if (iters > HEXMI_CALIBRATE_MAX_ITERS) return HEXMI_ETOOBIG;
   const int cus = hexmi_num_cus();
   if (cus <= 0) return HEXMI_ELAUNCH;
   hipStream_t st = as_stream(stream);
@@ -277,7 +279,8 @@ extern "C" int hexmi_issue_slots(int shape, int kind, int per_mfma, int64_t iter
 }
 
 extern "C" int hexmi_lds_read_pattern(int pattern, int64_t iters, float* sink, hexmi_stream_t stream) {
-  if (pattern < 0 || pattern > 6 || iters < 0 || iters > 0x7fffffff || !sink) return HEXMI_EINVAL;
+  if (pattern < 0 || pattern > 6 || iters < 0 || !sink) return HEXMI_EINVAL;
+  if (iters > HEXMI_CALIBRATE_MAX_ITERS) return HEXMI_ETOOBIG;
   const int cus = hexmi_num_cus();
   if (cus <= 0) return HEXMI_ELAUNCH;
   begin_call();

@@ -25,10 +25,14 @@ constexpr int kThreads = kWaves * kWave;
 // the whole grid is resident at once and nothing synchronises across tiles. Activation fragments are read
 // through L1/L2 (the activations are M*K*2 bytes, at most 128 KiB per 16 rows, shared by every workgroup).
 // MT: number of 16-row activation tiles handled per pass (rows m_base .. m_base + 16*MT).
-template <int MT>
+// ZP: the asymmetric forms of quant.dcast, f = (float(q) - zero_point) * scale with per-channel or per-tensor
+// parameters: the zero point (an int8, exact in fp16, as is every difference q - zero_point) is subtracted from the
+// widened weights; per_tensor reads scale and zero point at index 0 for every channel.
+template <int MT, bool ZP = false>
 __global__ __launch_bounds__(kThreads)
 void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
-                  f16* __restrict__ C, int M, int N, int K, int m_base) {
+                  f16* __restrict__ C, int M, int N, int K, int m_base, const int8_t* __restrict__ zero_points = nullptr,
+                  int per_tensor = 0) {
   __shared__ __attribute__((aligned(16))) float red[kWaves * MT * 256];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -37,6 +41,10 @@ void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const
   const int n = tile * 16 + r16;
   const int nc = n < N ? n : N - 1;
   const int8_t* wrow = W + (int64_t)nc * K + kg * 16;
+  f16 zp_h = (f16)0.0f;
+  if constexpr (ZP) {
+    if (zero_points) zp_h = (f16)(float)zero_points[per_tensor ? 0 : nc];
+  }
 
   const int steps = K / 64;
   const int per_wave = (steps + kWaves - 1) / kWaves;       // consecutive steps per wave: whole 128-byte lines
@@ -84,6 +92,10 @@ void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const
     for (int u = 0; u < U; ++u) {
       f16x8 w0, w1;
       cvt16(wv[u], w0, w1);                                 // a skipped step has zero weights and activations
+      if constexpr (ZP) {
+        w0 -= zp_h;                                         // exact: integers of magnitude <= 255
+        w1 -= zp_h;
+      }
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
@@ -107,7 +119,7 @@ void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const
     if (gm < M) {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (gn + e < N) C[(int64_t)gm * N + gn + e] = (f16)(sum[e] * (float)scales[gn + e]);
+        if (gn + e < N) C[(int64_t)gm * N + gn + e] = (f16)(sum[e] * (float)scales[ZP && per_tensor ? 0 : gn + e]);
     }
   }
 }
@@ -657,13 +669,25 @@ void dequant_kernel(const int8_t* __restrict__ W, const f16* __restrict__ scales
   }
 }
 
+__global__ __launch_bounds__(256)
+void dequant_ex_kernel(const int8_t* __restrict__ W, const f16* __restrict__ scales, const int8_t* __restrict__ zero_points,
+                       int per_tensor, float* __restrict__ out, int64_t N, int64_t K) {
+  const int64_t total = N * K;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t n = per_tensor ? 0 : i / K;
+    const float zp = zero_points ? (float)zero_points[n] : 0.0f;
+    out[i] = ((float)W[i] - zp) * (float)scales[n];    // the difference is an exact integer, then one fp32 multiply
+  }
+}
+
 // Any K and any alignment (the shapes the 16-byte-load kernels above do not take): one wave per output channel
 // and block of MR activation rows, lanes stride over k, fp32 multiply-add of the exact int8 -> fp32 and
 // fp16 -> fp32 values, butterfly sum, the channel scale on the finished sum as everywhere else.
 template <int MR>
 __global__ __launch_bounds__(256)
 void w8a16_generic_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
-                          f16* __restrict__ C, int M, int N, int K) {
+                          f16* __restrict__ C, int M, int N, int K, const int8_t* __restrict__ zero_points = nullptr,
+                          int per_tensor = 0) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = blockIdx.x * 4 + wave;
   const int m0 = blockIdx.y * MR;
@@ -672,13 +696,14 @@ void w8a16_generic_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
   float acc[MR];
 #pragma unroll
   for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+  const float zp = zero_points ? (float)zero_points[per_tensor ? 0 : n] : 0.0f;
   for (int k = lane; k < K; k += kWave) {
-    const float w = (float)wrow[k];
+    const float w = (float)wrow[k] - zp;
 #pragma unroll
     for (int m = 0; m < MR; ++m)
       if (m0 + m < M) acc[m] = fmaf((float)A[(int64_t)(m0 + m) * K + k], w, acc[m]);
   }
-  const float sc = (float)scales[n];
+  const float sc = (float)scales[per_tensor ? 0 : n];
 #pragma unroll
   for (int m = 0; m < MR; ++m) {
     const float tot = wave_sum(acc[m]);
@@ -691,6 +716,14 @@ int launch_pass(const f16* A, const int8_t* W, const f16* s, f16* C, int M, int 
                 hipStream_t st) {
   const int n_tiles = (N + 15) / 16;
   hipLaunchKernelGGL((w8a16_kernel<MT>), dim3(n_tiles), dim3(kThreads), 0, st, A, W, s, C, M, N, K, m_base);
+  return launch_status();
+}
+template <int MT>
+int launch_pass_zp(const f16* A, const int8_t* W, const f16* s, f16* C, int M, int N, int K, int m_base,
+                   const int8_t* zp, int per_tensor, hipStream_t st) {
+  const int n_tiles = (N + 15) / 16;
+  hipLaunchKernelGGL((w8a16_kernel<MT, true>), dim3(n_tiles), dim3(kThreads), 0, st, A, W, s, C, M, N, K, m_base, zp,
+                     per_tensor);
   return launch_status();
 }
 
@@ -903,4 +936,52 @@ extern "C" int hexmi_dequant_w8(int64_t N, int64_t K, const int8_t* W, const voi
   hipLaunchKernelGGL(dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), W,
                      static_cast<const f16*>(scales), out, N, K);
   return launch_status();
+}
+
+// ---- quant.dcast with a zero point and / or per-tensor parameters ------------------------------------------------
+
+extern "C" int hexmi_dequant_w8_ex(int64_t N, int64_t K, const int8_t* W, const void* scales, const int8_t* zero_points,
+                                   int per_tensor, float* out, hexmi_stream_t stream) {
+  if (N < 0 || K < 0) return HEXMI_EINVAL;
+  if (N == 0 || K == 0) return HEXMI_OK;
+  if (!W || !scales || !out) return HEXMI_EINVAL;
+  const int64_t total = N * K;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  begin_call();
+  hipLaunchKernelGGL(dequant_ex_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), W,
+                     static_cast<const f16*>(scales), zero_points, per_tensor ? 1 : 0, out, N, K);
+  return launch_status();
+}
+
+extern "C" int hexmi_gemm_w8a16_ex(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
+                                   const int8_t* zero_points, int per_tensor, void* C, hexmi_stream_t stream) {
+  if (!zero_points && !per_tensor) return hexmi_gemm_w8a16(M, N, K, A, W, scales, C, stream);   // the symmetric per-channel form
+  if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
+  if (M == 0 || N == 0) return HEXMI_OK;
+  if (!C || (K > 0 && (!A || !W || !scales))) return HEXMI_EINVAL;
+  if (M > 0x7fffffff || N > 0x7fffffff - 16 || K > 0x7fffffff) return HEXMI_ENOTSUP;
+  hipStream_t st = as_stream(stream);
+  const f16* a = static_cast<const f16*>(A);
+  const f16* s = static_cast<const f16*>(scales);
+  f16* c = static_cast<f16*>(C);
+  const int pt = per_tensor ? 1 : 0;
+  begin_call();
+  if (K == 0) return fill_zero_2d(C, M, N, N, 2, st);
+  if (K % 64 != 0 || !aligned_to(A, 16) || !aligned_to(W, 16)) {
+    constexpr int MR = 4;
+    const int64_t gy = (M + MR - 1) / MR;
+    if (gy > 65535) return HEXMI_ENOTSUP;
+    hipLaunchKernelGGL(w8a16_generic_kernel<MR>, dim3((unsigned)((N + 3) / 4), (unsigned)gy), dim3(256), 0, st, a, W, s,
+                       c, (int)M, (int)N, (int)K, zero_points, pt);
+    return launch_status();
+  }
+  int rc = HEXMI_OK;
+  for (int64_t m = 0; m < M && rc == HEXMI_OK; m += 64) {
+    const int64_t left = M - m;
+    if (left > 32) rc = launch_pass_zp<4>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zero_points, pt, st);
+    else if (left > 16) rc = launch_pass_zp<2>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zero_points, pt, st);
+    else rc = launch_pass_zp<1>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zero_points, pt, st);
+  }
+  return rc;
 }

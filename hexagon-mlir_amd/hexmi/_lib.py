@@ -23,7 +23,7 @@ class HexmiError(RuntimeError):
 _c = ctypes
 _i64, _int, _f32, _f64, _ptr = _c.c_int64, _c.c_int, _c.c_float, _c.c_double, _c.c_void_p
 
-# name -> (restype, argtypes); must list every symbol of include/hexmi.h
+# name -> (restype, argtypes); must list every symbol of include/hexmi.h (the operator ABI)
 SIGNATURES = {
     "hexmi_version": (_c.c_char_p, []),
     "hexmi_strerror": (_c.c_char_p, [_int]),
@@ -49,6 +49,8 @@ SIGNATURES = {
     "hexmi_pack_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr]),
     "hexmi_gemm_w8a16_packed": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "hexmi_dequant_w8": (_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "hexmi_dequant_w8_ex": (_int, [_i64, _i64, _ptr, _ptr, _ptr, _int, _ptr, _ptr]),
+    "hexmi_gemm_w8a16_ex": (_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _ptr]),
     "hexmi_flash_attn_fwd": (_int, [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _int, _ptr]),
     "hexmi_unary": (_int, [_int, _ptr, _ptr, _i64, _int, _ptr]),
     "hexmi_binary": (_int, [_int, _ptr, _ptr, _ptr, _i64, _int, _ptr]),
@@ -58,11 +60,15 @@ SIGNATURES = {
     "hexmi_block_sum_static_max_n": (_i64, []),
     "hexmi_block_sum_static": (_int, [_ptr, _ptr, _i64, _i64, _int, _ptr]),
     "hexmi_rope": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _f64, _int, _ptr]),
+    "hexmi_attention": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _ptr]),
+}
+
+# measurement probes of include/hexmi_calibrate.h: exported by the library, not part of the operator ABI
+PROBE_SIGNATURES = {
     "hexmi_mfma_peak_flops": (_f64, [_int, _int, _i64]),
     "hexmi_mfma_peak": (_int, [_int, _int, _ptr, _i64, _int, _ptr, _ptr]),
     "hexmi_issue_slots": (_int, [_int, _int, _int, _i64, _int, _ptr, _ptr]),
     "hexmi_lds_read_pattern": (_int, [_int, _i64, _ptr, _ptr]),
-    "hexmi_attention": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _f32, _int, _int, _ptr]),
 }
 
 _lib = None
@@ -77,7 +83,7 @@ def lib():
                 "libhexmi.so is missing at %s: build it with `python hexagon-mlir_amd/build.py` "
                 "(there is no CPU or eager fallback)" % LIB_PATH)
         handle = ctypes.CDLL(LIB_PATH)
-        for name, (res, args) in SIGNATURES.items():
+        for name, (res, args) in list(SIGNATURES.items()) + list(PROBE_SIGNATURES.items()):
             fn = getattr(handle, name)          # AttributeError if the symbol is not exported
             fn.restype, fn.argtypes = res, args
         _lib = handle

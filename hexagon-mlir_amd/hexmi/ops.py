@@ -410,16 +410,43 @@ def pack_weight(w):
     return out
 
 
-def w8a16_matmul(a, w_int8, scales, out=None):
-    """C[m,n] = sum_k A[m,k] * (W[n,k] * scales[n]); A fp16 [M,K], W int8 [N,K], scales fp16 [N]."""
-    if a.dtype != torch.float16 or w_int8.dtype != torch.int8 or scales.dtype != torch.float16:
+def _quant_params(name, w_int8, scales, zero_points):
+    """Checks the parameters of `f = (float(q) - zero_point) * scale`; returns per_tensor (one scale, and one zero
+    point, for the whole tensor) against per output channel."""
+    if w_int8.dtype != torch.int8 or scales.dtype != torch.float16:
+        raise TypeError("hexmi.%s: expected int8 weights, fp16 scales" % name)
+    if w_int8.dim() != 2 or scales.dim() != 1 or scales.shape[0] not in (1, w_int8.shape[0]):
+        raise ValueError("hexmi.%s: shapes W[N,K] and scales[N] (per channel) or scales[1] (per tensor) required" % name)
+    per_tensor = scales.shape[0] == 1 and w_int8.shape[0] != 1
+    if zero_points is not None:
+        if zero_points.dtype != torch.int8:
+            raise TypeError("hexmi.%s: zero points are int8" % name)
+        if zero_points.shape != scales.shape:
+            raise ValueError("hexmi.%s: zero_points must have the shape of scales" % name)
+    return per_tensor
+
+
+def w8a16_matmul(a, w_int8, scales, out=None, zero_points=None):
+    """C[m,n] = sum_k A[m,k] * ((W[n,k] - zero_points[n]) * scales[n]); A fp16 [M,K], W int8 [N,K], scales fp16 [N]
+    (or [1]: one scale and zero point for the tensor), zero_points int8 or None (symmetric)."""
+    if a.dtype != torch.float16:
         raise TypeError("hexmi.w8a16_matmul: expected fp16 activations, int8 weights, fp16 scales")
-    if a.dim() != 2 or w_int8.dim() != 2 or a.shape[1] != w_int8.shape[1] or scales.shape != (w_int8.shape[0],):
+    if w_int8.dtype != torch.int8 or scales.dtype != torch.float16:
+        raise TypeError("hexmi.w8a16_matmul: expected fp16 activations, int8 weights, fp16 scales")
+    if a.dim() != 2 or w_int8.dim() != 2 or a.shape[1] != w_int8.shape[1]:
         raise ValueError("hexmi.w8a16_matmul: shapes A[M,K], W[N,K], scales[N] required")
+    per_tensor = _quant_params("w8a16_matmul", w_int8, scales, zero_points)
     dev = _device() if a.device.type != "cuda" else a.device
     ad, wd, sd = _stage(a, dev), _stage(w_int8, dev), _stage(scales, dev)
     od = _out_like(out, (a.shape[0], w_int8.shape[0]), torch.float16, dev)
-    _w8a16_impl(ad, wd, sd, od)
+    if zero_points is None and not per_tensor:
+        _w8a16_impl(ad, wd, sd, od)
+    else:
+        zd = _stage(zero_points, dev)
+        M, K = ad.shape
+        with _on(ad.device):
+            _lib.check(_lib.lib().hexmi_gemm_w8a16_ex(M, wd.shape[0], K, _p(ad), _p(wd), _p(sd), _p(zd),
+                                                      1 if per_tensor else 0, _p(od), _stream()), "hexmi_gemm_w8a16_ex")
     return _finish(od, out)
 
 
@@ -457,14 +484,20 @@ def w8a16_matmul_packed(a, w_packed, scales, out=None):
     return _finish(od, out)
 
 
-def dequant_w8(w_int8, scales, out=None):
-    """fp32 [N,K] = float(W[n,k]) * float(scales[n]) (the dequantisation the fused kernel applies)."""
-    if w_int8.dtype != torch.int8 or scales.dtype != torch.float16:
-        raise TypeError("hexmi.dequant_w8: expected int8 weights, fp16 scales")
+def dequant_w8(w_int8, scales, out=None, zero_points=None):
+    """fp32 [N,K] = (float(W[n,k]) - zero_points[n]) * float(scales[n]) (the dequantisation the fused kernel applies;
+    scales / zero_points of one element: per tensor)."""
+    per_tensor = _quant_params("dequant_w8", w_int8, scales, zero_points)
     dev = _device() if w_int8.device.type != "cuda" else w_int8.device
     wd, sd = _stage(w_int8, dev), _stage(scales, dev)
     od = _out_like(out, w_int8.shape, torch.float32, dev)
-    _dequant_impl(wd, sd, od)
+    if zero_points is None and not per_tensor:
+        _dequant_impl(wd, sd, od)
+    else:
+        zd = _stage(zero_points, dev)
+        with _on(wd.device):
+            _lib.check(_lib.lib().hexmi_dequant_w8_ex(wd.shape[0], wd.shape[1], _p(wd), _p(sd), _p(zd),
+                                                      1 if per_tensor else 0, _p(od), _stream()), "hexmi_dequant_w8_ex")
     return _finish(od, out)
 
 

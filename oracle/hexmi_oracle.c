@@ -272,6 +272,36 @@ void oracle_matmul_w8a16(const uint16_t *A, const int8_t *W, const uint16_t *sca
   }
 }
 
+/* The asymmetric / per-tensor forms of the same dequantisation (quant.dcast: f = (float(q) - zero_point) * scale,
+ * "per-tensor or per-axis", qcom_hexagon_backend/lib/Conversion/LinalgToLLVM/LinalgToLLVMPass.cpp:224-230,
+ * lib/Transforms/SeedLayoutConversions.cpp:135-157). zero_points may be NULL (0); per_tensor != 0 reads scale and
+ * zero point at index 0. The difference of two int8 values is an exact fp32 integer, then ONE fp32 multiply. */
+void oracle_dequant_w8_ex(const int8_t *W, const uint16_t *scales_f16, const int8_t *zero_points, int per_tensor,
+                          float *out, int64_t N, int64_t K) {
+  for (int64_t n = 0; n < N; ++n) {
+    const int64_t p = per_tensor ? 0 : n;
+    float s = f16_to_f32(scales_f16[p]);
+    float zp = zero_points ? (float)zero_points[p] : 0.0f;
+    for (int64_t k = 0; k < K; ++k) out[n * K + k] = ((float)W[n * K + k] - zp) * s;
+  }
+}
+
+void oracle_matmul_w8a16_ex(const uint16_t *A, const int8_t *W, const uint16_t *scales_f16, const int8_t *zero_points,
+                            int per_tensor, uint16_t *C, int64_t M, int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+  for (int64_t n = 0; n < N; ++n) {
+    const int64_t p = per_tensor ? 0 : n;
+    float s = f16_to_f32(scales_f16[p]);
+    float zp = zero_points ? (float)zero_points[p] : 0.0f;
+    for (int64_t m = 0; m < M; ++m) {
+      double acc = 0.0;
+      for (int64_t k = 0; k < K; ++k)
+        acc += (double)f16_to_f32(A[m * K + k]) * (double)(((float)W[n * K + k] - zp) * s);
+      C[m * N + n] = f32_to_f16((float)acc);
+    }
+  }
+}
+
 /* ---- attention -------------------------------------------------------------
  * Brute force: O = softmax(scale * Q K^T + mask) V per (z,h), the form
  * tm_tensor.attention lowers to (qcom_hexagon_backend/lib/Transforms/LowerTmTensor.cpp:120-227:

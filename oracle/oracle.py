@@ -163,6 +163,29 @@ def matmul_w8a16(a, w, scales):
     return c
 
 
+def dequant_w8_ex(w, scales, zero_points=None, per_tensor=False):
+    """(float(q) - zero_point) * scale with per-channel or per-tensor parameters (zero_points int8 or None)."""
+    w, scales = _c(w), _c(scales)
+    zp = None if zero_points is None else _c(zero_points)
+    assert w.dtype == np.int8 and scales.dtype == np.float16 and (zp is None or zp.dtype == np.int8)
+    out = np.empty(w.shape, np.float32)
+    _l().oracle_dequant_w8_ex(_ptr(w), _ptr(scales), _ptr(zp) if zp is not None else None, _int(1 if per_tensor else 0),
+                              _ptr(out), _i64(w.shape[0]), _i64(w.shape[1]))
+    return out
+
+
+def matmul_w8a16_ex(a, w, scales, zero_points=None, per_tensor=False):
+    a, w, scales = _c(a), _c(w), _c(scales)
+    zp = None if zero_points is None else _c(zero_points)
+    assert a.dtype == np.float16 and w.dtype == np.int8 and scales.dtype == np.float16
+    M, K = a.shape
+    N = w.shape[0]
+    c = np.empty((M, N), np.float16)
+    _l().oracle_matmul_w8a16_ex(_ptr(a), _ptr(w), _ptr(scales), _ptr(zp) if zp is not None else None,
+                                _int(1 if per_tensor else 0), _ptr(c), _i64(M), _i64(N), _i64(K))
+    return c
+
+
 def pack_w8(w):
     """Fragment-major re-layout of int8 weights [N, K] (K % 64 == 0): tiles of 16 channels x 64 k, tile (t, s) at
     byte ((t*K/64) + s)*1024, lane l = g*16 + r holds W[16t + r][64s + 16g : 64s + 16g + 16]; rows past N are 0.

@@ -8,10 +8,11 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "hexmi.h")
+PROBE_HEADER = os.path.join(ROOT, "include", "hexmi_calibrate.h")     # measurement probes, not the operator ABI
 
 
-def _declared():
-    text = open(HEADER).read()
+def _declared(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(hexmi_[a-z0-9_]+)\s*\(", text)))
 
@@ -28,13 +29,15 @@ def test_library_exports_every_declared_symbol():
     import hexmi
     assert os.path.exists(hexmi.LIB_PATH), "build libhexmi.so first: python hexagon-mlir_amd/build.py"
     handle = ctypes.CDLL(hexmi.LIB_PATH)
-    for name in _declared():
+    for name in _declared() + _declared(PROBE_HEADER):
         assert hasattr(handle, name), "libhexmi.so does not export %s" % name
 
 
 def test_loader_binds_exactly_the_header():
     from hexmi import _lib
     assert sorted(_lib.SIGNATURES) == _declared()
+    assert sorted(_lib.PROBE_SIGNATURES) == _declared(PROBE_HEADER)
+    assert not set(_lib.SIGNATURES) & set(_lib.PROBE_SIGNATURES)      # the operator header declares no probe
     lib = _lib.lib()
     assert lib.hexmi_version().decode().startswith("hexmi ")
     assert "invalid" in _lib.strerror(_lib.EINVAL)

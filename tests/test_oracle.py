@@ -246,6 +246,46 @@ def test_w8a16_vs_closed_form(oracle, M):
     assert _ulp16(got, want.half()) <= 1
 
 
+def test_dequant_with_zero_point_and_per_tensor_parameters(oracle):
+    # quant.dcast f = (float(q) - zero_point) * scale: integer arithmetic in float64 (exact), then the rounding of
+    # the one product to fp32; a dropped or mis-signed zero point, or one taken from the wrong channel, fails
+    g = torch.Generator().manual_seed(14)
+    w = torch.randint(-128, 128, (21, 50), generator=g, dtype=torch.int8)
+    s = (0.001 + 0.019 * torch.rand(21, generator=g)).half()
+    zp = torch.randint(-128, 128, (21,), generator=g, dtype=torch.int8)
+    got = oracle.dequant_w8_ex(w.numpy(), s.numpy(), zp.numpy())
+    want = ((w.double() - zp.double()[:, None]) * s.double()[:, None]).float()
+    assert (got.view(np.uint32) == want.numpy().view(np.uint32)).all()
+    # per tensor: index 0 for every channel
+    got = oracle.dequant_w8_ex(w.numpy(), s.numpy(), zp.numpy(), per_tensor=True)
+    want = ((w.double() - float(zp[0])) * float(s[0])).float()
+    assert (got.view(np.uint32) == want.numpy().view(np.uint32)).all()
+    # q == zero_point is exactly 0; scale 1 gives the integer difference; no zero point is the symmetric form
+    eq = oracle.dequant_w8_ex(np.int8([[5, 5], [-7, -7]]), np.float16([3.0, 2.0]), np.int8([5, -7]))
+    assert (eq == 0).all()
+    d = oracle.dequant_w8_ex(np.int8([[127, -128]]), np.float16([1.0]), np.int8([-128]))
+    assert (d == np.float32([[255.0, 0.0]])).all()
+    assert (oracle.dequant_w8_ex(w.numpy(), s.numpy()).view(np.uint32) == oracle.dequant_w8(w.numpy(), s.numpy()).view(np.uint32)).all()
+
+
+@pytest.mark.parametrize("per_tensor", [False, True])
+def test_w8a16_with_zero_point_vs_closed_form(oracle, per_tensor):
+    g = torch.Generator().manual_seed(15)
+    a = torch.randn(5, 256, generator=g).half()
+    w = torch.randint(-128, 128, (40, 256), generator=g, dtype=torch.int8)
+    s = (0.001 + 0.019 * torch.rand(40, generator=g)).half()
+    zp = torch.randint(-20, 21, (40,), generator=g, dtype=torch.int8)
+    got = _t(oracle.matmul_w8a16_ex(a.numpy(), w.numpy(), s.numpy(), zp.numpy(), per_tensor))
+    sd = s.double()[0].expand(40) if per_tensor else s.double()
+    zd = zp.double()[0].expand(40) if per_tensor else zp.double()
+    want = a.double() @ ((w.double() - zd[:, None]) * sd[:, None]).t()
+    assert _ulp16(got, want.half()) <= 1
+    # the zero point's share is -zp * s * rowsum(A): a row of ones makes it visible on its own
+    ones = np.ones((1, 256), np.float16)
+    c = oracle.matmul_w8a16_ex(ones, np.zeros((40, 256), np.int8), np.ones(40, np.float16), zp.numpy(), per_tensor)
+    assert np.array_equal(c[0].astype(np.float64), -256.0 * zd.numpy())
+
+
 # ------------------------------------------------------------------ attention
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_vs_sdpa(oracle, causal):

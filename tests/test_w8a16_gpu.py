@@ -280,3 +280,53 @@ def test_w8a16_workspace_contract(hexmi):
     assert rc == 0 and close16(no_ws.cpu(), with_ws.cpu(), max_ulp=2, atol=2e-4)
     rc, _ = _ws_call(hexmi, ad, wd, sd, ws, ws_bytes=-1)
     assert rc == hexmi._lib.EINVAL
+
+
+# ---- quant.dcast with a zero point, per channel or per tensor ------------------------------------------------------
+
+@pytest.mark.parametrize("per_tensor", [False, True])
+def test_dequant_with_zero_point_bit_exact(hexmi, oracle, per_tensor):
+    g = _gen(18)
+    w = torch.randint(-128, 128, (300, 192), generator=g, dtype=torch.int8)
+    n = 1 if per_tensor else 300
+    s = (0.001 + 0.019 * torch.rand(n, generator=g)).half()
+    zp = torch.randint(-128, 128, (n,), generator=g, dtype=torch.int8)
+    got = hexmi.dequant_w8(w.cuda(), s.cuda(), zero_points=zp.cuda()).cpu().numpy()
+    want = oracle.dequant_w8_ex(w.numpy(), s.numpy(), zp.numpy(), per_tensor)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+    # every (weight, zero point) pair of int8 with scale 1: the integer difference, exactly
+    allw = torch.arange(-128, 128, dtype=torch.int16).to(torch.int8).repeat(256, 1)
+    allz = torch.arange(-128, 128, dtype=torch.int16).to(torch.int8)
+    got = hexmi.dequant_w8(allw.cuda(), torch.ones(256, dtype=torch.float16).cuda(), zero_points=allz.cuda()).cpu()
+    assert torch.equal(got, allw.float() - allz.float()[:, None])
+    # without a zero point and per channel it is the symmetric entry point
+    s2 = (0.001 + 0.019 * torch.rand(300, generator=g)).half()
+    assert torch.equal(hexmi.dequant_w8(w.cuda(), s2.cuda()).cpu(), w.float() * s2.float()[:, None])
+
+
+@pytest.mark.parametrize("per_tensor", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 96, 512), (16, 1000, 256), (70, 130, 128), (33, 40, 4096), (5, 33, 100),
+                                   (3, 64, 72)])
+def test_w8a16_with_zero_point_parity(hexmi, oracle, per_tensor, M, N, K):
+    g = _gen(19)
+    a = torch.randn(M, K, generator=g).half()
+    w = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    n = 1 if per_tensor else N
+    s = (0.001 + 0.019 * torch.rand(n, generator=g)).half()
+    zp = torch.randint(-128, 128, (n,), generator=g, dtype=torch.int8)
+    got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda(), zero_points=zp.cuda()).cpu()
+    want = torch.from_numpy(oracle.matmul_w8a16_ex(a.numpy(), w.numpy(), s.numpy(), zp.numpy(), per_tensor))
+    assert close16(got, want, max_ulp=1, atol=4e-4)
+    # zero point selection is exact: activations that pick one weight give (w - zp) * s with s a power of two
+    sel = torch.zeros(1, K, dtype=torch.float16)
+    sel[0, K - 1] = 1.0
+    s2 = torch.tensor([2.0 ** -(i % 6) for i in range(n)], dtype=torch.float16)
+    got = hexmi.w8a16_matmul(sel.cuda(), w.cuda(), s2.cuda(), zero_points=zp.cuda()).cpu().double()
+    zd = zp.double().expand(N) if per_tensor else zp.double()
+    sd = s2.double().expand(N) if per_tensor else s2.double()
+    assert torch.equal(got[0], (w[:, K - 1].double() - zd) * sd)
+    # per-tensor scale without a zero point
+    if per_tensor:
+        got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
+        want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w.numpy(), s.expand(N).contiguous().numpy()))
+        assert close16(got, want, max_ulp=1, atol=2e-4)
