@@ -499,6 +499,11 @@ class AddMatmulSoftmax(Workload):
         self.sets[0]["out"] = torch.empty(self.M, self.N, dtype=dt, device="cuda")
 
     def step(self, i):
+        # the path the operator takes by itself at this size (one launch for small products, three beyond)
+        s = self.sets[0]
+        self.hexmi.add_matmul_softmax(s["x"], s["y"], s["z"], out=s["out"])
+
+    def step_fused(self, i):
         s = self.sets[0]
         self.hexmi.add_matmul_softmax(s["x"], s["y"], s["z"], out=s["out"], fused=True)
 
@@ -666,6 +671,28 @@ def report(wl, ms):
     return {"bound": wl.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
             "frac": round(achieved / peak, 4), "traffic": measured_traffic(wl), "kernel": wl.kernel,
             "work_per_step": wl.work}
+
+
+def box_calibration(torch, hexmi):
+    """This box's own ceilings, measured in the same run as everything else (boxes of one pool differ by 10 % and
+    more): what a plain device copy moves, and what the matrix cores sustain on U(-1,1) operands in a registers-only
+    stream of the instruction the GEMM is built on. A fraction of the published peak can be read against these."""
+    copy = CopyCalibration()
+    copy.setup(torch, hexmi)
+    cm = measure(torch, copy, 20, 3, use_graph=True, replays=3)
+    copy_gbs = copy.work / (cm["ms"] * 1e-3) / 1e9
+    copy.sets = None
+    peak = MfmaPeak(1, "f16", "uniform")
+    peak.iters = 4000                                   # about 40 ms per launch
+    peak.setup(torch, hexmi)
+    pm = measure(torch, peak, 3, 1, use_graph=False, replays=3)
+    mfma_tf = peak.work / (pm["ms"] * 1e-3) / 1e12
+    torch.cuda.empty_cache()
+    return {"copy_64MiB_GBs": round(copy_gbs, 1), "copy_frac_of_hbm_peak": round(copy_gbs / HBM_PEAK_GBS, 4),
+            "mfma_16x16x32_f16_uniform_TFLOPs": round(mfma_tf, 1),
+            "mfma_frac_of_peak": round(mfma_tf / MFMA_PEAK_TFLOPS, 4),
+            "note": "measured in this run on this box: a device copy (read + write bytes) and a registers-only MFMA "
+                    "stream on U(-1,1) data; the fractions in this line stay against the published peaks"}
 
 
 def steps_for(wl, steps):
@@ -971,6 +998,7 @@ def main():
                                 "sample": sample, "ms": round(sec * 1e3, 3)}
     primary.sets = None
     torch.cuda.empty_cache()
+    line["box"] = box_calibration(torch, hexmi)
 
     if not args.no_suite:
         suite, only = [], [ALIASES.get(n, n) for n in args.only.split(",") if n]
@@ -985,12 +1013,17 @@ def main():
             entry = entry_for(torch, wl, wm, whot, cores, not args.no_cpu)
             entry["steps"] = k
             if getattr(wl, "step_separate", None) is not None:
-                fused_step, wl.step = wl.step, wl.step_separate
+                # side figures: the graph forced into one launch, and forced into its separate launches
+                own_step = wl.step
+                wl.step = wl.step_fused
+                fm = measure(torch, wl, k, args.warmup, not args.no_graph)
+                wl.step = wl.step_separate
                 sm = measure(torch, wl, k, args.warmup, not args.no_graph)
-                wl.step = fused_step
+                wl.step = own_step
+                entry["one_launch"] = {"ms": round(fm["ms"], 5), "ms_min": round(fm["min"], 5)}
                 entry["separate_launches"] = {"launches": wl.launches_separate, "ms": round(sm["ms"], 5),
                                               "ms_min": round(sm["min"], 5),
-                                              "speedup_fused": round(sm["ms"] / wm["ms"], 3)}
+                                              "speedup_fused": round(sm["ms"] / fm["ms"], 3)}
             if name in ("softmax_f32_4096x1024", "w8a16_m1"):
                 entry["direct_launch"] = direct_launch_cost(torch, wl)
             suite.append(entry)

@@ -108,7 +108,10 @@ matmul_hexkl = matmul
 def attention_fwd_kernel(pid1, Q, K, V, sm_scale, Out, H, N_CTX, BLOCK_M=None, BLOCK_DMODEL=None, BLOCK_N=None,
                          STAGE=1, stride_0=None, stride_1=None, stride_2=None, stride_3=None):
     """test/python/triton/test_flash_attention.py:37-168. STAGE 1 is the full (non-causal) sweep, STAGE 3
-    the causal one; the reference launches one (z,h) per call via pid1, here every (z,h) is computed."""
+    the causal one. pid1 selects the (z, h) pair the launch works on, as in the reference (off_hz = pid1,
+    off_z = pid1 // H, off_h = pid1 % H, `:102-105`; its test passes 0 with Z = H = 1): a caller that loops pid1
+    over Z * H gets each head computed once. pid1=None (no counterpart in the reference) computes every head in
+    one launch."""
     if Q.dim() != 4 or Q.shape[1] != H or Q.shape[2] != N_CTX:
         raise ValueError("attention_fwd_kernel: Q must be [Z,H,N_CTX,D]")
     if BLOCK_DMODEL is not None and BLOCK_DMODEL != Q.shape[3]:
@@ -119,7 +122,15 @@ def attention_fwd_kernel(pid1, Q, K, V, sm_scale, Out, H, N_CTX, BLOCK_M=None, B
         raise ValueError("attention_fwd_kernel: only the contiguous [Z,H,N_CTX,D] strides %s are supported" % (want,))
     if STAGE not in (1, 3):
         raise ValueError("attention_fwd_kernel: STAGE must be 1 (full) or 3 (causal)")
-    ops.flash_attention(Q, K, V, sm_scale, causal=(STAGE == 3), out=Out)
+    if pid1 is None:
+        ops.flash_attention(Q, K, V, sm_scale, causal=(STAGE == 3), out=Out)
+        return
+    pid1 = int(pid1)
+    if not 0 <= pid1 < Q.shape[0] * H:
+        raise ValueError("attention_fwd_kernel: pid1 must be in [0, Z*H)")
+    z, h = pid1 // H, pid1 % H
+    ops.flash_attention(Q[z:z + 1, h:h + 1], K[z:z + 1, h:h + 1], V[z:z + 1, h:h + 1], sm_scale, causal=(STAGE == 3),
+                        out=Out[z:z + 1, h:h + 1])
 
 
 def _check_block(name, t, BLOCK_SIZE, programs):

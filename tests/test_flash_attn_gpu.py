@@ -95,6 +95,30 @@ def test_reference_call_site(hexmi, oracle):
     assert torch.allclose(out, _oracle(oracle, q, k, v, 0.5, False), rtol=1e-5, atol=1e-6)
 
 
+def test_reference_call_site_one_head_per_launch(hexmi, oracle):
+    # pid1 = off_hz picks the (z, h) pair a launch computes (test_flash_attention.py:102-105): a loop over Z * H
+    # fills the output head by head, and a single launch leaves the other heads untouched
+    Z, H, N_CTX, D_HEAD = 2, 3, 256, 64
+    q, k, v = _qkv(Z, H, N_CTX, D_HEAD, torch.float32, rand=True, seed=4)
+    want = _oracle(oracle, q, k, v, 0.5, False)
+    out = torch.full_like(q, -7.0)
+    kw = dict(Q=q, K=k, V=v, sm_scale=0.5, Out=out, H=H, N_CTX=N_CTX, BLOCK_M=64, BLOCK_DMODEL=D_HEAD, BLOCK_N=64,
+              STAGE=1, stride_0=H * N_CTX * D_HEAD, stride_1=N_CTX * D_HEAD, stride_2=D_HEAD, stride_3=1)
+    hexmi.kernels.attention_fwd_kernel[(4,)](pid1=4, **kw)              # z = 1, h = 1
+    assert torch.allclose(out[1, 1], want[1, 1], rtol=1e-5, atol=1e-6)
+    untouched = torch.ones(Z, H, dtype=torch.bool)
+    untouched[1, 1] = False
+    assert (out[untouched] == -7.0).all()
+    for pid1 in range(Z * H):
+        hexmi.kernels.attention_fwd_kernel[(4,)](pid1=pid1, **kw)
+    assert torch.allclose(out, want, rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        hexmi.kernels.attention_fwd_kernel[(4,)](pid1=Z * H, **kw)
+    all_heads = torch.zeros_like(q)
+    hexmi.kernels.attention_fwd_kernel[(4,)](pid1=None, **{**kw, "Out": all_heads})
+    assert torch.equal(all_heads, out)
+
+
 def test_hexkl_attention_fixture_types(hexmi, oracle):
     # test/python/mlir/hexkl_attention: fp16 Q/K/V ~ N(0, 0.5) rounded to 4 decimals, fp32 output, MAX_DIFF 1e-3
     g = _gen(2)
