@@ -197,12 +197,17 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
 // Epilogue operands of hexmi_gemm_ex: C = A B + bias[column] + residual[row, column], both of the output type, added
 // to the fp32 sums before the one rounding to the output type. ok4: the four columns col .. col+3 exist and the
 // operands may be read as one 4-element run (the fast kernels: N % 8 == 0, ldr % 4 == 0, aligned bases).
+// The output pointer of a tiled kernel: declared without aliasing (as every operand pointer here is) except in the
+// instantiations that add a residual, which may be the output buffer itself.
+template <typename P, bool MAY_ALIAS> struct OutPtr { typedef P* __restrict__ type; };
+template <typename P> struct OutPtr<P, true> { typedef P* type; };
+
 template <typename OutT> struct Run4;
 template <> struct Run4<float> { typedef f32x4 V; };
 template <> struct Run4<f16> { typedef f16x4 V; };
 template <> struct Run4<bf16> { typedef bf16x4 V; };
 template <typename OutT>
-__device__ __forceinline__ void add_epilogue4(f32x4& a, const OutT* __restrict__ bias, const OutT* __restrict__ resid,
+__device__ __forceinline__ void add_epilogue4(f32x4& a, const OutT* __restrict__ bias, const OutT* resid,
                                               int64_t ldr, int row, int col) {
   typedef typename Run4<OutT>::V V;
   if (bias) {
@@ -226,10 +231,10 @@ __device__ __forceinline__ void add_epilogue4(f32x4& a, const OutT* __restrict__
 template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false, int NWN = 2,
           bool EPI = false>
 __global__ __launch_bounds__(NWN * 128)
-void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __restrict__ C, int M, int N, int K,
+void gemm_kernel(const T* __restrict__ A, const void* __restrict__ Bv, typename OutPtr<OutT, EPI>::type C, int M, int N, int K,
                  int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
                  const f16* __restrict__ scales = nullptr, const OutT* __restrict__ bias = nullptr,
-                 const OutT* __restrict__ resid = nullptr, int64_t ldr = 0) {
+                 const OutT* resid = nullptr, int64_t ldr = 0) {
   const T* B = static_cast<const T*>(Bv);
   typedef typename Mfma<T>::Frag Frag;
   constexpr int NW = 2 * NWN;                       // waves per workgroup
@@ -605,10 +610,10 @@ template <> struct Mfma16<bf16> {
 template <typename T, typename OutT, int WM, int WN, bool TRANS_B, bool TAIL, bool B_I8 = false, int NS = 2,
           bool EPI = false>
 __global__ __launch_bounds__(256)
-void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT* __restrict__ C, int M, int N, int K,
+void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, typename OutPtr<OutT, EPI>::type C, int M, int N, int K,
                      int64_t lda, int64_t ldb, int64_t ldc, int tiles_m, int tiles_n,
                      const f16* __restrict__ scales = nullptr, const OutT* __restrict__ bias = nullptr,
-                     const OutT* __restrict__ resid = nullptr, int64_t ldr = 0) {
+                     const OutT* resid = nullptr, int64_t ldr = 0) {
   static_assert(!B_I8 || (TRANS_B && sizeof(T) == 2), "int8 B is [N,K] and multiplies fp16 A");
   const T* B = static_cast<const T*>(Bv);
   typedef typename Mfma<T>::Frag Frag;
@@ -930,9 +935,9 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
 // Any shape, any alignment: 64x64 tile, scalar guarded loads through LDS, MFMA 32x32x16 with zero padding.
 template <typename T, typename OutT, bool TRANS_B>
 __global__ __launch_bounds__(256)
-void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT* __restrict__ C, int M, int N, int K,
+void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT* C, int M, int N, int K,
                          int64_t lda, int64_t ldb, int64_t ldc, const OutT* __restrict__ bias = nullptr,
-                         const OutT* __restrict__ resid = nullptr, int64_t ldr = 0) {
+                         const OutT* resid = nullptr, int64_t ldr = 0) {
   typedef typename Mfma<T>::Frag Frag;
   constexpr int TB = 64, TK = 16, PAD = 8;
   __shared__ __attribute__((aligned(16))) T a_s[TB][TK + PAD];   // [m][k]
@@ -979,9 +984,9 @@ void gemm_kernel_generic(const T* __restrict__ A, const T* __restrict__ B, OutT*
 // Any shape.
 template <bool TRANS_B>
 __global__ __launch_bounds__(256)
-void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C, int M, int N,
+void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N,
                      int K, int64_t lda, int64_t ldb, int64_t ldc, const float* __restrict__ bias = nullptr,
-                     const float* __restrict__ resid = nullptr, int64_t ldr = 0) {
+                     const float* resid = nullptr, int64_t ldr = 0) {
   constexpr int TB = 64, TK = 16;
   __shared__ float a_s[TK][TB + 4];                  // [k][m]
   __shared__ float b_s[TK][TB + 4];                  // [k][n]

@@ -1,7 +1,7 @@
 // Library-level entry points: version, status text, device query.
 #include "hexmi_common.h"
 
-extern "C" const char* hexmi_version(void) { return "hexmi 0.1 gfx950"; }
+extern "C" const char* hexmi_version(void) { return "hexmi 0.3 gfx950"; }
 
 extern "C" const char* hexmi_strerror(int status) {
   switch (status) {

@@ -292,7 +292,28 @@ def _out_like(out, shape, dtype, dev):
 # --------------------------------------------------------------------------
 # public operators. They call the implementations above directly: the same code `torch.ops.hexmi.*` runs, without
 # the dispatcher's round trip into Python (several microseconds, more than the shortest kernels here take).
+# A caller that traces a model (torch.compile, FakeTensor propagation) needs the operators to appear as
+# `torch.ops.hexmi.*` nodes: `through_dispatcher(True)` routes the operators that have a registered schema through
+# the dispatcher (2-D operands, no column blocks; anything else keeps the direct call).
 # --------------------------------------------------------------------------
+_THROUGH_DISPATCHER = False
+
+
+def through_dispatcher(enable=True):
+    """Route softmax / rms_norm / layer_norm / matmul / w8a16_matmul / flash_attention through `torch.ops.hexmi.*`
+    (visible to tracing) instead of calling the library directly. Returns the previous setting."""
+    global _THROUGH_DISPATCHER
+    previous, _THROUGH_DISPATCHER = _THROUGH_DISPATCHER, bool(enable)
+    return previous
+
+
+def _run(name, impl, simple, *args):
+    """impl(*args) directly, or torch.ops.hexmi.<name>(*simple) when tracing asked for the dispatcher and the call
+    has the registered operator's form (simple is not None)."""
+    if _THROUGH_DISPATCHER and simple is not None:
+        getattr(torch.ops.hexmi, name)(*simple)
+    else:
+        impl(*args)
 def _row_strided(t):
     """A 2-D device tensor whose rows are contiguous but not adjacent (a column slice, a padded buffer): the row
     operators read and write it in place through its row stride, as the reference's kernels take a memref with
@@ -324,7 +345,7 @@ def softmax(x, out=None, dim=-1, block_cols=0):
         raise ValueError("hexmi.softmax needs at least 1 dimension")
     dev = _device() if x.device.type != "cuda" else x.device
     xd, od, rows, cols = _row_operands(x, out, dev)
-    _softmax_impl(xd, od, rows, cols, int(block_cols))
+    _run("softmax", _softmax_impl, (xd, od) if xd.dim() == 2 and not block_cols else None, xd, od, rows, cols, int(block_cols))
     return _finish(od, out)
 
 
@@ -335,7 +356,9 @@ def rms_norm(x, weight=None, eps=1e-5, out=None, block_cols=0):
     if weight is not None and (weight.shape != (cols,) or weight.dtype != x.dtype):
         raise ValueError("hexmi.rms_norm: weight must be [%d] of %s" % (cols, x.dtype))
     xd, od, rows, c = _row_operands(x, out, dev)
-    _rms_norm_impl(xd, _stage(weight, dev), float(eps), od, rows, c, int(block_cols))
+    wd = _stage(weight, dev)
+    _run("rms_norm", _rms_norm_impl, (xd, wd, float(eps), od) if xd.dim() == 2 and not block_cols else None,
+         xd, wd, float(eps), od, rows, c, int(block_cols))
     return _finish(od, out)
 
 
@@ -352,7 +375,8 @@ def layer_norm(x, weight=None, bias=None, eps=1e-5, out=None, mean=None, rstd=No
     wd, bd = _stage(weight, dev), _stage(bias, dev)
     md = None if mean is None else _out_like(mean if mean.dtype == torch.float32 else None, (nrows,), torch.float32, dev)
     rd = None if rstd is None else _out_like(rstd if rstd.dtype == torch.float32 else None, (nrows,), torch.float32, dev)
-    _layer_norm_impl(xd, wd, bd, float(eps), od, md, rd, rows, c, int(block_cols))
+    _run("layer_norm", _layer_norm_impl, (xd, wd, bd, float(eps), od, md, rd) if xd.dim() == 2 and not block_cols else None,
+         xd, wd, bd, float(eps), od, md, rd, rows, c, int(block_cols))
     if mean is not None:
         _finish(md, mean)
     if rstd is not None:
@@ -388,7 +412,7 @@ def matmul(a, b, out=None, out_dtype=None, trans_b=False, bias=None, residual=No
     ad, bd = _stage(a, dev), _stage(b, dev)
     od = _out_like(out, (M, N), out_dtype, dev)
     if bias is None and residual is None:
-        _matmul_impl(ad, bd, bool(trans_b), od)
+        _run("matmul", _matmul_impl, (ad, bd, bool(trans_b), od), ad, bd, bool(trans_b), od)
     else:
         _linear_impl(ad, bd, _stage(bias, dev), _stage(residual, dev), bool(trans_b), od)
     return _finish(od, out)
@@ -440,7 +464,7 @@ def w8a16_matmul(a, w_int8, scales, out=None, zero_points=None):
     ad, wd, sd = _stage(a, dev), _stage(w_int8, dev), _stage(scales, dev)
     od = _out_like(out, (a.shape[0], w_int8.shape[0]), torch.float16, dev)
     if zero_points is None and not per_tensor:
-        _w8a16_impl(ad, wd, sd, od)
+        _run("w8a16_matmul", _w8a16_impl, (ad, wd, sd, od), ad, wd, sd, od)
     else:
         zd = _stage(zero_points, dev)
         M, K = ad.shape
@@ -515,7 +539,7 @@ def flash_attention(q, k, v, sm_scale=None, causal=False, out=None, out_dtype=No
     dev = _device() if q.device.type != "cuda" else q.device
     qd, kd, vd = _stage(q, dev), _stage(k, dev), _stage(v, dev)
     od = _out_like(out, q.shape, out_dtype, dev)
-    _flash_impl(qd, kd, vd, float(sm_scale), bool(causal), od)
+    _run("flash_attention", _flash_impl, (qd, kd, vd, float(sm_scale), bool(causal), od), qd, kd, vd, float(sm_scale), bool(causal), od)
     return _finish(od, out)
 
 

@@ -333,15 +333,20 @@ def test_gemm_ex_rounds_once(hexmi):
     assert (fused - want.half().double()).abs().max().item() <= 2 * torch.finfo(torch.float16).eps * want.abs().max().item()
 
 
-def test_gemm_ex_residual_may_alias_output(hexmi):
+# one shape per kernel that takes a residual: paired 64-k slabs, 32-k slabs (K % 64 != 0), the any-shape kernel
+# (odd N), the fp32 matrix-core kernel and the fp32 vector-ALU kernel (K % 32 != 0)
+@pytest.mark.parametrize("dtype,M,N,K", [(torch.float16, 384, 768, 768), (torch.float16, 256, 512, 96),
+                                         (torch.bfloat16, 200, 333, 64), (torch.float32, 256, 512, 128),
+                                         (torch.float32, 130, 77, 50)])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gemm_ex_residual_may_alias_output(hexmi, dtype, M, N, K, trans_b):
     g = torch.Generator().manual_seed(12)
-    M, N, K = 384, 768, 768
-    a = (torch.randn(M, K, generator=g) * 0.1).half().cuda()
-    b = (torch.randn(K, N, generator=g) * 0.1).half().cuda()
-    x = torch.randn(M, N, generator=g).half().cuda()
-    want = hexmi.matmul(a, b, residual=x)
+    a = (torch.randn(M, K, generator=g) * 0.1).to(dtype).cuda()
+    b = (torch.randn(*((N, K) if trans_b else (K, N)), generator=g) * 0.1).to(dtype).cuda()
+    x = torch.randn(M, N, generator=g).to(dtype).cuda()
+    want = hexmi.matmul(a, b, residual=x, trans_b=trans_b)
     acc = x.clone()
-    hexmi.matmul(a, b, residual=acc, out=acc)                       # x += a @ b, in place
+    hexmi.matmul(a, b, residual=acc, out=acc, trans_b=trans_b)      # x += a @ b, in place
     assert torch.equal(acc, want)
 
 

@@ -17,6 +17,8 @@ def _cases(hexmi):
         return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
 
     w8 = torch.randint(-127, 128, (512, 1024), generator=g, dtype=torch.int8).cuda()
+    w8k = torch.randint(-127, 128, (320, 8192), generator=g, dtype=torch.int8).cuda()      # a long K: summed over K parts
+    sck = (0.001 + 0.01 * torch.rand(320, generator=g)).half().cuda()
     sc = (0.001 + 0.01 * torch.rand(512, generator=g)).half().cuda()
     wn, bn = r(4096), r(4096)
     bmat, bias, zs = r(768, 512, scale=0.05), r(512), r(64, 96, dtype=torch.float32)
@@ -33,6 +35,9 @@ def _cases(hexmi):
         ("w8a16_m16", r(16, 1024), lambda x, o: hexmi.w8a16_matmul(x, w8, sc, out=o), (16, 512)),
         ("w8a16_m64", r(64, 1024), lambda x, o: hexmi.w8a16_matmul(x, w8, sc, out=o), (64, 512)),
         ("w8a16_m200", r(200, 1024), lambda x, o: hexmi.w8a16_matmul(x, w8, sc, out=o), (200, 512)),
+        ("w8a16_k_parts", r(96, 8192), lambda x, o: hexmi.w8a16_matmul(x, w8k, sck, out=o), (96, 320)),
+        ("softmax_split_rows", r(4, 65536, dtype=torch.float32), lambda x, o: hexmi.softmax(x, out=o), None),
+        ("layer_norm_column_blocks", r(64, 4096), lambda x, o: hexmi.layer_norm(x, wn, bn, 1e-5, out=o, block_cols=1024), None),
         ("flash_causal", r(2, 4, 512, 128), lambda x, o: hexmi.flash_attention(x, k4, v4, 128 ** -0.5, True, out=o), None),
         ("attention_masked", r(4, 256, 128), lambda x, o: hexmi.attention(x, k3, v3, mask, out=o), None),
         ("gelu", r(1000, 333), lambda x, o: hexmi.gelu(x, out=o), None),
@@ -101,3 +106,19 @@ def test_calls_on_two_streams_do_not_interfere(hexmi):
         torch.cuda.synchronize()
         for got, ref in zip((c, y, o, t), want):
             assert torch.equal(got, ref)
+
+
+def test_operators_through_the_dispatcher(hexmi):
+    # the route tracing needs: the public operators as torch.ops.hexmi.* calls, same results bit for bit
+    g = torch.Generator().manual_seed(80)
+    x = torch.randn(64, 1024, generator=g).half().cuda()
+    w = (1 + 0.1 * torch.randn(1024, generator=g)).half().cuda()
+    b = torch.randn(1024, 256, generator=g).half().cuda()
+    direct = (hexmi.softmax(x), hexmi.rms_norm(x, w, 1e-5), hexmi.layer_norm(x, w, w, 1e-5), hexmi.matmul(x, b))
+    previous = hexmi.through_dispatcher(True)
+    try:
+        routed = (hexmi.softmax(x), hexmi.rms_norm(x, w, 1e-5), hexmi.layer_norm(x, w, w, 1e-5), hexmi.matmul(x, b))
+    finally:
+        hexmi.through_dispatcher(previous)
+    for d, r in zip(direct, routed):
+        assert torch.equal(d, r)

@@ -18,10 +18,17 @@ def _both(lib, _lib, x, n, block, code):
     want = torch.zeros(programs, dtype=x.dtype, device="cuda")
     got = torch.full((programs,), 7.0, dtype=x.dtype, device="cuda")
     assert lib.hexmi_block_sum_ws(x.data_ptr(), want.data_ptr(), n, block, code, ws.data_ptr(), need, None) == _lib.OK
-    before = torch.cuda.memory_allocated()
+    # The first launch of a kernel in a process makes the HIP runtime load its code object (device memory the runtime
+    # owns), and the first call on a device looks up the scratch array: one call goes ahead of the measured one.
     assert lib.hexmi_block_sum_static(x.data_ptr(), got.data_ptr(), n, block, code, None) == _lib.OK
-    assert torch.cuda.memory_allocated() == before
+    got.fill_(7.0)
     torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]                 # hipMemGetInfo: sees every allocation on the device,
+    assert lib.hexmi_block_sum_static(x.data_ptr(), got.data_ptr(), n, block, code, None) == _lib.OK
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before             # torch's own allocator included
+    assert torch.cuda.mem_get_info()[0] == free_before
     return got.cpu(), want.cpu(), need
 
 
@@ -58,3 +65,29 @@ def test_static_block_sum_limits(hexmi):
     assert lib.hexmi_block_sum_static(x.data_ptr(), x.data_ptr(), (1 << 30) + 1, 1 << 20, _lib.F32, None) == _lib.ETOOBIG
     assert lib.hexmi_block_sum_static(None, None, 4, 4, _lib.F32, None) == _lib.EINVAL
     assert lib.hexmi_block_sum_static(None, None, 0, 4, _lib.F32, None) == _lib.OK
+
+
+def test_static_block_sum_under_graph_capture(hexmi):
+    # the callers this entry point is for: code under HIP graph capture. Captured after one warm-up call (the first
+    # call on a device looks up the scratch array's address), replayed on changing inputs with eager work between.
+    from hexmi import _lib
+    lib = _lib.lib()
+    n, block = 1 << 21, 1 << 20
+    g = _gen(8)
+    x = torch.randn(n, generator=g).cuda()
+    out = torch.zeros(2, device="cuda")
+    eager = torch.zeros(2, device="cuda")
+    assert lib.hexmi_block_sum_static(x.data_ptr(), eager.data_ptr(), n, block, _lib.F32, None) == _lib.OK
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            assert lib.hexmi_block_sum_static(x.data_ptr(), out.data_ptr(), n, block, _lib.F32, stream.cuda_stream) == _lib.OK
+    for replay in range(3):
+        x.copy_((torch.randn(n, generator=g) * (1 + replay)).cuda())
+        assert lib.hexmi_block_sum_static(x.data_ptr(), eager.data_ptr(), n, block, _lib.F32, None) == _lib.OK
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), replay
