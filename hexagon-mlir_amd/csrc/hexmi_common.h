@@ -215,12 +215,10 @@ int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t
 // W8A16 on a (channel range x K part) decomposition with the K parts summed through a caller workspace
 // (w8a16_split.hip). w8a16_split_workspace: bytes the shape needs (0: one K part, or a shape the kernel does not
 // take). w8a16_split returns false when it does not take the call (shape, alignment, workspace too small).
-// force_parts / force_cols > 0 override the plan's K parts and channel ranges (measurement only).
 int64_t w8a16_split_workspace(int64_t M, int64_t N, int64_t K, int cus);
 int64_t w8a16_split_header(int64_t M, int64_t N, int64_t K, int cus);   // leading bytes that must be zero at launch
 bool w8a16_split(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,
-                 void* workspace, int64_t workspace_bytes, int cus, hipStream_t stream, int* status,
-                 int force_parts = 0, int force_cols = 0);
+                 void* workspace, int64_t workspace_bytes, int cus, hipStream_t stream, int* status);
 // zeroes the first `bytes` of a workspace (a kernel, not a memset: callers may be under graph capture)
 int w8a16_split_clear(void* workspace, int64_t bytes, hipStream_t stream);
 

@@ -867,21 +867,6 @@ extern "C" int hexmi_gemm_w8a16_ws(int64_t M, int64_t N, int64_t K, const void* 
   return hexmi_gemm_w8a16(M, N, K, A, W, scales, C, stream);
 }
 
-#ifdef HEXMI_TUNE
-// measurement hook (not built into the library): the split kernel with a forced decomposition
-extern "C" int hexmi_w8_tune(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
-                             void* C, void* ws, int64_t ws_bytes, int parts, int cols, int clear,
-                             hexmi_stream_t stream) {
-  hipStream_t st = as_stream(stream);
-  int rc = HEXMI_OK;
-  if (clear) rc = w8a16_split_clear(ws, 4096, st);
-  if (!w8a16_split(M, N, K, static_cast<const f16*>(A), W, static_cast<const f16*>(scales), static_cast<f16*>(C), ws,
-                   ws_bytes, hexmi_num_cus(), st, &rc, parts, cols))
-    return HEXMI_ENOTSUP;
-  return rc;
-}
-#endif
-
 extern "C" int hexmi_pack_w8(int64_t N, int64_t K, const int8_t* W, int8_t* Wp, hexmi_stream_t stream) {
   if (N < 0 || K < 0) return HEXMI_EINVAL;
   if (N == 0 || K == 0) return HEXMI_OK;

@@ -406,7 +406,7 @@ struct SplitPlan {
 
 inline int round_up(int64_t v, int to) { return (int)((v + to - 1) / to * to); }
 
-SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int cus, int force_parts = 0, int force_cols = 0) {
+SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int cus) {
   SplitPlan pl = {};
   if (M < 1 || M > 256 || N < 16 || N % 4 != 0 || K < kSlab || K % kSlab != 0 || cus <= 0) return pl;
   if (N > (1 << 24) || K > (1 << 24)) return pl;
@@ -418,11 +418,9 @@ SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int cus, int force_parts =
   // the ranges, the more often A crosses L2); at most 8, each of three slabs or more
   int parts = 1;
   while (parts < 8 && pl.row_tiles * min_cols * parts * 2 <= cus && slabs / (parts * 2) >= 3) parts *= 2;
-  if (force_parts > 0) parts = force_parts;
   if (parts > slabs) parts = slabs;
   int cols = cus / (pl.row_tiles * parts);
   if (cols < min_cols) cols = min_cols;
-  if (force_cols > 0) cols = force_cols < min_cols ? min_cols : force_cols;
   int chan = round_up((N + cols - 1) / cols, 4);
   if (chan < 16) chan = 16;
   cols = (int)((N + chan - 1) / chan);
@@ -452,9 +450,8 @@ int64_t w8a16_split_header(int64_t M, int64_t N, int64_t K, int cus) { return pl
 
 // true: the split kernel took the call (status in *status)
 bool w8a16_split(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,
-                 void* workspace, int64_t workspace_bytes, int cus, hipStream_t st, int* status, int force_parts,
-                 int force_cols) {
-  const SplitPlan pl = plan_split(M, N, K, cus, force_parts, force_cols);
+                 void* workspace, int64_t workspace_bytes, int cus, hipStream_t st, int* status) {
+  const SplitPlan pl = plan_split(M, N, K, cus);
   if (pl.parts == 0) return false;
   if (pl.parts > 1 && (!workspace || workspace_bytes < pl.bytes)) return false;
   if (!aligned_to(A, 16) || !aligned_to(W, 16) || !aligned_to(C, 8) || !aligned_to(workspace, 16)) return false;

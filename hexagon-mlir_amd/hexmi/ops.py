@@ -314,6 +314,8 @@ def _run(name, impl, simple, *args):
         getattr(torch.ops.hexmi, name)(*simple)
     else:
         impl(*args)
+
+
 def _row_strided(t):
     """A 2-D device tensor whose rows are contiguous but not adjacent (a column slice, a padded buffer): the row
     operators read and write it in place through its row stride, as the reference's kernels take a memref with
