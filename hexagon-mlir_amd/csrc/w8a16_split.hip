@@ -47,7 +47,7 @@ struct SplitArgs {
   int chan_per_wg, col_tiles, row_tiles, parts;
   float* partials;                                          // [part][tile][wave][HB][CT][64 lanes][4]
   unsigned* counters;                                       // [tiles][parts]: nonzero once a part's partial tile is out
-  unsigned* error;                                          // set when a bounded wait ran out
+  unsigned* error;                                          // word 0 of the workspace: set when a bounded wait ran out
 };
 
 template <int RB, int CT>
@@ -459,8 +459,8 @@ bool w8a16_split(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W,
   args.A = A; args.W = W; args.scales = scales; args.C = C;
   args.M = (int)M; args.N = (int)N; args.K = (int)K;
   args.chan_per_wg = pl.chan_per_wg; args.col_tiles = pl.col_tiles; args.row_tiles = pl.row_tiles; args.parts = pl.parts;
-  args.counters = static_cast<unsigned*>(workspace);
-  args.error = args.counters + pl.col_tiles * pl.row_tiles * pl.parts;
+  args.error = static_cast<unsigned*>(workspace);          // word 0: where a caller can find it
+  args.counters = args.error + 1;
   args.partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + pl.header_bytes);
   if (pl.rb == 1) *status = launch_split_ct<1>(pl, args, st);
   else if (pl.rb == 2) *status = launch_split_ct<2>(pl, args, st);

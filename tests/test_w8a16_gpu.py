@@ -272,8 +272,12 @@ def test_w8a16_workspace_contract(hexmi):
     a, w, s = _inputs(M, N, K, seed=17)
     ad, wd, sd = a.cuda(), w.cuda(), s.cuda()
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ws.fill_(0xA5)                                            # garbage: the library clears what it needs
     rc, with_ws = _ws_call(hexmi, ad, wd, sd, ws)
     assert rc == 0
+    # word 0 is the guard's error word (no bounded wait expired); the flags behind it are back to zero for the next call
+    header = ws[:1024].view(torch.int32).cpu()
+    assert header[0].item() == 0 and int(header[:64].abs().sum()) == 0
     rc, _ = _ws_call(hexmi, ad, wd, sd, ws, ws_bytes=need - 1)
     assert rc == hexmi._lib.EINVAL
     rc, no_ws = _ws_call(hexmi, ad, wd, sd, None)             # the plain kernels
