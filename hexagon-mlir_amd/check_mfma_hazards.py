@@ -1,14 +1,24 @@
-"""Check the compiled kernels for reads of an accumulator too soon after an inline-assembly MFMA.
+"""Check the compiled kernels for two register hazards that the compiler cannot see through inline assembly.
 
-    python hexagon-mlir_amd/check_mfma_hazards.py            # compiles csrc/gemm.hip and csrc/calibrate.hip to gfx950
-                                                             # assembly and scans it
+    python hexagon-mlir_amd/check_mfma_hazards.py            # compiles the sources below to gfx950 assembly
+                                                             # and scans it
 
-The 16x16x32 MFMAs of the paired-slab GEMM are `asm volatile` (the accumulator is tied to the destination), so the
-compiler's hazard recogniser does not see them and inserts no wait states between such an MFMA and a later read of
-its result (`v_accvgpr_read`, a store from an AGPR, ...). The kernel spends the wait states itself at the end of its
-K loop; this script verifies, on the assembly the compiler actually produced, that every instruction that reads an
-accumulator register is at least NEED wait states behind the last assembly MFMA in layout order (`s_nop k` counts
-k + 1, every other instruction 1; an unconditional branch ends the fall-through). Exit status 1 lists offenders.
+1. Reads of an accumulator too soon after an inline-assembly MFMA. The 16x16x32 MFMAs of the paired-slab GEMM are
+`asm volatile` (the accumulator is tied to the destination), so the compiler's hazard recogniser does not see them
+and inserts no wait states between such an MFMA and a later read of its result (`v_accvgpr_read`, a store from an
+AGPR, ...). The kernel spends the wait states itself at the end of its K loop; `scan` verifies, on the assembly the
+compiler actually produced, that every instruction that reads an accumulator register is at least NEED wait states
+behind the last assembly MFMA in layout order (`s_nop k` counts k + 1, every other instruction 1; an unconditional
+branch ends the fall-through).
+
+2. A matrix instruction that reads a register too soon after an inline-assembly conversion wrote it. A matrix
+instruction must not read a vector register in the two issue slots after a vector instruction wrote it; the compiler
+keeps that distance for its own instructions but cannot see the writes of the SDWA int8 -> fp16 conversions
+(hexmi_common.h). One slot was enough wherever the matrix pipe was idle and lost the last converted byte where the
+pipe was still busy with the MFMA before. `scan_conversions` verifies that every conversion is at least CVT_NEED
+slots ahead of the first matrix instruction that reads its result.
+
+Exit status 1 lists offenders.
 """
 import os
 import re
@@ -58,24 +68,76 @@ def scan(asm_path):
     return bad
 
 
+CVT_NEED = 2       # issue slots between a vector write of a register and a matrix instruction that reads it
+_CVT = re.compile(r"\s*v_cvt_f16_i16_sdwa v(\d+),")
+_MFMA_SRC = re.compile(r"v_mfma\S+ \S+, v\[(\d+):(\d+)\], v\[(\d+):(\d+)\]")
+
+
+def scan_conversions(asm_path, window=400):
+    """{kernel: [(slots, assembly line)]} for conversions whose first matrix-instruction reader is too close."""
+    with open(asm_path) as f:
+        lines = f.read().split("\n")
+    name, bad = None, {}
+    for i, line in enumerate(lines):
+        m = re.match(r"^(_Z\S+):", line)
+        if m:
+            name = m.group(1)
+        m = _CVT.match(line)
+        if not m:
+            continue
+        reg, slots = int(m.group(1)), 0
+        for j in range(i + 1, min(i + window, len(lines))):
+            t = lines[j].strip()
+            if not t or t[0] in ";." or t.endswith(":"):
+                continue
+            mm = _MFMA_SRC.match(t)
+            if mm:
+                a0, a1, b0, b1 = map(int, mm.groups())
+                if a0 <= reg <= a1 or b0 <= reg <= b1:
+                    if slots < CVT_NEED:
+                        bad.setdefault(name, []).append((slots, i + 1))
+                    break
+            if t.startswith("v_cvt_f16_i16_sdwa v%d," % reg) and "UNUSED_PAD" in t:
+                break                                       # the register is written again from scratch
+            if t.split()[0] in ("s_branch", "s_endpgm", "s_setpc_b64") or t.startswith("s_cbranch"):
+                break                                       # control flow: no straight-line distance to measure
+            slots += int(t.split()[1]) + 1 if t.startswith("s_nop") else 1
+    return bad
+
+
 SOURCES = ("gemm.hip", "calibrate.hip")      # the files with MFMAs written as inline assembly
+CVT_SOURCES = ("gemm.hip", "w8a16.hip", "w8a16_split.hip")   # the files that call cvt4 / cvt16
+
+
+def _assembly(name, tmp):
+    out = os.path.join(tmp, name[:-4] + ".s")
+    cmd = [_build.HIPCC] + _build.FLAGS + ["--cuda-device-only", "-S", os.path.join(_build.CSRC, name), "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        sys.exit("hipcc failed:\n" + r.stderr)
+    return out
 
 
 def main():
-    bad = {}
+    import concurrent.futures
+    bad, bad_cvt = {}, {}
+    names = sorted(set(SOURCES) | set(CVT_SOURCES))
     with tempfile.TemporaryDirectory() as tmp:
+        with concurrent.futures.ThreadPoolExecutor(max_workers=len(names)) as ex:
+            outs = dict(zip(names, ex.map(lambda n: _assembly(n, tmp), names)))
         for name in SOURCES:
-            out = os.path.join(tmp, name[:-4] + ".s")
-            cmd = [_build.HIPCC] + _build.FLAGS + ["--cuda-device-only", "-S", os.path.join(_build.CSRC, name), "-o", out]
-            r = subprocess.run(cmd, capture_output=True, text=True)
-            if r.returncode != 0:
-                sys.exit("hipcc failed:\n" + r.stderr)
-            bad.update(scan(out))
+            bad.update(scan(outs[name]))
+        for name in CVT_SOURCES:
+            bad_cvt.update(scan_conversions(outs[name]))
     for k, v in bad.items():
         print("%s: %d accumulator reads too close to an assembly MFMA, first: %d wait states before `%s`"
               % (k, len(v), v[0][0], v[0][1]))
+    for k, v in bad_cvt.items():
+        print("%s: %d conversions too close to the MFMA that reads them, first: %d slot(s), assembly line %d"
+              % (k, len(v), v[0][0], v[0][1]))
     print("kernels with accumulator reads too close to an assembly MFMA: %d" % len(bad))
-    return 1 if bad else 0
+    print("kernels with a conversion too close to its MFMA: %d" % len(bad_cvt))
+    return 1 if bad or bad_cvt else 0
 
 
 if __name__ == "__main__":

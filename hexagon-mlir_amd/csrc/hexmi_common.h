@@ -115,13 +115,25 @@ __device__ __forceinline__ void cvt4(uint32_t w, uint32_t& lo, uint32_t& hi) {
       : "v"(w));
 }
 
-// 16 int8 -> two 8-element fp16 fragments (bytes 0..7 and 8..15).
+// 16 int8 -> two 8-element fp16 fragments (bytes 0..7 and 8..15), as ONE statement that ends in two idle issue
+// slots. A matrix instruction must not read a register in the two slots after a vector instruction wrote it, and
+// the compiler, which keeps that distance for its own instructions, cannot see the writes inside an asm statement:
+// with a conversion one slot ahead of its MFMA, and the matrix pipe still busy with the MFMA before, the MFMA read
+// the register without the last converted byte (k = 11 mod 16 lost in every product; one slot was enough wherever
+// the pipe was idle). Callers of cvt4 keep the distance themselves.
 __device__ __forceinline__ void cvt16(const u32x4& w, f16x8& f0, f16x8& f1) {
   union { uint32_t u[4]; f16x8 f; } a, b;
-  cvt4(w[0], a.u[0], a.u[1]);
-  cvt4(w[1], a.u[2], a.u[3]);
-  cvt4(w[2], b.u[0], b.u[1]);
-  cvt4(w[3], b.u[2], b.u[3]);
+#define HEXMI_CVT4(LO, HI, SRC) \
+      "v_cvt_f16_i16_sdwa " LO ", sext(" SRC ") dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0\n\t" \
+      "v_cvt_f16_i16_sdwa " LO ", sext(" SRC ") dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1\n\t" \
+      "v_cvt_f16_i16_sdwa " HI ", sext(" SRC ") dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_2\n\t" \
+      "v_cvt_f16_i16_sdwa " HI ", sext(" SRC ") dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3\n\t"
+  asm(HEXMI_CVT4("%0", "%1", "%8") HEXMI_CVT4("%2", "%3", "%9") HEXMI_CVT4("%4", "%5", "%10")
+      HEXMI_CVT4("%6", "%7", "%11") "s_nop 1"
+      : "=&v"(a.u[0]), "=&v"(a.u[1]), "=&v"(a.u[2]), "=&v"(a.u[3]), "=&v"(b.u[0]), "=&v"(b.u[1]), "=&v"(b.u[2]),
+        "=&v"(b.u[3])
+      : "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
+#undef HEXMI_CVT4
   f0 = a.f;
   f1 = b.f;
 }

@@ -250,7 +250,12 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
 // converting the same weights, 8 to 10 instructions per MFMA) the kernel took 18.4 us at M = 64, N = 11008, K = 4096,
 // this way 15.0 (22.6 -> 21.1 with the weights coming from HBM). Fragments are read back from LDS in 16-byte chunks
 // permuted inside their row through the copies' source addresses (conflict-free). The K units of a tile are summed
-// through LDS after the K loop, in a fixed order.
+// through LDS after the K loop, in a fixed order, and the tile is stored row by row (one wave, one row's channels).
+// What a launch of this kernel costs besides the stream, from wall-clock stamps inside it (N = 11008, K = 4096,
+// weights from HBM, median workgroup): 0.2-0.4 us to the first copy, 1.3-1.8 us until its data is there, then a
+// chunk every 0.45 us at 16 rows (6.3 TB/s: the HBM rate), 0.73 us at 64 (activations through L2); 0.3 us from the
+// last chunk's barrier to the end of the loop and 0.7 us (16 rows) to 1.9 us (64, 128 rows) for the sum of the K
+// units and the stores.
 // With every CU fetching all of A the kernel moves M * 8 KiB per CU through L2: 29 us at M = 128 (the 128 x 128
 // tile kernel, 86 tiles: 34), but 47 us at M = 256 with 64-k chunks (tile kernel: 37), so it stops at 128 rows.
 constexpr int kMidWeightPolicy = 2;                         // nt: weights are read once (12.4 against 13.0 us at M = 16)
@@ -260,6 +265,8 @@ constexpr int kMidCompute = 12;                             // compute waves: th
 constexpr int kMidWWave0 = 12;                              // first of the four weight-copy waves
 constexpr int kMidMaxM = 128;
 constexpr int mid_kc(int mb) { return mb <= 4 ? 256 : 128; }
+// s_waitcnt immediate (gfx9 encoding) that leaves `vm` vector-memory operations outstanding, LDS counter untouched
+constexpr int wait_vm(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
 // position of 16-byte chunk c inside its row of CH chunks (an involution in c for a given row); rows of 256 and
 // 512 bytes start at the same banks, so the row number itself spreads the chunks
@@ -299,6 +306,14 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   const int n_chunks = K / KC;
   const bool computes = wave < kMidCompute;                 // also copies activations
   const bool copies_w = wave >= kMidWWave0;
+  // The channel scales come from HBM: requested first (older than every copy of this wave, so the counted waits
+  // below see them finished) they are there when the K loop ends; requested after it they are a memory latency
+  // on the way out.
+  f16 my_scale = (f16)0.0f;
+  if (threadIdx.x < kMidCh) {
+    const int gn = n_begin + (int)threadIdx.x;
+    my_scale = scales[gn < n_end ? gn : n_end - 1];
+  }
 
   // ---- copy slots: every copy moves 1 KiB (1024 / row bytes whole rows); lane positions are permuted inside a row
   //      (see the fragment side). Slots past the last real copy repeat one (same bytes, rewritten).
@@ -324,19 +339,24 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     }
   }
   // chunk indices past the end repeat the last chunk (copied, never read): every chunk issues the same copies
-  auto issue_a = [&](int chunk, f16* dst) __attribute__((always_inline)) {
+  // LDS stages by byte address (a stage index counted at run time must not turn into generic pointers)
+  typedef __attribute__((address_space(3))) char* lds_ptr;
+  const unsigned a_lds = (unsigned)(size_t)(lds_ptr)(&a_s[0][0]);
+  const unsigned w_lds = (unsigned)(size_t)(lds_ptr)(&w_s[0][0]);
+  constexpr unsigned kAStage = MB * 16 * KC * 2, kWStage = kMidCh * KC;
+  auto issue_a = [&](int chunk, unsigned dst) __attribute__((always_inline)) {
     const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
 #pragma unroll
     for (int j = 0; j < ASL; ++j)
       __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * KC * 2),
-                                       HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, 0);
+                                       (lds_ptr)(size_t)(dst + slot_dst[j]), 16, 0, 0);
   };
-  auto issue_w = [&](int chunk, int8_t* dst) __attribute__((always_inline)) {
+  auto issue_w = [&](int chunk, unsigned dst) __attribute__((always_inline)) {
     const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
 #pragma unroll
     for (int j = 0; j < WSL; ++j)
       __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * KC),
-                                       HEXMI_LDS(reinterpret_cast<char*>(dst) + slot_dst[j]), 16, 0, kMidWeightPolicy);
+                                       (lds_ptr)(size_t)(dst + slot_dst[j]), 16, 0, kMidWeightPolicy);
   };
 
   // ---- fragment side: compute wave w owns channel tile nt = w % 3, K unit ku and row-block group rg
@@ -362,9 +382,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   // and waited for at the top of the next round, so the LDS latency passes under the conversions and MFMAs. The wait
   // statement names every fragment register as modified: nothing that uses one can be scheduled above it.
   struct Frags { u32x4 raw, a0[RB], a1[RB]; };
-  auto read_frags = [&](Frags& f, const f16* a_src, const int8_t* w_src) __attribute__((always_inline)) {
-    const unsigned a_base = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(a_src);
-    const unsigned w_base = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(w_src);
+  auto read_frags = [&](Frags& f, unsigned a_base, unsigned w_base) __attribute__((always_inline)) {
     asm volatile("ds_read_b128 %0, %1" : "=&v"(f.raw) : "v"(w_base + w_off) : "memory");
     const unsigned a_at0 = a_base + a_off[0], a_at1 = a_base + a_off[1];
 #pragma unroll
@@ -396,100 +414,133 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     for (int rb = 0; rb < RB; ++rb)
       acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, __builtin_bit_cast(f16x8, f.a1[rb]), acc[rb], 0, 0, 0);
   };
-  // s_waitcnt immediates (gfx9 encoding), LDS counter untouched: copies of the newer chunks may stay in flight
-  constexpr int kNewerA = (kMidAStages - 2) * ASL, kNewerW = (WS - 2) * WSL;
-  constexpr int kWaitA = (kNewerA & 0xF) | ((kNewerA >> 4) << 14) | (0x7 << 4) | (0xF << 8);
-  constexpr int kWaitW = (kNewerW & 0xF) | ((kNewerW >> 4) << 14) | (0x7 << 4) | (0xF << 8);
-
   // prologue: activations of chunks 0, 1; weights of chunks 0 .. 3
   if (computes) {
-    issue_a(0, a_s[0]);
-    issue_a(1, a_s[1]);
+    issue_a(0, a_lds);
+    issue_a(1, a_lds + kAStage);
   } else if (copies_w) {
 #pragma unroll
-    for (int i = 0; i < WS - 1; ++i) issue_w(i, w_s[i]);
+    for (int i = 0; i < WS - 1; ++i) issue_w(i, w_lds + i * kWStage);
   }
   // Round u: chunk u+1 has landed for every wave after the barrier (each role waited for its own copies of it) and
   // every wave has the fragments of chunk u in registers, so the stages of chunk u are free: the copies of chunk
   // u+3 (activations) and u+WS (weights) go there. Then the fragments of chunk u+1 are requested and chunk u is
   // multiplied. Round -1 (before the loop) fetches the fragments of chunk 0.
-  constexpr int kWaitA0 = (ASL & 0xF) | ((ASL >> 4) << 14) | (0x7 << 4) | (0xF << 8);                      // chunk 0 landed
-  constexpr int kWaitW0 = (((WS - 2) * WSL) & 0xF) | ((((WS - 2) * WSL) >> 4) << 14) | (0x7 << 4) | (0xF << 8);
-  if (computes) __builtin_amdgcn_s_waitcnt(kWaitA0);
-  else if (copies_w) __builtin_amdgcn_s_waitcnt(kWaitW0);
+  if (computes) __builtin_amdgcn_s_waitcnt(wait_vm(ASL));                  // chunk 0 landed
+  else if (copies_w) __builtin_amdgcn_s_waitcnt(wait_vm((WS - 2) * WSL));
   __builtin_amdgcn_s_barrier();
   Frags fa, fb;
   if (computes) {
-    issue_a(2, a_s[2]);
-    read_frags(fa, a_s[0], w_s[0]);
+    issue_a(2, a_lds + 2 * kAStage);
+    read_frags(fa, a_lds, w_lds);
   } else if (copies_w) {
-    issue_w(WS - 1, w_s[WS - 1]);
+    issue_w(WS - 1, w_lds + (WS - 1) * kWStage);
   }
-  constexpr int kBase = WS % kMidAStages == 0 ? WS : kMidAStages * WS;
-  constexpr int kPeriod = kBase % 2 == 0 ? kBase : 2 * kBase;   // stage and register-buffer assignment repeat
-  // Registers with a read in flight must never be moved: the round's body is straight-line code (the loop is left
-  // with a break, not skipped round by round), the last round requests nothing, and the one pending buffer that
-  // crosses the loop's back edge is waited for first.
-  for (int base = 0; base < n_chunks; base += kPeriod) {
-#pragma unroll
-    for (int u = 0; u < kPeriod; ++u) {
-      const int chunk = base + u;
-      if (chunk >= n_chunks) break;
-      Frags& cur = u % 2 == 0 ? fa : fb;
-      Frags& nxt = u % 2 == 0 ? fb : fa;
-      if (computes) {
-        wait_frags(cur);                                    // fragments of this chunk are in registers
-        __builtin_amdgcn_s_waitcnt(kWaitA);                 // own copies of chunk + 1 have landed
-      } else if (copies_w) {
-        __builtin_amdgcn_s_waitcnt(kWaitW);
-      }
-      // A bare s_barrier: __syncthreads() would add a wait for every outstanding copy and undo the pipelining.
-      __builtin_amdgcn_s_barrier();
-      if (computes) {
-        issue_a(chunk + 3, a_s[u % kMidAStages]);
-        if (chunk + 1 < n_chunks) read_frags(nxt, a_s[(u + 1) % kMidAStages], w_s[(u + 1) % WS]);
-        multiply(cur);
-        if (u == kPeriod - 1 && chunk + 1 < n_chunks) wait_frags(nxt);
-      } else if (copies_w) {
-        issue_w(chunk + WS, w_s[u % WS]);
-      }
+  // The loop is unrolled by two only (the two register buffers alternate); the LDS stages are counted at run time
+  // in scalar registers. A kernel's instruction cache starts cold and a jump to code not yet fetched costs about
+  // half a microsecond here (measured: the exit from the middle of a long unrolled loop to the code behind it), so
+  // the loop is short, every round after the first two runs from the cache, and the way out is a fall through: an
+  // odd last chunk is a copy of the round placed behind the loop, and the sum of the K units follows it in line.
+  // A round with `togo` rounds to go (itself included) copies activations only if togo > 3 and weights only if
+  // togo > 5: nothing is fetched twice and nothing is in flight when the K loop ends. Its waits leave fewer copies
+  // outstanding accordingly; the count of an s_waitcnt is an immediate, so each is a short ladder of uniform
+  // branches with nothing but the wait inside.
+  // Registers with a read in flight must never be moved: apart from those ladders a round's body is straight-line
+  // code, and the buffer whose reads cross the back edge is waited for first. The fragment reads of a round with
+  // nothing behind it fetch a stage nobody multiplies: the same instructions every round.
+  unsigned sa = a_lds, sw = w_lds;                           // stages of the current chunk, as LDS addresses
+  auto round = [&](int chunk, Frags& cur, Frags& nxt, bool reads) __attribute__((always_inline)) {
+    const int togo = n_chunks - chunk;
+    if (computes) {
+      wait_frags(cur);                                      // fragments of this chunk are in registers
+      // own copies of chunk + 1 have landed; those of chunk + 2, if there is one, may be outstanding
+      if (togo >= 3) __builtin_amdgcn_s_waitcnt(wait_vm(ASL));
+      else __builtin_amdgcn_s_waitcnt(wait_vm(0));
+    } else if (copies_w) {
+      // chunk + 1 has landed; up to three younger chunks may be outstanding
+      if (togo >= 5) __builtin_amdgcn_s_waitcnt(wait_vm(3 * WSL));
+      else if (togo == 4) __builtin_amdgcn_s_waitcnt(wait_vm(2 * WSL));
+      else if (togo == 3) __builtin_amdgcn_s_waitcnt(wait_vm(WSL));
+      else __builtin_amdgcn_s_waitcnt(wait_vm(0));
     }
-  }
-  // channel scales of this lane's four outputs: requested here, their latency passes under the sum of the K units
-  f16 sc[4] = {(f16)0, (f16)0, (f16)0, (f16)0};
-  if (computes && ku == 0) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int gn = n_begin + nt * 16 + kg * 4 + e;
-      sc[e] = scales[gn < n_end ? gn : n_end - 1];
+    // A bare s_barrier: __syncthreads() would add a wait for every outstanding copy and undo the pipelining.
+    __builtin_amdgcn_s_barrier();
+    const unsigned sa1 = sa + kAStage == a_lds + kMidAStages * kAStage ? a_lds : sa + kAStage;
+    const unsigned sw1 = sw + kWStage == w_lds + WS * kWStage ? w_lds : sw + kWStage;
+    if (computes) {
+      if (togo > 3) issue_a(chunk + 3, sa);
+      if (reads) read_frags(nxt, sa1, sw1);
+      multiply(cur);
+    } else if (copies_w) {
+      if (togo > WS) issue_w(chunk + WS, sw);
     }
+    sa = sa1;
+    sw = sw1;
+  };
+  static_assert(kMidAStages == 3 && kMidWStages == 5, "the waits of a round are written for these depths");
+  int chunk = 0;
+  for (; chunk + 2 <= n_chunks; chunk += 2) {
+    round(chunk, fa, fb, true);
+    round(chunk + 1, fb, fa, true);
+    if (computes) wait_frags(fa);
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // trailing copies land before the stages are reused
-  __syncthreads();
+  if (chunk < n_chunks) round(chunk, fa, fb, false);
 
-  // the K units of a tile are summed through the activation stages (RB KiB per wave), in the fixed order 0 + 1 + ...
+  // ---- the K units of every tile are summed through LDS and the tile goes out in rows: partial tiles as
+  //      [unit][row][48 channels] fp32 in the activation stages, then compute wave w adds up rows w, w + 12, ... in
+  //      the fixed order unit 0 + 1 + ..., lane = channel, scales them and stores them: a store covers one row's
+  //      channels side by side (a lane's own four outputs are 2-byte pieces of 16 different rows).
+  // After the last round's barrier every wave holds its last fragments in registers and no copy is in flight, so
+  // the stages are free. Only with fewer than three chunks (activations) or five (weights) can a copy of the
+  // prologue, which then repeats the last chunk, still be on its way: the compute waves then wait for theirs and
+  // meet once more before the stages are written, and the copy waves, whose stages nothing below touches, wait for
+  // theirs alone before they end (the LDS is released when the last wave has ended). The barriers are bare
+  // s_barriers with the waits each role needs written out.
+  constexpr int ROWS = MB * 16;
   float* red = reinterpret_cast<float*>(&a_s[0][0]);
-  static_assert((KU - 1) * 3 * MB * 1024 <= kMidAStages * MB * 16 * KC * 2, "the partial tiles fit the activation stages");
-  if (computes && ku > 0) {
-    float* dst = red + (((ku - 1) * 3 + nt) * RG + rg) * RB * 256;
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(dst + (rb * 64 + lane) * 4) = acc[rb];
+  // rows of 52 floats: a wave's 16 rows of four-float pieces then fall on 16 different groups of four banks
+  // (rows of 48 floats put four rows on every group)
+  constexpr int RS = kMidCh + 4;
+  float* sc_s = red + KU * ROWS * RS;                       // the channel scales of this workgroup, as fp32
+  static_assert((KU * ROWS + 1) * RS * 4 <= kMidAStages * ROWS * KC * 2, "the partial tiles fit the activation stages");
+  if (n_chunks < kMidAStages) {
+    if (computes) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
   }
-  if constexpr (KU > 1) __syncthreads();
-  if (computes && ku == 0) {
-    const int gn = n_begin + nt * 16 + kg * 4;
+  if (computes) {
+    if (threadIdx.x < kMidCh) sc_s[threadIdx.x] = (float)my_scale;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      f32x4 sum = acc[rb];
+      const int row = (rg * RB + rb) * 16 + r16;
+      *reinterpret_cast<f32x4*>(red + ((ku * ROWS + row) * RS + nt * 16 + kg * 4)) = acc[rb];
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  if (!computes) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
+  }
+  const int rows = M < ROWS ? M : ROWS;
+  if (lane < n_end - n_begin) {                              // a wave writes one row's channels side by side
+    const float scale = sc_s[lane];
+    constexpr int PASSES = (ROWS + kMidCompute - 1) / kMidCompute;
+    float part[PASSES][KU];
 #pragma unroll
-      for (int q = 1; q < KU; ++q)
-        sum += *reinterpret_cast<const f32x4*>(red + ((((q - 1) * 3 + nt) * RG + rg) * RB * 64 + rb * 64 + lane) * 4);
-      const int gm = (rg * RB + rb) * 16 + r16;
-      if (gm < M) {
+    for (int i = 0; i < PASSES; ++i) {                       // all reads first: one LDS latency, not one per row
+      const int row = wave + i * kMidCompute < ROWS ? wave + i * kMidCompute : ROWS - 1;
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (gn + e < n_end) C[(int64_t)gm * N + gn + e] = (f16)(sum[e] * (float)sc[e]);
-      }
+      for (int q = 0; q < KU; ++q) part[i][q] = red[(q * ROWS + row) * RS + lane];
+    }
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      const int row = wave + i * kMidCompute;
+      float sum = part[i][0];
+#pragma unroll
+      for (int q = 1; q < KU; ++q) sum += part[i][q];
+      if (row < rows) C[(int64_t)row * N + n_begin + lane] = (f16)(sum * scale);
     }
   }
 }

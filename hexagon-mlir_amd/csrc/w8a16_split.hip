@@ -107,6 +107,14 @@ void w8a16_split_kernel(const SplitArgs p) {
     wp[ct] = p.W + (int64_t)n * K + (int64_t)slab0 * kSlab + kh * 64 + kg * 16;
   }
   auto slab_at = [&](int j) { return j < n_slabs ? j : n_slabs - 1; };   // past the end: the last slab again, unused
+  // where the loads past the end of the K part go: kMaxCT KiB of the activation matrix, a different place for
+  // every wave of the grid so that they do not all queue on the same L2 lines
+  const char* idle_src;
+  {
+    const int64_t a_bytes = (int64_t)p.M * K * 2;
+    const int64_t spots = a_bytes >= (kMaxCT + 1) * 1024 ? (a_bytes - kMaxCT * 1024) / 1024 : 1;
+    idle_src = reinterpret_cast<const char*>(p.A) + (((int64_t)blockIdx.x * (kCG * kKH) + wave) % spots) * 1024 + lane * 16;
+  }
 
   // ---- activations: a copy moves 4 rows x 256 bytes; the 16-byte chunk c of row r sits at position c ^ (r % 16)
   const f16* a_src[NAW];
@@ -156,6 +164,12 @@ void w8a16_split_kernel(const SplitArgs p) {
       for (int ct = 0; ct < NCT; ++ct)
         dst[ct] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp[ct] + off));
     };
+    // the same number of loads from a place that is certain to hit L2, results never used
+    auto load_idle = [&](u32x4* dst) __attribute__((always_inline)) {
+#pragma unroll
+      for (int ct = 0; ct < NCT; ++ct)
+        dst[ct] = *reinterpret_cast<const u32x4*>(idle_src + ct * 1024);
+    };
     // dwords [d0, d1) of a slab's 4 * NCT raw dwords -> fragments
     auto widen = [&](const u32x4* w, u32x4 (*dst)[2], int d0, int d1) __attribute__((always_inline)) {
 #pragma unroll
@@ -181,7 +195,14 @@ void w8a16_split_kernel(const SplitArgs p) {
     HEXMI_FENCE;
     load_w(3, raw[0]);
     HEXMI_FENCE;
-    auto slab = [&](int j, const f16* cur, f16* fill, u32x4 (*bcur)[2], u32x4 (*bnxt)[2], u32x4* wnxt) __attribute__((always_inline)) {
+    // last_slabs: one of the last slabs of this K part, whose loads may lie past its end. Every slab issues the
+    // same copies and loads (the waits count them); past the end the activation copy repeats the last slab, an L2
+    // hit, and the weight load reads a piece of the activation matrix instead, which every workgroup has just
+    // pulled through L2: re-reading the last weight slab would be another trip to HBM (they are read past the
+    // caches), four slabs out of a K part's dozen or two, and the end of the loop would wait for it.
+    auto slab = [&](int j, const f16* cur, f16* fill, u32x4 (*bcur)[2], u32x4 (*bnxt)[2], u32x4* wnxt,
+                    auto last_slabs) __attribute__((always_inline)) {
+      constexpr bool LAST = decltype(last_slabs)::value;
       HEXMI_FENCE;
       __builtin_amdgcn_s_waitcnt(wait_vm(2 * NCT + NAW));   // own copies of slab j have landed (and W(j+1))
       __builtin_amdgcn_s_barrier();                         // everyone's have; the stage of slab j-1 is free
@@ -212,26 +233,34 @@ void w8a16_split_kernel(const SplitArgs p) {
         }
       }
       HEXMI_FENCE;
-      load_w(j + 4, wnxt);
+      if (LAST && j + 4 >= n_slabs) load_idle(wnxt);
+      else load_w(j + 4, wnxt);
       HEXMI_FENCE;
     };
-    // Whole rounds of six slabs (three stages and raw slots, two fragment buffers), then the up to five that are
-    // left: no exit from the middle of a round (with one, the compiler loses count of the loads in flight at the
-    // loop head and waits for all of them).
+    // Whole rounds of six slabs (three stages and raw slots, two fragment buffers) as long as every slab of the
+    // round still has four behind it, then the up to nine that are left, each with the tests of a last slab: no
+    // exit from the middle of a round (with one, the compiler loses count of the loads in flight at the loop head
+    // and waits for all of them).
+    constexpr std::false_type kBody{};
+    constexpr std::true_type kLast{};
     int j = 0;
-    for (; j + 6 <= n_slabs; j += 6) {
-      slab(j, a_s0, a_s2, bf[0], bf[1], raw[1]);
-      slab(j + 1, a_s1, a_s0, bf[1], bf[0], raw[2]);
-      slab(j + 2, a_s2, a_s1, bf[0], bf[1], raw[0]);
-      slab(j + 3, a_s0, a_s2, bf[1], bf[0], raw[1]);
-      slab(j + 4, a_s1, a_s0, bf[0], bf[1], raw[2]);
-      slab(j + 5, a_s2, a_s1, bf[1], bf[0], raw[0]);
+    for (; j + 10 <= n_slabs; j += 6) {
+      slab(j, a_s0, a_s2, bf[0], bf[1], raw[1], kBody);
+      slab(j + 1, a_s1, a_s0, bf[1], bf[0], raw[2], kBody);
+      slab(j + 2, a_s2, a_s1, bf[0], bf[1], raw[0], kBody);
+      slab(j + 3, a_s0, a_s2, bf[1], bf[0], raw[1], kBody);
+      slab(j + 4, a_s1, a_s0, bf[0], bf[1], raw[2], kBody);
+      slab(j + 5, a_s2, a_s1, bf[1], bf[0], raw[0], kBody);
     }
-    if (j < n_slabs) slab(j, a_s0, a_s2, bf[0], bf[1], raw[1]);
-    if (j + 1 < n_slabs) slab(j + 1, a_s1, a_s0, bf[1], bf[0], raw[2]);
-    if (j + 2 < n_slabs) slab(j + 2, a_s2, a_s1, bf[0], bf[1], raw[0]);
-    if (j + 3 < n_slabs) slab(j + 3, a_s0, a_s2, bf[1], bf[0], raw[1]);
-    if (j + 4 < n_slabs) slab(j + 4, a_s1, a_s0, bf[0], bf[1], raw[2]);
+    if (j < n_slabs) slab(j, a_s0, a_s2, bf[0], bf[1], raw[1], kLast);
+    if (j + 1 < n_slabs) slab(j + 1, a_s1, a_s0, bf[1], bf[0], raw[2], kLast);
+    if (j + 2 < n_slabs) slab(j + 2, a_s2, a_s1, bf[0], bf[1], raw[0], kLast);
+    if (j + 3 < n_slabs) slab(j + 3, a_s0, a_s2, bf[1], bf[0], raw[1], kLast);
+    if (j + 4 < n_slabs) slab(j + 4, a_s1, a_s0, bf[0], bf[1], raw[2], kLast);
+    if (j + 5 < n_slabs) slab(j + 5, a_s2, a_s1, bf[1], bf[0], raw[0], kLast);
+    if (j + 6 < n_slabs) slab(j + 6, a_s0, a_s2, bf[0], bf[1], raw[1], kLast);
+    if (j + 7 < n_slabs) slab(j + 7, a_s1, a_s0, bf[1], bf[0], raw[2], kLast);
+    if (j + 8 < n_slabs) slab(j + 8, a_s2, a_s1, bf[0], bf[1], raw[0], kLast);
   };
   if (nct == CT) k_loop(std::integral_constant<int, CT>{});
   else if (CT > 2 && nct == 2) k_loop(std::integral_constant<int, (CT > 2 ? 2 : 0)>{});
@@ -410,6 +439,7 @@ SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int cus) {
   SplitPlan pl = {};
   if (M < 1 || M > 256 || N < 16 || N % 4 != 0 || K < kSlab || K % kSlab != 0 || cus <= 0) return pl;
   if (N > (1 << 24) || K > (1 << 24)) return pl;
+  if (M * K * 2 < (kMaxCT + 1) * 1024) return pl;           // the kernel's idle loads read that much of A
   pl.rb = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
   pl.row_tiles = (int)((M + pl.rb * 16 - 1) / (pl.rb * 16));
   const int slabs = (int)(K / kSlab);

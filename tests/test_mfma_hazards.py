@@ -1,5 +1,6 @@
-"""The GEMM's MFMAs are inline assembly, invisible to the compiler's hazard recogniser: the compiled kernels must keep
-every read of an accumulator register far enough behind the last of them. Checked on the assembly hipcc produces
+"""The GEMM's MFMAs and the int8 -> fp16 conversions are inline assembly, invisible to the compiler's hazard
+recogniser: the compiled kernels must keep every read of an accumulator register far enough behind the last such
+MFMA, and every conversion far enough ahead of the MFMA that reads it. Checked on the assembly hipcc produces
 (no GPU needed)."""
 import os
 import sys
@@ -54,6 +55,26 @@ def test_scanner_accepts_spent_wait_states_builtin_mfmas_and_other_paths(tmp_pat
     assert bad == {}
 
 
+def test_scanner_flags_a_conversion_one_slot_ahead_of_its_mfma(tmp_path):
+    text = """\
+        _Zkernel:
+        \tv_cvt_f16_i16_sdwa v41, sext(v8) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_2
+        \tv_cvt_f16_i16_sdwa v41, sext(v8) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3
+        \ts_nop 0
+        \tv_mfma_f32_16x16x32_f16 v[2:5], v[40:43], v[14:17], v[2:5]
+        \ts_endpgm
+        """
+    p = tmp_path / "k.s"
+    p.write_text(textwrap.dedent(text))
+    bad = chk.scan_conversions(str(p))
+    assert list(bad) == ["_Zkernel"] and bad["_Zkernel"][0][0] == 1       # the second conversion: one slot
+    p.write_text(textwrap.dedent(text).replace("s_nop 0", "s_nop 1"))
+    assert chk.scan_conversions(str(p)) == {}
+    # another register, or an MFMA that only writes the register, is no reader
+    p.write_text(textwrap.dedent(text).replace("v[40:43]", "v[44:47]"))
+    assert chk.scan_conversions(str(p)) == {}
+
+
 @pytest.mark.timeout(600)
-def test_compiled_gemm_kernels_keep_their_distance():
+def test_compiled_kernels_keep_their_distance():
     assert chk.main() == 0

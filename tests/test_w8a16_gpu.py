@@ -78,6 +78,18 @@ def test_w8a16_parity(hexmi, oracle, M, N, K):
     assert (got.float() - want.float()).abs().max() / math.sqrt(K) <= 2e-2
 
 
+@pytest.mark.parametrize("M", [9, 16, 32, 48, 64, 100, 128])
+@pytest.mark.parametrize("chunks", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 13])
+def test_w8a16_every_tail_of_the_chunked_kernel(hexmi, oracle, M, chunks):
+    # the chunked kernel (8 < M <= 128) ends its K loop in rounds written out one by one, entered by the number of
+    # chunks left: every entry point and both parities, for every count of row blocks
+    K = 256 * chunks
+    a, w, s = _inputs(M, 100, K, seed=23 + chunks)
+    got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
+    want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w.numpy(), s.numpy()))
+    assert close16(got, want, max_ulp=1, atol=2e-4)
+
+
 @pytest.mark.parametrize("M", [1, 16, 32, 48, 64, 128, 256])
 def test_w8a16_config_sizes(hexmi, oracle, M):
     # measured configuration: N=11008, K=4096; the oracle covers every 43rd output channel, all M rows
