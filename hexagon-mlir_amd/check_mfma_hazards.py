@@ -11,12 +11,12 @@ compiler actually produced, that every instruction that reads an accumulator reg
 behind the last assembly MFMA in layout order (`s_nop k` counts k + 1, every other instruction 1; an unconditional
 branch ends the fall-through).
 
-2. A matrix instruction that reads a register too soon after an inline-assembly conversion wrote it. A matrix
-instruction must not read a vector register in the two issue slots after a vector instruction wrote it; the compiler
-keeps that distance for its own instructions but cannot see the writes of the SDWA int8 -> fp16 conversions
-(hexmi_common.h). One slot was enough wherever the matrix pipe was idle and lost the last converted byte where the
-pipe was still busy with the MFMA before. `scan_conversions` verifies that every conversion is at least CVT_NEED
-slots ahead of the first matrix instruction that reads its result.
+2. A matrix instruction that reads a register too soon after a vector instruction wrote it, where one of the two is
+inline assembly. A matrix instruction must not read a vector register in the two issue slots after a vector
+instruction wrote it; the compiler keeps that distance for the pairs it can see, but it sees neither the writes of
+the SDWA int8 -> fp16 conversions (hexmi_common.h) nor the reads of an assembly MFMA. One slot was enough wherever
+the matrix pipe was idle and lost the last converted byte where the pipe was still busy with the MFMA before.
+`scan_conversions` verifies that no such pair is closer than CVT_NEED slots.
 
 Exit status 1 lists offenders.
 """
@@ -69,44 +69,64 @@ def scan(asm_path):
 
 
 CVT_NEED = 2       # issue slots between a vector write of a register and a matrix instruction that reads it
-_CVT = re.compile(r"\s*v_cvt_f16_i16_sdwa v(\d+),")
 _MFMA_SRC = re.compile(r"v_mfma\S+ \S+, v\[(\d+):(\d+)\], v\[(\d+):(\d+)\]")
+_VALU_DST = re.compile(r"(v_\w+) v(?:\[(\d+):(\d+)\]|(\d+))\b")
 
 
-def scan_conversions(asm_path, window=400):
-    """{kernel: [(slots, assembly line)]} for conversions whose first matrix-instruction reader is too close."""
+def scan_conversions(asm_path):
+    """{kernel: [(slots, assembly line)]}: a matrix instruction reads a vector register fewer than CVT_NEED issue
+    slots after a vector instruction wrote it, where one of the two sits inside an asm statement (the compiler
+    spaces the pairs it can see)."""
     with open(asm_path) as f:
         lines = f.read().split("\n")
-    name, bad = None, {}
+    name, in_asm, bad = None, False, {}
+    recent = []                                             # (slots ago is implied by position) [(lo, hi, hidden, line)]
     for i, line in enumerate(lines):
+        t = line.strip()
         m = re.match(r"^(_Z\S+):", line)
         if m:
-            name = m.group(1)
-        m = _CVT.match(line)
-        if not m:
+            name, recent = m.group(1), []
             continue
-        reg, slots = int(m.group(1)), 0
-        for j in range(i + 1, min(i + window, len(lines))):
-            t = lines[j].strip()
-            if not t or t[0] in ";." or t.endswith(":"):
-                continue
+        if t.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not t or t[0] in ";.":
+            continue
+        if t.endswith(":"):
+            recent = []                                     # a label: other paths arrive here, no distance to measure
+            continue
+        op = t.split()[0]
+        if op.startswith("v_mfma"):
             mm = _MFMA_SRC.match(t)
             if mm:
                 a0, a1, b0, b1 = map(int, mm.groups())
-                if a0 <= reg <= a1 or b0 <= reg <= b1:
-                    if slots < CVT_NEED:
-                        bad.setdefault(name, []).append((slots, i + 1))
-                    break
-            if t.startswith("v_cvt_f16_i16_sdwa v%d," % reg) and "UNUSED_PAD" in t:
-                break                                       # the register is written again from scratch
-            if t.split()[0] in ("s_branch", "s_endpgm", "s_setpc_b64") or t.startswith("s_cbranch"):
-                break                                       # control flow: no straight-line distance to measure
-            slots += int(t.split()[1]) + 1 if t.startswith("s_nop") else 1
+                for age, (lo, hi, hidden, at) in enumerate(reversed(recent)):
+                    if age >= CVT_NEED:
+                        break
+                    if lo is not None and (hidden or in_asm) and (lo <= a1 and hi >= a0 or lo <= b1 and hi >= b0):
+                        bad.setdefault(name, []).append((age, at))
+            recent.append((None, None, False, i + 1))
+        elif op == "s_nop":
+            recent += [(None, None, False, i + 1)] * (int(t.split()[1]) + 1)
+        elif op in ("s_branch", "s_endpgm", "s_setpc_b64") or op.startswith("s_cbranch"):
+            recent = []
+        else:
+            md = _VALU_DST.match(t)
+            if md and not md.group(1).startswith("v_accvgpr_write"):
+                lo = int(md.group(2) if md.group(2) is not None else md.group(4))
+                hi = int(md.group(3) if md.group(3) is not None else md.group(4))
+                recent.append((lo, hi, in_asm, i + 1))
+            else:
+                recent.append((None, None, False, i + 1))
+        recent = recent[-4:]
     return bad
 
 
 SOURCES = ("gemm.hip", "calibrate.hip")      # the files with MFMAs written as inline assembly
-CVT_SOURCES = ("gemm.hip", "w8a16.hip", "w8a16_split.hip")   # the files that call cvt4 / cvt16
+CVT_SOURCES = ("gemm.hip", "calibrate.hip", "w8a16.hip", "w8a16_split.hip")   # asm conversions or asm MFMAs
 
 
 def _assembly(name, tmp):
@@ -133,10 +153,10 @@ def main():
         print("%s: %d accumulator reads too close to an assembly MFMA, first: %d wait states before `%s`"
               % (k, len(v), v[0][0], v[0][1]))
     for k, v in bad_cvt.items():
-        print("%s: %d conversions too close to the MFMA that reads them, first: %d slot(s), assembly line %d"
+        print("%s: %d vector writes too close to the MFMA that reads them, first: %d slot(s), assembly line %d"
               % (k, len(v), v[0][0], v[0][1]))
     print("kernels with accumulator reads too close to an assembly MFMA: %d" % len(bad))
-    print("kernels with a conversion too close to its MFMA: %d" % len(bad_cvt))
+    print("kernels with a vector write too close to the MFMA that reads it: %d" % len(bad_cvt))
     return 1 if bad or bad_cvt else 0
 
 

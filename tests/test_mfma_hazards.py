@@ -55,11 +55,13 @@ def test_scanner_accepts_spent_wait_states_builtin_mfmas_and_other_paths(tmp_pat
     assert bad == {}
 
 
-def test_scanner_flags_a_conversion_one_slot_ahead_of_its_mfma(tmp_path):
+def test_scanner_flags_a_hidden_write_one_slot_ahead_of_its_mfma(tmp_path):
     text = """\
         _Zkernel:
+        \t;;#ASMSTART
         \tv_cvt_f16_i16_sdwa v41, sext(v8) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_2
         \tv_cvt_f16_i16_sdwa v41, sext(v8) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3
+        \t;;#ASMEND
         \ts_nop 0
         \tv_mfma_f32_16x16x32_f16 v[2:5], v[40:43], v[14:17], v[2:5]
         \ts_endpgm
@@ -70,9 +72,22 @@ def test_scanner_flags_a_conversion_one_slot_ahead_of_its_mfma(tmp_path):
     assert list(bad) == ["_Zkernel"] and bad["_Zkernel"][0][0] == 1       # the second conversion: one slot
     p.write_text(textwrap.dedent(text).replace("s_nop 0", "s_nop 1"))
     assert chk.scan_conversions(str(p)) == {}
-    # another register, or an MFMA that only writes the register, is no reader
+    # another register is no reader
     p.write_text(textwrap.dedent(text).replace("v[40:43]", "v[44:47]"))
     assert chk.scan_conversions(str(p)) == {}
+    # a write the compiler can see, read by an MFMA it can see: its own business
+    p.write_text(textwrap.dedent(text).replace("\t;;#ASMSTART\n", "").replace("\t;;#ASMEND\n", ""))
+    assert chk.scan_conversions(str(p)) == {}
+    # a write the compiler can see, read by an assembly MFMA
+    p.write_text(textwrap.dedent("""\
+        _Zkernel:
+        \tv_mov_b32_e32 v40, v9
+        \t;;#ASMSTART
+        \tv_mfma_f32_16x16x32_f16 a[0:3], v[40:43], v[14:17], a[0:3]
+        \t;;#ASMEND
+        \ts_endpgm
+        """))
+    assert chk.scan_conversions(str(p))["_Zkernel"][0][0] == 0
 
 
 @pytest.mark.timeout(600)
