@@ -210,26 +210,59 @@ void w8a16_split_kernel(const SplitArgs p) {
       copy_a(j + 2, fill);
       HEXMI_FENCE;
       if constexpr (NCT > 0) {
-        f16x8 a0 = *reinterpret_cast<const f16x8*>(cur + a_off0);
-        f16x8 a1 = *reinterpret_cast<const f16x8*>(cur + a_off1);
+        // Row blocks in groups of GR: the fragments of group g+1 are requested before the arithmetic of group g and
+        // waited for with a count that leaves them in flight (left to the compiler, every row block waited for the
+        // reads it had just issued: a full LDS latency eight times per slab), and a group's MFMAs run step 0 of
+        // all its row blocks, then step 1, so that independent MFMAs lie between two that update the
+        // same accumulator (GR * NCT >= 3: a 16x16x32 MFMA is in the pipe for two issue slots of 16 cycles). The reads are
+        // assembly for the reason given at wait_group.
+        constexpr int GW = NCT >= 3 ? 1 : NCT == 2 ? 2 : 4;   // three or four MFMAs between two on one accumulator
+        constexpr int GR = RB < GW ? RB : GW;
+        constexpr int NG = RB / GR;
+        static_assert(RB % GR == 0, "whole groups");
+        u32x4 fa[2][GR][2];                                 // [buffer][row block of the group][step]
+        const unsigned at0 = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(cur) + a_off0 * 2;
+        const unsigned at1 = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(cur) + a_off1 * 2;
+        auto read_group = [&](int g, u32x4 (*dst)[2]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          f16x8 n0 = a0, n1 = a1;
-          if (rb + 1 < RB) {                                // the next row block's fragments, under this one's MFMAs
-            n0 = *reinterpret_cast<const f16x8*>(cur + (rb + 1) * 16 * kSlab + a_off0);
-            n1 = *reinterpret_cast<const f16x8*>(cur + (rb + 1) * 16 * kSlab + a_off1);
+          for (int i = 0; i < GR; ++i) {
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(dst[i][0]) : "v"(at0), "n"((g * GR + i) * 16 * kSlab * 2) : "memory");
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(dst[i][1]) : "v"(at1), "n"((g * GR + i) * 16 * kSlab * 2) : "memory");
+          }
+        };
+        // waits until at most `newer` LDS reads are outstanding; names the group's registers as modified so that
+        // nothing that uses them is scheduled above the wait (and nothing moves them while their reads are in flight)
+        auto wait_group = [&](u32x4 (*f)[2], auto newer) __attribute__((always_inline)) {
+          constexpr int NEWER = decltype(newer)::value;
+          if constexpr (GR == 1)
+            asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(f[0][0]), "+v"(f[0][1]) : "n"(NEWER) : "memory");
+          else if constexpr (GR == 2)
+            asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f[0][0]), "+v"(f[0][1]), "+v"(f[1][0]), "+v"(f[1][1]) : "n"(NEWER) : "memory");
+          else
+            asm volatile("s_waitcnt lgkmcnt(%8)" : "+v"(f[0][0]), "+v"(f[0][1]), "+v"(f[1][0]), "+v"(f[1][1]), "+v"(f[2][0]),
+                         "+v"(f[2][1]), "+v"(f[3][0]), "+v"(f[3][1]) : "n"(NEWER) : "memory");
+        };
+        read_group(0, fa[0]);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          u32x4 (*fc)[2] = fa[g % 2];
+          if (g + 1 < NG) {
+            read_group(g + 1, fa[(g + 1) % 2]);
+            wait_group(fc, std::integral_constant<int, 2 * GR>{});
+          } else {
+            wait_group(fc, std::integral_constant<int, 0>{});
           }
           // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
 #pragma unroll
-          for (int ct = 0; ct < NCT; ++ct)
-            acc[rb][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bcur[ct][0]), a0, acc[rb][ct], 0, 0, 0);
+          for (int st = 0; st < 2; ++st)
 #pragma unroll
-          for (int ct = 0; ct < NCT; ++ct)
-            acc[rb][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bcur[ct][1]), a1, acc[rb][ct], 0, 0, 0);
-          widen(wnxt, bnxt, rb * 4 * NCT / RB, (rb + 1) * 4 * NCT / RB);
+            for (int i = 0; i < GR; ++i)
+#pragma unroll
+              for (int ct = 0; ct < NCT; ++ct)
+                acc[g * GR + i][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                    __builtin_bit_cast(f16x8, bcur[ct][st]), __builtin_bit_cast(f16x8, fc[i][st]), acc[g * GR + i][ct], 0, 0, 0);
+          widen(wnxt, bnxt, g * GR * 4 * NCT / RB, (g + 1) * GR * 4 * NCT / RB);
           HEXMI_FENCE;
-          a0 = n0;
-          a1 = n1;
         }
       }
       HEXMI_FENCE;
