@@ -927,6 +927,35 @@ def run_lds_patterns(torch, hexmi, args):
                                        "lds_pattern_kernel", rows, "lds_patterns")), flush=True)
 
 
+def run_l2_stream(torch, hexmi, args):
+    """--workload l2_stream: what the compute units take in from L2 (hexmi_l2_stream): one workgroup of 16 waves per
+    CU streaming a cache-resident region into LDS or into registers, every CU the same region or each its own; the
+    last case streams regions far larger than the caches, for the same loop's rate from HBM."""
+    from hexmi import _lib
+    lib = _lib.lib()
+    cus = lib.hexmi_num_cus()
+    sink = torch.empty(cus * 1024, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for region_kib, shared in ((512, 1), (64, 1), (64, 0), (8192, 0)):     # the last: 2 GiB over the grid, from HBM
+        region = region_kib << 10
+        src = torch.randint(0, 255, (region * (1 if shared else cus),), dtype=torch.uint8, device="cuda")
+        for to_lds in (1, 0):
+            passes = max(1, (2 << 30) // (region * 8))     # 256 MiB through every CU per launch
+            fn = lambda: _lib.check(lib.hexmi_l2_stream(to_lds, shared, region, passes, src.data_ptr(), sink.data_ptr(), st),
+                                    "hexmi_l2_stream")
+            med, best = _time_launch(torch, fn)
+            moved = cus * passes * region
+            rows.append({"region_KiB": region_kib, "every_cu_the_same_region": bool(shared), "into": "LDS" if to_lds else "registers",
+                         "TBs": round(moved / (med * 1e-3) / 1e12, 2), "GBs_per_cu": round(moved / cus / (med * 1e-3) / 1e9, 1),
+                         "launch_ms": round(med, 3), "launch_ms_min": round(best, 3)})
+            print("# %d KiB, %s, into %s: %.1f GB/s per CU" % (region_kib, "shared" if shared else "own region",
+                                                               rows[-1]["into"], rows[-1]["GBs_per_cu"]), file=sys.stderr, flush=True)
+        del src
+    print(json.dumps(_calibration_line(args, "l2_stream", "16 waves per CU streaming an L2-resident region in 1 KiB pieces; "
+                                       "a calibration, not a product kernel", "l2_stream_kernel", rows, "l2_stream")), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -962,6 +991,8 @@ def main():
         return run_issue_slots(torch, hexmi, args)
     if args.workload == "lds_patterns":
         return run_lds_patterns(torch, hexmi, args)
+    if args.workload == "l2_stream":
+        return run_l2_stream(torch, hexmi, args)
     if args.workload == "vendor":
         return run_vendor(torch, hexmi, args)
 

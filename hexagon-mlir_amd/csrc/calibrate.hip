@@ -209,6 +209,42 @@ void lds_pattern_kernel(int pattern, int iters, float* __restrict__ sink) {
   sink[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = (float)(acc[0] ^ acc[1] ^ acc[2] ^ acc[3]);
 }
 
+
+// What a compute unit can take in from L2: 16 waves per workgroup, one workgroup per CU, every wave streaming
+// 1 KiB pieces of a region that stays in L2, either straight into LDS (global_load_lds, the path of the W8A16
+// kernels' activation and weight copies) or into registers. `shared`: every workgroup reads the same region at
+// the same time (activations: one matrix, every CU) or a region of its own. No waits inside the loop: the
+// hardware's queues set the pace.
+template <bool TO_LDS>
+__global__ __launch_bounds__(1024)
+void l2_stream_kernel(const char* __restrict__ src, int64_t region_bytes, int shared, int passes, float* __restrict__ sink) {
+  __shared__ __attribute__((aligned(16))) char stage[64 << 10];
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const char* base = src + (shared ? 0 : (int64_t)blockIdx.x * region_bytes);
+  const int64_t pieces = region_bytes / (16 << 10);          // 16 KiB per workgroup and step
+  u32x4 keep = {0u, 0u, 0u, 0u};
+  for (int p = 0; p < passes; ++p) {
+    for (int64_t i = 0; i < pieces; i += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const char* at = base + ((i + u) % pieces) * (16 << 10) + wave * 1024 + lane * 16;
+        if constexpr (TO_LDS) {
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)at,
+                                           (__attribute__((address_space(3))) void*)(stage + u * (16 << 10) + wave * 1024), 16, 0, 0);
+        } else {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(at);
+          keep[0] ^= v[0]; keep[1] ^= v[1]; keep[2] ^= v[2]; keep[3] ^= v[3];
+        }
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  float out = (float)(keep[0] ^ keep[1] ^ keep[2] ^ keep[3]);
+  if constexpr (TO_LDS) out += (float)stage[threadIdx.x * 16];
+  sink[blockIdx.x * 1024 + threadIdx.x] = out;
+}
+
 }  // namespace
 }  // namespace hexmi
 
@@ -285,5 +321,23 @@ extern "C" int hexmi_lds_read_pattern(int pattern, int64_t iters, float* sink, h
   if (cus <= 0) return HEXMI_ELAUNCH;
   begin_call();
   hipLaunchKernelGGL(lds_pattern_kernel, dim3((unsigned)cus), dim3(1024), 0, as_stream(stream), pattern, (int)iters, sink);
+  return launch_status();
+}
+
+extern "C" int hexmi_l2_stream(int to_lds, int shared, int64_t region_bytes, int64_t passes, const void* src, float* sink,
+                               hexmi_stream_t stream) {
+  if (region_bytes < (64 << 10) || region_bytes % (64 << 10) != 0 || passes < 0 || !src || !sink || !aligned_to(src, 16))
+    return HEXMI_EINVAL;
+  // at most 64 GiB through a compute unit: a few seconds at any rate worth measuring
+  if (passes > HEXMI_CALIBRATE_MAX_ITERS || (double)passes * (double)region_bytes > 64.0 * (1 << 30)) return HEXMI_ETOOBIG;
+  const int cus = hexmi_num_cus();
+  if (cus <= 0) return HEXMI_ELAUNCH;
+  begin_call();
+  if (to_lds)
+    hipLaunchKernelGGL(l2_stream_kernel<true>, dim3((unsigned)cus), dim3(1024), 0, as_stream(stream),
+                       static_cast<const char*>(src), region_bytes, shared, (int)passes, sink);
+  else
+    hipLaunchKernelGGL(l2_stream_kernel<false>, dim3((unsigned)cus), dim3(1024), 0, as_stream(stream),
+                       static_cast<const char*>(src), region_bytes, shared, (int)passes, sink);
   return launch_status();
 }

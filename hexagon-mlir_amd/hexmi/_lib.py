@@ -69,6 +69,7 @@ PROBE_SIGNATURES = {
     "hexmi_mfma_peak": (_int, [_int, _int, _ptr, _i64, _int, _ptr, _ptr]),
     "hexmi_issue_slots": (_int, [_int, _int, _int, _i64, _int, _ptr, _ptr]),
     "hexmi_lds_read_pattern": (_int, [_int, _i64, _ptr, _ptr]),
+    "hexmi_l2_stream": (_int, [_int, _int, _i64, _i64, _ptr, _ptr, _ptr]),
 }
 
 _lib = None

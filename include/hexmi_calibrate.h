@@ -4,7 +4,8 @@
  * and an integrator binds include/hexmi.h only. bench.py uses these entry
  * points to put this GPU's own ceilings (what its matrix cores sustain on given
  * operand data, what vector work hides behind a matrix instruction, what an LDS
- * read pattern costs) on record next to the published peaks.
+ * read pattern costs, what a compute unit takes in from L2) on record next to
+ * the published peaks.
  *
  * Same conventions as hexmi.h (device pointers, stream as void*, int status).
  * Every launch is bounded: iters above HEXMI_CALIBRATE_MAX_ITERS (2^20, about a
@@ -66,6 +67,19 @@ int hexmi_issue_slots(int shape, int kind, int per_mfma, int64_t iters,
                       int waves_per_simd, float *sink, hexmi_stream_t stream);
 int hexmi_lds_read_pattern(int pattern, int64_t iters, float *sink,
                            hexmi_stream_t stream);
+
+/* hexmi_l2_stream: what a compute unit takes in from L2. One workgroup of 16
+ * waves per compute unit streams `region_bytes` (a multiple of 64 KiB) `passes`
+ * times in 1 KiB pieces per wave, to_lds != 0 straight into LDS
+ * (global_load_lds, the path of the W8A16 kernels' copies), else into
+ * registers; shared != 0: every workgroup reads the same region at the same
+ * time, else workgroup b reads [b * region_bytes, (b + 1) * region_bytes) of
+ * src, which must hold hexmi_num_cus() regions. Bytes moved:
+ * hexmi_num_cus() * passes * region_bytes. sink: 1024 floats per compute unit.
+ * passes * region_bytes above 64 GiB is HEXMI_ETOOBIG. */
+int hexmi_l2_stream(int to_lds, int shared, int64_t region_bytes,
+                    int64_t passes, const void *src, float *sink,
+                    hexmi_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -64,3 +64,21 @@ def test_launches_are_bounded():
     assert lib.hexmi_mfma_peak(0, _lib.F16, ops.data_ptr(), too_many, 1, sink.data_ptr(), st) == _lib.ETOOBIG
     assert lib.hexmi_issue_slots(0, 0, 0, too_many, 1, sink.data_ptr(), st) == _lib.ETOOBIG
     assert lib.hexmi_lds_read_pattern(0, too_many, sink.data_ptr(), st) == _lib.ETOOBIG
+
+
+def test_l2_stream_runs_and_is_bounded():
+    lib = _lib.lib()
+    cus = lib.hexmi_num_cus()
+    sink = torch.empty(cus * 1024, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    region = 64 << 10
+    own = torch.zeros(region * cus, dtype=torch.uint8, device="cuda")
+    for to_lds in (0, 1):
+        for shared in (0, 1):
+            assert lib.hexmi_l2_stream(to_lds, shared, region, 4, own.data_ptr(), sink.data_ptr(), st) == _lib.OK
+    torch.cuda.synchronize()
+    assert lib.hexmi_l2_stream(1, 1, region + 1024, 4, own.data_ptr(), sink.data_ptr(), st) == _lib.EINVAL
+    assert lib.hexmi_l2_stream(1, 1, region, -1, own.data_ptr(), sink.data_ptr(), st) == _lib.EINVAL
+    assert lib.hexmi_l2_stream(1, 1, region, 1, None, sink.data_ptr(), st) == _lib.EINVAL
+    assert lib.hexmi_l2_stream(1, 1, region, (1 << 20) + 1, own.data_ptr(), sink.data_ptr(), st) == _lib.ETOOBIG
+    assert lib.hexmi_l2_stream(1, 1, 1 << 30, 1 << 10, own.data_ptr(), sink.data_ptr(), st) == _lib.ETOOBIG
