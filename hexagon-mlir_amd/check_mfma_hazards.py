@@ -1,4 +1,5 @@
-"""Check the compiled kernels for two register hazards that the compiler cannot see through inline assembly.
+"""Check the compiled kernels for register hazards that the compiler cannot see through inline assembly, and for
+register spills where the code cannot afford them.
 
     python hexagon-mlir_amd/check_mfma_hazards.py            # compiles the sources below to gfx950 assembly
                                                              # and scans it
@@ -125,6 +126,40 @@ def scan_conversions(asm_path):
     return bad
 
 
+# 3. Register spills in kernels whose waits are counted by hand. These kernels wait for their global -> LDS copies
+# with `s_waitcnt vmcnt(n)` immediates that assume every outstanding vector-memory operation is one of those copies; a
+# spilled register is reloaded with a vector-memory operation of its own, the count is off by one from then on and
+# a wave reads a stage before its data is there (seen: 192 bytes of scratch in one variant, wrong sums).
+COUNTED_WAITS = ("w8a16_mid_kernel", "w8a16_split_kernel", "w8a16_persist_kernel", "gemm_kernel_k64")
+
+
+def scan_scratch(asm_path):
+    """{kernel: [assembly lines]} for kernels of COUNTED_WAITS with a scratch access between their first and their
+    last global -> LDS copy in layout order (before the first and behind the last, a spill disturbs no count)."""
+    bad, name, copies, scratch = {}, None, [], []
+
+    def close():
+        if name and copies and any(k in name for k in COUNTED_WAITS):
+            inside = [n for n in scratch if copies[0] < n < copies[-1]]
+            if inside:
+                bad[name] = inside
+
+    with open(asm_path) as f:
+        for n, line in enumerate(f, 1):
+            m = re.match(r"^(_Z\S+):", line)
+            if m:
+                close()
+                name, copies, scratch = m.group(1), [], []
+                continue
+            t = line.strip()
+            if re.match(r"(global_load_lds|buffer_load\S*)\b.*\blds\b", t) or t.startswith("global_load_lds"):
+                copies.append(n)
+            elif t.startswith("scratch_"):
+                scratch.append(n)
+    close()
+    return bad
+
+
 SOURCES = ("gemm.hip", "calibrate.hip")      # the files with MFMAs written as inline assembly
 CVT_SOURCES = ("gemm.hip", "calibrate.hip", "w8a16.hip", "w8a16_split.hip")   # asm conversions or asm MFMAs
 
@@ -140,7 +175,7 @@ def _assembly(name, tmp):
 
 def main():
     import concurrent.futures
-    bad, bad_cvt = {}, {}
+    bad, bad_cvt, bad_scratch = {}, {}, {}
     names = sorted(set(SOURCES) | set(CVT_SOURCES))
     with tempfile.TemporaryDirectory() as tmp:
         with concurrent.futures.ThreadPoolExecutor(max_workers=len(names)) as ex:
@@ -149,15 +184,21 @@ def main():
             bad.update(scan(outs[name]))
         for name in CVT_SOURCES:
             bad_cvt.update(scan_conversions(outs[name]))
+        for name in names:
+            bad_scratch.update(scan_scratch(outs[name]))
     for k, v in bad.items():
         print("%s: %d accumulator reads too close to an assembly MFMA, first: %d wait states before `%s`"
               % (k, len(v), v[0][0], v[0][1]))
     for k, v in bad_cvt.items():
         print("%s: %d vector writes too close to the MFMA that reads them, first: %d slot(s), assembly line %d"
               % (k, len(v), v[0][0], v[0][1]))
+    for k, v in bad_scratch.items():
+        print("%s: %d scratch accesses among the copies of a kernel that counts its vector-memory operations by "
+              "hand, first at assembly line %d" % (k, len(v), v[0]))
     print("kernels with accumulator reads too close to an assembly MFMA: %d" % len(bad))
     print("kernels with a vector write too close to the MFMA that reads it: %d" % len(bad_cvt))
-    return 1 if bad or bad_cvt else 0
+    print("kernels with counted waits that spill registers: %d" % len(bad_scratch))
+    return 1 if bad or bad_cvt or bad_scratch else 0
 
 
 if __name__ == "__main__":

@@ -282,7 +282,11 @@ template <int CH> __device__ __forceinline__ int mid_w_pos(int c, int row) {
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 
-template <int MB>
+// NT: channel tiles of 16 in use (a narrow matrix leaves a workgroup fewer than 48 channels): only their weight rows
+// are copied. The compute waves of the other tiles run the same code on whatever their part of the stage holds
+// (their sums are never stored): they are needed for the activation copies and the barriers, and a second code
+// path for them costs the kernel registers it does not have.
+template <int MB, int NT = 3>
 __global__ __launch_bounds__(1024)
 void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
                       f16* __restrict__ C, int M, int N, int K, int chan_per_wg) {
@@ -292,7 +296,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   constexpr int RB = MB / RG;                               // row blocks per compute wave
   static_assert(MB % RG == 0 && RB >= 1 && RB <= 4, "row blocks split evenly over the groups");
   constexpr int ACH = KC / 8, WCH = KC / 16;                // 16-byte chunks per activation / weight row
-  constexpr int NAC = MB * KC / 32, NWC = kMidCh * KC / 1024;   // 1 KiB copies per chunk
+  constexpr int NAC = MB * KC / 32, NWC = NT * 16 * KC / 1024;  // 1 KiB copies per chunk
   constexpr int ASL = (NAC + kMidCompute - 1) / kMidCompute, WSL = (NWC + 3) / 4;   // copy slots per wave
   constexpr int SL = ASL > WSL ? ASL : WSL;
   constexpr int WS = kMidWStages;
@@ -854,11 +858,15 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     if (chan_per_wg < 16) chan_per_wg = 16;
     if (chan_per_wg > kMidCh) chan_per_wg = kMidCh;         // more workgroups than CUs beyond 48 channels per CU
     const int grid = (int)((N + chan_per_wg - 1) / chan_per_wg);
+    const int tiles = (chan_per_wg + 15) / 16;              // channel tiles of a workgroup that hold channels
+#define HEXMI_MID_NT(MB, NT) \
+  hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg)
 #define HEXMI_MID(MB) \
-  hipLaunchKernelGGL(w8a16_mid_kernel<MB>, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg)
-    if (M <= 16) HEXMI_MID(1); else if (M <= 32) HEXMI_MID(2); else if (M <= 48) HEXMI_MID(3); else if (M <= 64) HEXMI_MID(4);
-    else HEXMI_MID(8);
+  { if (tiles == 1) HEXMI_MID_NT(MB, 1); else if (tiles == 2) HEXMI_MID_NT(MB, 2); else HEXMI_MID_NT(MB, 3); }
+    if (M <= 16) HEXMI_MID(1) else if (M <= 32) HEXMI_MID(2) else if (M <= 48) HEXMI_MID(3) else if (M <= 64) HEXMI_MID(4)
+    else HEXMI_MID(8)
 #undef HEXMI_MID
+#undef HEXMI_MID_NT
     return launch_status();
   }
   if (M > 64 && K % 32 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8))

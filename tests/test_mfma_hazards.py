@@ -90,6 +90,25 @@ def test_scanner_flags_a_hidden_write_one_slot_ahead_of_its_mfma(tmp_path):
     assert chk.scan_conversions(str(p))["_Zkernel"][0][0] == 0
 
 
+def test_scanner_flags_scratch_among_the_copies_of_a_kernel_with_counted_waits(tmp_path):
+    p = tmp_path / "k.s"
+    p.write_text(textwrap.dedent("""\
+        _ZN5hexmi16w8a16_mid_kernelILi8ELi1EEEvPKh:
+        \tscratch_store_dword off, v1, off
+        \tglobal_load_lds_dwordx4 v[2:3], off
+        \tscratch_load_dword v1, off, off
+        \tglobal_load_lds_dwordx4 v[2:3], off nt
+        \tscratch_load_dword v1, off, off
+        \ts_endpgm
+        _ZN5hexmi10row_kernelIfEEvPKf:
+        \tglobal_load_lds_dwordx4 v[2:3], off
+        \tscratch_load_dword v1, off, off
+        \tglobal_load_lds_dwordx4 v[2:3], off
+        \ts_endpgm
+        """))
+    assert chk.scan_scratch(str(p)) == {"_ZN5hexmi16w8a16_mid_kernelILi8ELi1EEEvPKh": [4]}
+
+
 @pytest.mark.timeout(600)
 def test_compiled_kernels_keep_their_distance():
     assert chk.main() == 0
