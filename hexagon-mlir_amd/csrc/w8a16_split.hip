@@ -30,6 +30,9 @@ constexpr int kCG = 4, kKH = 2;                             // channel groups x 
 constexpr int kThreads = kCG * kKH * kWave;
 constexpr int kMaxCT = 3;
 constexpr unsigned kSpinLimit = 1u << 22;                   // polls of a counter before a workgroup gives up
+// bytes of one partial tile in the workspace: eight wave regions of (row blocks / 2, at least one) x ct KiB; the
+// kernel's indexing and the size the host asks the caller for both come from here
+constexpr int split_tile_bytes(int rb, int ct) { return kCG * kKH * (rb >= 2 ? rb / 2 : 1) * ct * 1024; }
 
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -46,6 +49,7 @@ struct SplitArgs {
   int M, N, K;
   int chan_per_wg, col_tiles, row_tiles, parts;
   float* partials;                                          // [part][tile][wave][HB][CT][64 lanes][4]
+  unsigned partial_bytes;                                   // size of that area: the buffer descriptor's bound
   unsigned* counters;                                       // [tiles][parts]: nonzero once a part's partial tile is out
   unsigned* error;                                          // word 0 of the workspace: set when a bounded wait ran out
 };
@@ -363,11 +367,13 @@ void w8a16_split_kernel(const SplitArgs p) {
     const int tiles = p.col_tiles * p.row_tiles;
     const int tile = rtile * p.col_tiles + ctile;
     unsigned* flags = p.counters + tile * p.parts;
-    constexpr int kTileBytes = kCG * kKH * kRegion * 4;     // eight wave regions (four when RB == 1: half the space)
+    constexpr int kTileBytes = split_tile_bytes(RB, CT);    // eight wave regions (a single row block uses four of them)
+    static_assert(kTileBytes == kCG * kKH * kRegion * 4, "the regions fill a partial tile");
     unsigned xcc;
     asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID, 0, 4)" : "=s"(xcc));
     const __amdgpu_buffer_rsrc_t rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(p.partials), 0, 0x7fffffff, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(p.partials), 0, (int)p.partial_bytes, 0x00020000);
+    // (bounded by the area's size: an access past it is dropped by the hardware instead of landing in someone's memory)
     const int wave_off = (RB >= 2 ? wave : cg) * kRegion * 4 + lane * 16;
     constexpr int kThrough = 1 | (1 << 4);                  // sc0 sc1: system scope, past both cache levels
     constexpr int kDevice = 1 << 4;                         // sc1: device scope, served by this XCD's L2
@@ -493,7 +499,7 @@ SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int cus) {
   pl.ct = (chan + 63) / 64;
   const int64_t tiles = (int64_t)cols * pl.row_tiles;
   pl.header_bytes = round_up((tiles * parts + 1) * 4, 256);
-  pl.bytes = parts > 1 ? pl.header_bytes + (int64_t)parts * tiles * kCG * pl.rb * pl.ct * 1024 : 0;
+  pl.bytes = parts > 1 ? pl.header_bytes + (int64_t)parts * tiles * split_tile_bytes(pl.rb, pl.ct) : 0;
   return pl;
 }
 
@@ -525,6 +531,7 @@ bool w8a16_split(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W,
   args.error = static_cast<unsigned*>(workspace);          // word 0: where a caller can find it
   args.counters = args.error + 1;
   args.partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + pl.header_bytes);
+  args.partial_bytes = (unsigned)(pl.bytes > pl.header_bytes ? pl.bytes - pl.header_bytes : 0);
   if (pl.rb == 1) *status = launch_split_ct<1>(pl, args, st);
   else if (pl.rb == 2) *status = launch_split_ct<2>(pl, args, st);
   else if (pl.rb == 4) *status = launch_split_ct<4>(pl, args, st);
