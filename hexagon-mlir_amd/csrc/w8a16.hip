@@ -124,9 +124,10 @@ void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const
   }
 }
 
-// Up to 16 activation rows, K <= 4096 (used for M <= 8, and for M <= 16 on pre-packed weights; 9 .. 16 rows of
-// plain weights go through the chunked kernel further down): persistent workgroups of 16 waves, one per compute unit. The per-CU rate
-// of the 16-row strided weight reads is what bounds this shape, so the output channels are dealt in equal
+// Up to 16 activation rows on pre-packed weights, K <= 4096 (plain weights go through the chunked kernel further
+// down, which is faster at every row count: 11.3 against 11.8-12.3 us at M = 4 and 8, N = 11008, K = 4096; 6.9
+// against 8.6 at N = K = 4096): persistent workgroups of 16 waves, one per compute unit. The per-CU rate
+// of the weight reads is what bounds this shape, so the output channels are dealt in equal
 // contiguous ranges over exactly as many workgroups as there are CUs (N = 11008 on 256 CUs: 43 channels each,
 // walked as tiles of 16, 16 and 11 channels; the lanes of a short tile re-read its last row and drop the result).
 // Wave w owns the K slice [w*K/16, (w+1)*K/16) of every tile of its workgroup: it needs only a 16 x K/16 slice of
@@ -139,9 +140,8 @@ void w8a16_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const
 constexpr int kPWaves = 16;
 constexpr int kPTiles = 3;                                  // tiles per workgroup per pass
 constexpr int kPSteps = 4;                                  // 64-wide steps per wave: K <= 16 * 4 * 64
-// PACKED: W is the fragment-major layout written by pack_w8_kernel (chan_per_wg is then a multiple of 16): the
-// 16 rows x 64 k of a tile step are one contiguous KiB in lane order, so a wave's loads are fully contiguous.
-template <bool PACKED>
+// W is the fragment-major layout written by pack_w8_kernel (chan_per_wg is a multiple of 16): the 16 rows x 64 k
+// of a tile step are one contiguous KiB in lane order, so a wave's loads are fully contiguous.
 __global__ __launch_bounds__(1024)
 void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
                           f16* __restrict__ C, int M, int N, int K, int chan_per_wg) {
@@ -167,25 +167,14 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
     u32x4 wv[kPTiles][kPSteps];
 #pragma unroll
     for (int q = 0; q < kPTiles; ++q) {
-      if constexpr (PACKED) {
-        int tile = base / 16 + q;
-        const int last = (N + 15) / 16 - 1;
-        tile = tile <= last ? tile : last;                  // past the end: re-read the last tile, unused
-        const int8_t* blk = W + ((int64_t)tile * (K / 64) + (int64_t)wave * steps) * 1024 + lane * 16;
+      int tile = base / 16 + q;
+      const int last = (N + 15) / 16 - 1;
+      tile = tile <= last ? tile : last;                    // past the end: re-read the last tile, unused
+      const int8_t* blk = W + ((int64_t)tile * (K / 64) + (int64_t)wave * steps) * 1024 + lane * 16;
 #pragma unroll
-        for (int u = 0; u < kPSteps; ++u) {
-          const int st = u < steps ? u : steps - 1;
-          wv[q][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(blk + st * 1024));
-        }
-      } else {
-        int n = base + q * 16 + r16;
-        n = n < n_end ? n : n_end - 1;                      // past the range: re-read its last row, unused
-        const int8_t* wrow = W + (int64_t)n * K + (int64_t)wave * ksl + kg * 16;
-#pragma unroll
-        for (int u = 0; u < kPSteps; ++u) {
-          const int st = u < steps ? u : steps - 1;
-          wv[q][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + st * 64));
-        }
+      for (int u = 0; u < kPSteps; ++u) {
+        const int st = u < steps ? u : steps - 1;
+        wv[q][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(blk + st * 1024));
       }
     }
     // this wave's activation slice: rows r16, k in [wave*ksl + u*64 + kg*16, +16)
@@ -234,16 +223,17 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
   }
 }
 
-// 16 < M <= 128 (MB = 2..8 blocks of 16 activation rows), K % 256 == 0: one persistent workgroup of 16 waves per
-// CU, each owning an equal contiguous range of at most 48 output channels, so the weights cross HBM once, in
-// contiguous row segments. K is walked in chunks of KC = 256 (MB <= 4) or 128 (MB = 8): an activation chunk is at
-// most 32 KiB. The raw int8 weight chunk [48][KC] and the activation chunk [MB*16][KC] fp16 are copied
+// 2 < M <= 128 (MB = 1..8 blocks of 16 activation rows; K % 256 == 0, or any multiple of 64 with MB = 1): persistent
+// workgroups of 16 waves, each owning an equal contiguous range of at most 48 output channels, so the weights cross
+// HBM once, in contiguous row segments. K is walked in chunks of KC = 256 (MB <= 4) or 128 (MB = 8): an activation
+// chunk is at most 32 KiB; with MB = 1 and one or two channel tiles the chunks are 768 and 384 k long (mid_kc()). The raw int8 weight chunk [48][KC] and the activation chunk [MB*16][KC] fp16 are copied
 // global -> LDS (global_load_lds, no registers) by different waves: waves 12..15 copy weights, four chunks ahead
 // (five stages: three or four measured the same, seven and nine 5-10 % slower), waves 0..11 copy activations, two
 // chunks ahead (three stages; L2 hits). A wave's outstanding-copy counter only sees its own copies, so each role
 // waits with its own count and the workgroup barrier publishes both.
 // Compute wave w < 12 owns channel tile w % 3 and, of every chunk, one unit of 64 k for one group of row blocks
-// (four K units and all row blocks at KC = 256; two units and two groups of four row blocks at KC = 128). It converts
+// (four K units and all row blocks at KC = 256; two units and two groups of four row blocks at KC = 128; twelve
+// units of one tile at KC = 768 and six of each of two tiles at KC = 384, where no wave is left over). It converts
 // its 16 x 64 int8 weights to fp16 once per chunk (16 vector instructions) and multiplies them into its RB
 // accumulators (2 * RB MFMAs). A SIMD issues one instruction at a time and a 16x16x32 MFMA hides only two vector
 // instructions, so the conversions per MFMA set the pace: with one 16 x 16 tile per wave (every row-block wave
@@ -264,19 +254,23 @@ constexpr int kMidAStages = 3, kMidWStages = 5;
 constexpr int kMidCompute = 12;                             // compute waves: three channel tiles x four (unit, group)
 constexpr int kMidWWave0 = 12;                              // first of the four weight-copy waves
 constexpr int kMidMaxM = 128;
-constexpr int mid_kc(int mb) { return mb <= 4 ? 256 : 128; }
+// K per chunk. Sixteen rows leave LDS for longer chunks, and a workgroup with one or two channel tiles needs them:
+// what a CU has in flight is four chunks of weights, 16 KiB with one tile of 256 k, too little to keep HBM busy
+// (N = 4096, K = 11008, M = 16: 19.1 us), 48 KiB with 768 k.
+constexpr int mid_kc(int mb, int nt) { return mb == 1 ? (nt == 1 ? 768 : nt == 2 ? 384 : 256) : mb <= 4 ? 256 : 128; }
 // s_waitcnt immediate (gfx9 encoding) that leaves `vm` vector-memory operations outstanding, LDS counter untouched
 constexpr int wait_vm(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
 // position of 16-byte chunk c inside its row of CH chunks (an involution in c for a given row); rows of 256 and
 // 512 bytes start at the same banks, so the row number itself spreads the chunks
 template <int CH> __device__ __forceinline__ int mid_a_pos(int c, int row) {
-  if constexpr (CH == 32) return (c & 16) | ((c ^ row) & 15);
-  else return (c ^ row) & 15;
+  static_assert(CH % 16 == 0, "activation rows are whole bank cycles of 256 bytes");
+  return (c & ~15) | ((c ^ row) & 15);
 }
 template <int CH> __device__ __forceinline__ int mid_w_pos(int c, int row) {
-  if constexpr (CH == 16) return (c ^ row) & 15;
-  else return (c ^ (row >> 1)) & 7;                         // 128-byte rows read as chunk 4u + g
+  if constexpr (CH % 16 == 0) return (c & ~15) | ((c ^ row) & 15);
+  // rows of 128 or 384 bytes: consecutive rows start half a bank cycle apart, so pairs of rows share the low bits
+  else return (c & ~7) | ((c ^ (row >> 1)) & 7);
 }
 
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
@@ -286,13 +280,19 @@ template <int CH> __device__ __forceinline__ int mid_w_pos(int c, int row) {
 // are copied. The compute waves of the other tiles run the same code on whatever their part of the stage holds
 // (their sums are never stored): they are needed for the activation copies and the barriers, and a second code
 // path for them costs the kernel registers it does not have.
-template <int MB, int NT = 3>
-__global__ __launch_bounds__(1024)
+// KC: K per chunk. With sixteen rows (MB = 1) K need not be a multiple of it: copies of a last, shorter chunk are
+// clamped to the row and the 64-k units past K are multiplied as zeros.
+template <int MB, int NT = 3, int KC = mid_kc(MB, NT)>
+__global__ __launch_bounds__(1024, (MB == 1 && NT == 2 && KC == 256) ? 8 : 4)
 void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
-                      f16* __restrict__ C, int M, int N, int K, int chan_per_wg) {
-  constexpr int KC = mid_kc(MB);
+                      f16* __restrict__ C, int M, int N, int K, int chan_per_wg, int rotate) {
   constexpr int KU = KC / 64;                               // 64-k units per chunk
-  constexpr int RG = 4 / KU;                                // row-block groups
+  // channel-tile slots the twelve compute waves are laid out for: the tiles in use when their units take all
+  // twelve, else three (the waves of a slot without channels run along)
+  constexpr int TS = NT * KU == kMidCompute ? NT : 3;
+  constexpr int RG = kMidCompute / TS / KU;                 // row-block groups
+  constexpr bool TAIL = MB == 1;                            // K % KC != 0 allowed
+  static_assert(TS * KU * RG == kMidCompute && KC % 64 == 0, "every compute wave has a tile slot, a unit and a group");
   constexpr int RB = MB / RG;                               // row blocks per compute wave
   static_assert(MB % RG == 0 && RB >= 1 && RB <= 4, "row blocks split evenly over the groups");
   constexpr int ACH = KC / 8, WCH = KC / 16;                // 16-byte chunks per activation / weight row
@@ -301,13 +301,22 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   constexpr int SL = ASL > WSL ? ASL : WSL;
   constexpr int WS = kMidWStages;
   __shared__ __attribute__((aligned(16))) f16 a_s[kMidAStages][MB * 16 * KC];
-  __shared__ __attribute__((aligned(16))) int8_t w_s[WS][kMidCh * KC];
+  __shared__ __attribute__((aligned(16))) int8_t w_s[WS][NT * 16 * KC];
 
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int r16 = lane % 16, kg = lane / 16;
   const int n_begin = blockIdx.x * chan_per_wg;
   const int n_end = n_begin + chan_per_wg < N ? n_begin + chan_per_wg : N;
-  const int n_chunks = K / KC;
+  const int n_chunks = TAIL ? (K + KC - 1) / KC : K / KC;
+  // Workgroup b walks K from chunk b % n_chunks on and wraps round. With every workgroup at the same k at the
+  // same time, all the addresses in flight on the chip agree in their low bits when the weight rows are a power of
+  // two long, and the memory channels those bits select take the whole load (N = 8192, M = 16: 20.9 us at
+  // K = 8192, 14.2 at 7936, 15.0 at 8320). The order of a channel's sum so depends on the workgroup it falls in.
+  // Not with two workgroups per CU at a time (rotate = 0): there it costs 4-7 %.
+  const int rot = rotate ? (int)(blockIdx.x % (unsigned)n_chunks) : 0;
+  auto k_chunk = [&](int chunk) __attribute__((always_inline)) {
+    return chunk + rot < n_chunks ? chunk + rot : chunk + rot - n_chunks;
+  };
   const bool computes = wave < kMidCompute;                 // also copies activations
   const bool copies_w = wave >= kMidWWave0;
   // The channel scales come from HBM: requested first (older than every copy of this wave, so the counted waits
@@ -323,23 +332,29 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   //      (see the fragment side). Slots past the last real copy repeat one (same bytes, rewritten).
   const char* slot_src[SL];                                 // source of this lane for chunk 0
   int slot_dst[SL];                                         // byte offset of the copy inside its stage
+  int slot_lim[SL];                                         // largest chunk offset that keeps this lane inside its row
 #pragma unroll
   for (int j = 0; j < SL; ++j) {
     slot_src[j] = nullptr;
     slot_dst[j] = 0;
+    slot_lim[j] = 0;
     if (computes && j < ASL) {
       const int i = (j * kMidCompute + wave) % NAC;
-      const int row = i * (64 / ACH) + lane / ACH;          // 64 chunks per copy
-      const int src_c = mid_a_pos<ACH>(lane % ACH, row);    // the chunk that belongs at this position
+      const int f = i * 64 + lane;                          // 16-byte piece of the stage: 64 per copy
+      const int row = f / ACH;
+      const int src_c = mid_a_pos<ACH>(f % ACH, row);       // the chunk that belongs at this position
       slot_src[j] = reinterpret_cast<const char*>(A + (int64_t)(row < M ? row : M - 1) * K) + src_c * 16;
       slot_dst[j] = i * 1024;
+      slot_lim[j] = K * 2 - 16 - src_c * 16;
     } else if (copies_w && j < WSL) {
       const int t = (j * 4 + (wave - kMidWWave0)) % NWC;
-      const int row = t * (64 / WCH) + lane / WCH;
-      const int src_c = mid_w_pos<WCH>(lane % WCH, row);
+      const int f = t * 64 + lane;
+      const int row = f / WCH;
+      const int src_c = mid_w_pos<WCH>(f % WCH, row);
       const int n = n_begin + row < n_end ? n_begin + row : n_end - 1;
       slot_src[j] = reinterpret_cast<const char*>(W + (int64_t)n * K) + src_c * 16;
       slot_dst[j] = t * 1024;
+      slot_lim[j] = K - 16 - src_c * 16;
     }
   }
   // chunk indices past the end repeat the last chunk (copied, never read): every chunk issues the same copies
@@ -347,29 +362,35 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   typedef __attribute__((address_space(3))) char* lds_ptr;
   const unsigned a_lds = (unsigned)(size_t)(lds_ptr)(&a_s[0][0]);
   const unsigned w_lds = (unsigned)(size_t)(lds_ptr)(&w_s[0][0]);
-  constexpr unsigned kAStage = MB * 16 * KC * 2, kWStage = kMidCh * KC;
+  constexpr unsigned kAStage = MB * 16 * KC * 2, kWStage = NT * 16 * KC;
+  // With TAIL a lane whose piece of the last chunk lies past K fetches the last 16 bytes of its row instead (never
+  // multiplied: see the mask in multiply()).
   auto issue_a = [&](int chunk, unsigned dst) __attribute__((always_inline)) {
-    const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
+    const int ck = k_chunk(chunk < n_chunks ? chunk : n_chunks - 1);
 #pragma unroll
-    for (int j = 0; j < ASL; ++j)
-      __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * KC * 2),
-                                       (lds_ptr)(size_t)(dst + slot_dst[j]), 16, 0, 0);
+    for (int j = 0; j < ASL; ++j) {
+      const int off = ck * (KC * 2);
+      const char* src = TAIL ? slot_src[j] + (off < slot_lim[j] ? off : slot_lim[j]) : slot_src[j] + (int64_t)ck * (KC * 2);
+      __builtin_amdgcn_global_load_lds(HEXMI_GLB(src), (lds_ptr)(size_t)(dst + slot_dst[j]), 16, 0, 0);
+    }
   };
   auto issue_w = [&](int chunk, unsigned dst) __attribute__((always_inline)) {
-    const int ck = chunk < n_chunks ? chunk : n_chunks - 1;
+    const int ck = k_chunk(chunk < n_chunks ? chunk : n_chunks - 1);
 #pragma unroll
-    for (int j = 0; j < WSL; ++j)
-      __builtin_amdgcn_global_load_lds(HEXMI_GLB(slot_src[j] + (int64_t)ck * KC),
-                                       (lds_ptr)(size_t)(dst + slot_dst[j]), 16, 0, kMidWeightPolicy);
+    for (int j = 0; j < WSL; ++j) {
+      const int off = ck * KC;
+      const char* src = TAIL ? slot_src[j] + (off < slot_lim[j] ? off : slot_lim[j]) : slot_src[j] + (int64_t)ck * KC;
+      __builtin_amdgcn_global_load_lds(HEXMI_GLB(src), (lds_ptr)(size_t)(dst + slot_dst[j]), 16, 0, kMidWeightPolicy);
+    }
   };
 
   // ---- fragment side: compute wave w owns channel tile nt = w % 3, K unit ku and row-block group rg
-  const int nt = wave % 3, ku = (wave / 3) % KU, rg = (wave / 3) / KU;
+  const int nt = wave % TS, ku = (wave / TS) % KU, rg = (wave / TS) / KU;
   // A chunk's position depends on the row only through its low four bits, so row block rb of the group is a
   // constant 16 * KC * 2 * rb bytes further: an immediate offset of the read, not a register.
   int w_off, a_off[2];
   {
-    const int wrow = nt * 16 + r16;
+    const int wrow = (nt < NT ? nt : 0) * 16 + r16;          // a tile without channels reads tile 0's part of the stage
     w_off = wrow * KC + mid_w_pos<WCH>(ku * 4 + kg, wrow) * 16;
     const int arow = rg * RB * 16 + r16;
 #pragma unroll
@@ -407,9 +428,16 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     else
       asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.raw), "+v"(f.a0[0]), "+v"(f.a1[0]) :: "memory");
   };
-  auto multiply = [&](const Frags& f) __attribute__((always_inline)) {
+  auto multiply = [&](const Frags& f, int chunk) __attribute__((always_inline)) {
     f16x8 w0, w1;
-    cvt16(f.raw, w0, w1);                                   // converted once, used for every row block
+    if constexpr (TAIL) {
+      // a unit past the end of K holds the bytes its copies were clamped to: its weights count as zeros
+      const unsigned keep = k_chunk(chunk) * KC + ku * 64 < K ? 0xffffffffu : 0u;
+      const u32x4 raw = {f.raw[0] & keep, f.raw[1] & keep, f.raw[2] & keep, f.raw[3] & keep};
+      cvt16(raw, w0, w1);
+    } else {
+      cvt16(f.raw, w0, w1);                                 // converted once, used for every row block
+    }
     // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
@@ -474,7 +502,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     if (computes) {
       if (togo > 3) issue_a(chunk + 3, sa);
       if (reads) read_frags(nxt, sa1, sw1);
-      multiply(cur);
+      multiply(cur, chunk);
     } else if (copies_w) {
       if (togo > WS) issue_w(chunk + WS, sw);
     }
@@ -799,7 +827,10 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
   f16* c = static_cast<f16*>(C);
   begin_call();
   if (K == 0) return fill_zero_2d(C, M, N, N, 2, st);      // an empty sum
-  if (M <= 2 && K % 16 == 0 && K <= 16384 && K != 1024 && K != 2048 && K != 4096 && K != 8192 && aligned_to(A, 16) &&
+  // two rows over a long K and at least 16 channels per CU go faster through the chunked kernel further down
+  // (N = 4096, K = 11008: 11.2 against 12.9 us; N = K = 8192: 14.1 against 18.0)
+  const bool chunked_pair = M == 2 && K >= 8192 && K % 64 == 0 && N >= 4096 && aligned_to(A, 16) && aligned_to(W, 16);
+  if (M <= 2 && !chunked_pair && K % 16 == 0 && K <= 16384 && K != 1024 && K != 2048 && K != 4096 && K != 8192 && aligned_to(A, 16) &&
       aligned_to(W, 16)) {
     // any other row length: the masked form of the same kernel, instantiated per KiB of row
     const unsigned blocks = (unsigned)((N + 15) / 16);
@@ -826,7 +857,7 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
                        c, (int)M, (int)N, (int)K);
     return launch_status();
   }
-  if (M <= 2 && (K == 1024 || K == 2048 || K == 4096 || K == 8192)) {
+  if (M <= 2 && !chunked_pair && (K == 1024 || K == 2048 || K == 4096 || K == 8192)) {
     // one channel per wave, eight waves per workgroup: measured against two and four channels per wave and
     // workgroups of two, four and sixteen waves at N = 11008, K = 4096 (0.60 of the HBM figure against 0.57 for two
     // channels x four waves on the same box)
@@ -839,34 +870,44 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
 #undef HEXMI_GEMV
     return launch_status();
   }
-  // up to 8 rows; 9 .. 16 rows stream faster through the chunked kernel below (12.6 against 13.8 us at M = 16,
-  // N = 11008, K = 4096 with the weights from HBM; 12.5 against 12.1 at M = 4)
-  if (M <= 8 && K % (kPWaves * 64) == 0 && K / (kPWaves * 64) <= kPSteps) {
+  // the chunked kernel: K in whole chunks of 256, or any K (a multiple of 64 here) with up to 16 rows
+  if (M <= kMidMaxM && (K % 256 == 0 || M <= 16) && K <= (1 << 29)) {
     const int cus = hexmi_num_cus();
     if (cus <= 0) return HEXMI_ELAUNCH;
-    int chan_per_wg = (int)((N + cus - 1) / cus);
-    if (chan_per_wg < 16) chan_per_wg = 16;                 // one full tile at least
-    const int grid = (int)((N + chan_per_wg - 1) / chan_per_wg);
-    hipLaunchKernelGGL(w8a16_persist_kernel<false>, dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K,
-                       chan_per_wg);
-    return launch_status();
-  }
-  if (M <= kMidMaxM && K % 256 == 0 && N <= 0x7fffffff) {
-    const int cus = hexmi_num_cus();
-    if (cus <= 0) return HEXMI_ELAUNCH;
-    int chan_per_wg = (int)((N + cus - 1) / cus);
-    if (chan_per_wg < 16) chan_per_wg = 16;
-    if (chan_per_wg > kMidCh) chan_per_wg = kMidCh;         // more workgroups than CUs beyond 48 channels per CU
-    const int grid = (int)((N + chan_per_wg - 1) / chan_per_wg);
+    const int64_t per_cu = (N + cus - 1) / cus;
+    int chan_per_wg = (int)(per_cu < 16 ? 16 : per_cu);     // one full tile at least
+    bool paired = false;
+    if (per_cu > kMidCh) {
+      // More than a workgroup's 48 channels per CU: equal workgroups in whole rounds over the CUs, not 48 each and
+      // a last round of a few (N = 14336, K = 4096, M = 16: 19.3 us that way). Either one workgroup per CU at a
+      // time, of up to three channel tiles, or, with up to 16 rows, two of up to two tiles each (their LDS fits
+      // twice, so their starts and ends overlap: 14.8 us); whichever copies fewer tile rows, empty ones counted.
+      const int64_t r1 = (per_cu + kMidCh - 1) / kMidCh, c1 = (N + cus * r1 - 1) / (cus * r1);
+      chan_per_wg = (int)c1;
+      if (M <= 16) {
+        const int64_t r2 = (per_cu + 63) / 64, c2 = (N + cus * 2 * r2 - 1) / (cus * 2 * r2);
+        if (c2 > 16 && r2 * 2 * ((c2 + 15) / 16) <= r1 * ((c1 + 15) / 16)) {
+          chan_per_wg = (int)c2;
+          paired = true;
+        }
+      }
+    }
+    const int64_t grid64 = (N + chan_per_wg - 1) / chan_per_wg;
+    if (grid64 > 0x7fffffff) return HEXMI_ENOTSUP;
+    const int grid = (int)grid64;
     const int tiles = (chan_per_wg + 15) / 16;              // channel tiles of a workgroup that hold channels
-#define HEXMI_MID_NT(MB, NT) \
-  hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg)
+#define HEXMI_MID_KC(MB, NT, KC) \
+  hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT, KC>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg, paired ? 0 : 1)
+#define HEXMI_MID_NT(MB, NT) HEXMI_MID_KC(MB, NT, mid_kc(MB, NT))
 #define HEXMI_MID(MB) \
   { if (tiles == 1) HEXMI_MID_NT(MB, 1); else if (tiles == 2) HEXMI_MID_NT(MB, 2); else HEXMI_MID_NT(MB, 3); }
-    if (M <= 16) HEXMI_MID(1) else if (M <= 32) HEXMI_MID(2) else if (M <= 48) HEXMI_MID(3) else if (M <= 64) HEXMI_MID(4)
+    if (M <= 16) {
+      if (paired) HEXMI_MID_KC(1, 2, 256); else HEXMI_MID(1)
+    } else if (M <= 32) HEXMI_MID(2) else if (M <= 48) HEXMI_MID(3) else if (M <= 64) HEXMI_MID(4)
     else HEXMI_MID(8)
 #undef HEXMI_MID
 #undef HEXMI_MID_NT
+#undef HEXMI_MID_KC
     return launch_status();
   }
   if (M > 64 && K % 32 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8))
@@ -961,7 +1002,7 @@ extern "C" int hexmi_gemm_w8a16_packed(int64_t M, int64_t N, int64_t K, const vo
   int rc = HEXMI_OK;
   for (int64_t m = 0; m < M && rc == HEXMI_OK; m += 16) {
     const int rows = (int)(M - m < 16 ? M - m : 16);
-    hipLaunchKernelGGL(w8a16_persist_kernel<true>, dim3(grid), dim3(1024), 0, st, static_cast<const f16*>(A) + m * K, Wp,
+    hipLaunchKernelGGL(w8a16_persist_kernel, dim3(grid), dim3(1024), 0, st, static_cast<const f16*>(A) + m * K, Wp,
                        static_cast<const f16*>(scales), static_cast<f16*>(C) + m * N, rows, (int)N, (int)K, chan_per_wg);
     rc = launch_status();
   }

@@ -196,7 +196,11 @@ int hexmi_add_matmul_softmax(int64_t M, int64_t N, int64_t K, const void *x,
 /* Weight-only int8 GEMM (W8A16): C[m,n] = sum_k A[m,k] * (float(W[n,k]) *
  * float(scales[n])), fp32 accumulation, C fp16.
  * A fp16 [M,K]; W int8 [N,K] row-major (symmetric, zero-point 0); scales fp16
- * [N], one per output channel. The reference has no such kernel; this is the
+ * [N], one per output channel. Results are reproducible bit for bit; the order
+ * of a channel's sum over k may depend on where the channel stands in W (for
+ * 2 <= M <= 128 the workgroup that owns it sets the k it starts at), so moving a
+ * channel can change its outputs in the last place. The reference has no such
+ * kernel; this is the
  * fusion of quant.dcast lowering
  * (qcom_hexagon_backend/lib/Conversion/LinalgToLLVM/LinalgToLLVMPass.cpp:224-230)
  * with the transposed-weight matmul of test_hexkl_macro_matmul.py:24-28. */
@@ -275,9 +279,8 @@ int hexmi_pack_w8(int64_t N, int64_t K, const int8_t *W, int8_t *Wp,
 /* hexmi_gemm_w8a16 on weights packed by hexmi_pack_w8: every weight load of a
  * wave is a contiguous KiB already in MFMA fragment order. K % 1024 == 0 and
  * K <= 4096. Meant for M <= 16 (decode batches); larger M runs 16 rows per
- * launch. For 3 <= M <= 8 hexmi_gemm_w8a16 runs the same kernel and the results
- * agree bit for bit; for other M its kernels sum in another order and the
- * results agree to one fp16 unit in the last place. */
+ * launch. hexmi_gemm_w8a16's kernels sum in another order: the results agree
+ * to one fp16 unit in the last place. */
 int hexmi_gemm_w8a16_packed(int64_t M, int64_t N, int64_t K, const void *A,
                             const int8_t *Wp, const void *scales, void *C,
                             hexmi_stream_t stream);
