@@ -223,10 +223,10 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
   }
 }
 
-// 2 < M <= 128 (MB = 1..8 blocks of 16 activation rows; K % 256 == 0, or any multiple of 64 with MB = 1): persistent
+// 2 < M <= 128 (MB = 1..8 blocks of 16 activation rows; K % 256 == 0, or any multiple of 64 with MB <= 2): persistent
 // workgroups of 16 waves, each owning an equal contiguous range of at most 48 output channels, so the weights cross
 // HBM once, in contiguous row segments. K is walked in chunks of KC = 256 (MB <= 4) or 128 (MB = 8): an activation
-// chunk is at most 32 KiB; with MB = 1 and one or two channel tiles the chunks are 768 and 384 k long (mid_kc()). The raw int8 weight chunk [48][KC] and the activation chunk [MB*16][KC] fp16 are copied
+// chunk is at most 32 KiB; with MB <= 2 and one or two channel tiles the chunks are 768 or 384 k long (mid_kc()). The raw int8 weight chunk [48][KC] and the activation chunk [MB*16][KC] fp16 are copied
 // global -> LDS (global_load_lds, no registers) by different waves: waves 12..15 copy weights, four chunks ahead
 // (five stages: three or four measured the same, seven and nine 5-10 % slower), waves 0..11 copy activations, two
 // chunks ahead (three stages; L2 hits). A wave's outstanding-copy counter only sees its own copies, so each role
@@ -257,7 +257,9 @@ constexpr int kMidMaxM = 128;
 // K per chunk. Sixteen rows leave LDS for longer chunks, and a workgroup with one or two channel tiles needs them:
 // what a CU has in flight is four chunks of weights, 16 KiB with one tile of 256 k, too little to keep HBM busy
 // (N = 4096, K = 11008, M = 16: 19.1 us), 48 KiB with 768 k.
-constexpr int mid_kc(int mb, int nt) { return mb == 1 ? (nt == 1 ? 768 : nt == 2 ? 384 : 256) : mb <= 4 ? 256 : 128; }
+constexpr int mid_kc(int mb, int nt) {
+  return mb == 1 ? (nt == 1 ? 768 : nt == 2 ? 384 : 256) : mb == 2 ? (nt <= 2 ? 384 : 256) : mb <= 4 ? 256 : 128;
+}
 // s_waitcnt immediate (gfx9 encoding) that leaves `vm` vector-memory operations outstanding, LDS counter untouched
 constexpr int wait_vm(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
@@ -280,18 +282,18 @@ template <int CH> __device__ __forceinline__ int mid_w_pos(int c, int row) {
 // are copied. The compute waves of the other tiles run the same code on whatever their part of the stage holds
 // (their sums are never stored): they are needed for the activation copies and the barriers, and a second code
 // path for them costs the kernel registers it does not have.
-// KC: K per chunk. With sixteen rows (MB = 1) K need not be a multiple of it: copies of a last, shorter chunk are
+// KC: K per chunk. With up to 32 rows (MB <= 2) K need not be a multiple of it: copies of a last, shorter chunk are
 // clamped to the row and the 64-k units past K are multiplied as zeros.
 template <int MB, int NT = 3, int KC = mid_kc(MB, NT)>
 __global__ __launch_bounds__(1024, (MB == 1 && NT == 2 && KC == 256) ? 8 : 4)
 void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
                       f16* __restrict__ C, int M, int N, int K, int chan_per_wg, int rotate) {
   constexpr int KU = KC / 64;                               // 64-k units per chunk
-  // channel-tile slots the twelve compute waves are laid out for: the tiles in use when their units take all
-  // twelve, else three (the waves of a slot without channels run along)
-  constexpr int TS = NT * KU == kMidCompute ? NT : 3;
+  // channel-tile slots the twelve compute waves are laid out for: the tiles in use when their units and whole
+  // groups of row blocks take all twelve, else three (the waves of a slot without channels run along)
+  constexpr int TS = kMidCompute % (NT * KU) == 0 && MB % (kMidCompute / (NT * KU)) == 0 ? NT : 3;
   constexpr int RG = kMidCompute / TS / KU;                 // row-block groups
-  constexpr bool TAIL = MB == 1;                            // K % KC != 0 allowed
+  constexpr bool TAIL = MB <= 2;                            // K % KC != 0 allowed
   static_assert(TS * KU * RG == kMidCompute && KC % 64 == 0, "every compute wave has a tile slot, a unit and a group");
   constexpr int RB = MB / RG;                               // row blocks per compute wave
   static_assert(MB % RG == 0 && RB >= 1 && RB <= 4, "row blocks split evenly over the groups");
@@ -870,8 +872,8 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
 #undef HEXMI_GEMV
     return launch_status();
   }
-  // the chunked kernel: K in whole chunks of 256, or any K (a multiple of 64 here) with up to 16 rows
-  if (M <= kMidMaxM && (K % 256 == 0 || M <= 16) && K <= (1 << 29)) {
+  // the chunked kernel: K in whole chunks of 256, or any K (a multiple of 64 here) with up to 32 rows
+  if (M <= kMidMaxM && (K % 256 == 0 || M <= 32) && K <= (1 << 29)) {
     const int cus = hexmi_num_cus();
     if (cus <= 0) return HEXMI_ELAUNCH;
     const int64_t per_cu = (N + cus - 1) / cus;
