@@ -928,11 +928,13 @@ namespace {
 // Shapes the (channel range x K part) kernel takes ahead of the kernels of hexmi_gemm_w8a16, from timings of both over
 // N in 1024 .. 28672 and K in 2048 .. 14336 on 256 CUs. Those kernels give every workgroup all of K and up to 48
 // channels (M <= 128) or a 128 x 128 tile (M > 128): they fall behind when that leaves CUs idle or oversubscribed
-// (N > 48 channels per CU; fewer tiles than a third of the CUs, or than half of them with a long K) and when K is
-// long (every workgroup pulls M x K of activations through L2).
+// (N > 48 channels per CU, twice that up to 32 rows; fewer tiles than a third of the CUs, or than half of them with
+// a long K) and when K is long (every workgroup pulls M x K of activations through L2; up to 64 rows only when K is
+// also longer than N: N = K = 8192 takes 26.4 us against 28.8 at M = 64, 44.6 against 35.4 at M = 128).
 bool prefer_split(int64_t M, int64_t N, int64_t K, int cus) {
   if (M < 32 || M > 256) return false;
-  if (M <= 128) return N > 48 * (int64_t)cus || (K >= 8192 && M >= 64);
+  if (M <= 32) return N > 96 * (int64_t)cus;
+  if (M <= 128) return N > 48 * (int64_t)cus || (K >= 8192 && (M > 64 || K > N));
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
   return tiles * 3 <= cus || (tiles * 2 <= cus && K >= 8192);
 }

@@ -210,9 +210,10 @@ int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void *A,
 
 /* hexmi_gemm_w8a16 with a caller-owned scratch buffer, for the shapes whose
  * kernels of choice split K over several workgroups and add the fp32 partial
- * tiles up afterwards: 32 <= M <= 256 with more than 48 output channels per
- * compute unit, with K >= 8192 (M >= 64), or, for M > 128, with fewer 128 x 128
- * tiles than a third of the compute units (than half of them when K >= 8192)
+ * tiles up afterwards: 32 < M <= 128 with more than 48 output channels per
+ * compute unit (M = 32: more than 96) or with K >= 8192 (up to M = 64 only when
+ * also K > N), and 128 < M <= 256 with fewer 128 x 128 tiles than a third of
+ * the compute units (than half of them when K >= 8192)
  * (the down projection N = 4096, K = 11008 of
  * the model whose up projection is the benchmark shape is one: M = 256 in 40 us
  * where hexmi_gemm_w8a16 takes 75). hexmi_gemm_w8a16_workspace returns the bytes
