@@ -275,6 +275,8 @@ template <int CH> __device__ __forceinline__ int mid_w_pos(int c, int row) {
   else return (c & ~7) | ((c ^ (row >> 1)) & 7);
 }
 
+// a branch on a wave's role (see the note at the copy slots)
+#define HEXMI_EITHER(c) __builtin_expect((c), 1)
 #define HEXMI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define HEXMI_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 
@@ -335,28 +337,34 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   const char* slot_src[SL];                                 // source of this lane for chunk 0
   int slot_dst[SL];                                         // byte offset of the copy inside its stage
   int slot_lim[SL];                                         // largest chunk offset that keeps this lane inside its row
+  // Before the loop, every piece of code that only one role runs is an `if` of its own marked as expected, never an
+  // else branch: the compiler places an else branch it takes for the unlikely one behind the loop, and a jump into
+  // code not yet fetched costs a kernel that has just started about half a microsecond (the weight waves' slots,
+  // their first copies and their first wait were three such jumps; 1-2 % of the kernel at 16 rows). The slots of
+  // the other role stay unset: nothing reads them.
+  if (HEXMI_EITHER(copies_w)) {
 #pragma unroll
-  for (int j = 0; j < SL; ++j) {
-    slot_src[j] = nullptr;
-    slot_dst[j] = 0;
-    slot_lim[j] = 0;
-    if (computes && j < ASL) {
-      const int i = (j * kMidCompute + wave) % NAC;
-      const int f = i * 64 + lane;                          // 16-byte piece of the stage: 64 per copy
-      const int row = f / ACH;
-      const int src_c = mid_a_pos<ACH>(f % ACH, row);       // the chunk that belongs at this position
-      slot_src[j] = reinterpret_cast<const char*>(A + (int64_t)(row < M ? row : M - 1) * K) + src_c * 16;
-      slot_dst[j] = i * 1024;
-      slot_lim[j] = K * 2 - 16 - src_c * 16;
-    } else if (copies_w && j < WSL) {
+    for (int j = 0; j < WSL; ++j) {
       const int t = (j * 4 + (wave - kMidWWave0)) % NWC;
-      const int f = t * 64 + lane;
+      const int f = t * 64 + lane;                          // 16-byte piece of the stage: 64 per copy
       const int row = f / WCH;
-      const int src_c = mid_w_pos<WCH>(f % WCH, row);
+      const int src_c = mid_w_pos<WCH>(f % WCH, row);       // the chunk that belongs at this position
       const int n = n_begin + row < n_end ? n_begin + row : n_end - 1;
       slot_src[j] = reinterpret_cast<const char*>(W + (int64_t)n * K) + src_c * 16;
       slot_dst[j] = t * 1024;
       slot_lim[j] = K - 16 - src_c * 16;
+    }
+  }
+  if (HEXMI_EITHER(computes)) {
+#pragma unroll
+    for (int j = 0; j < ASL; ++j) {
+      const int i = (j * kMidCompute + wave) % NAC;
+      const int f = i * 64 + lane;
+      const int row = f / ACH;
+      const int src_c = mid_a_pos<ACH>(f % ACH, row);
+      slot_src[j] = reinterpret_cast<const char*>(A + (int64_t)(row < M ? row : M - 1) * K) + src_c * 16;
+      slot_dst[j] = i * 1024;
+      slot_lim[j] = K * 2 - 16 - src_c * 16;
     }
   }
   // chunk indices past the end repeat the last chunk (copied, never read): every chunk issues the same copies
@@ -449,26 +457,26 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
       acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, __builtin_bit_cast(f16x8, f.a1[rb]), acc[rb], 0, 0, 0);
   };
   // prologue: activations of chunks 0, 1; weights of chunks 0 .. 3
-  if (computes) {
-    issue_a(0, a_lds);
-    issue_a(1, a_lds + kAStage);
-  } else if (copies_w) {
+  if (HEXMI_EITHER(copies_w)) {
 #pragma unroll
     for (int i = 0; i < WS - 1; ++i) issue_w(i, w_lds + i * kWStage);
+  }
+  if (HEXMI_EITHER(computes)) {
+    issue_a(0, a_lds);
+    issue_a(1, a_lds + kAStage);
   }
   // Round u: chunk u+1 has landed for every wave after the barrier (each role waited for its own copies of it) and
   // every wave has the fragments of chunk u in registers, so the stages of chunk u are free: the copies of chunk
   // u+3 (activations) and u+WS (weights) go there. Then the fragments of chunk u+1 are requested and chunk u is
   // multiplied. Round -1 (before the loop) fetches the fragments of chunk 0.
-  if (computes) __builtin_amdgcn_s_waitcnt(wait_vm(ASL));                  // chunk 0 landed
-  else if (copies_w) __builtin_amdgcn_s_waitcnt(wait_vm((WS - 2) * WSL));
+  if (HEXMI_EITHER(copies_w)) __builtin_amdgcn_s_waitcnt(wait_vm((WS - 2) * WSL));   // chunk 0 landed
+  if (HEXMI_EITHER(computes)) __builtin_amdgcn_s_waitcnt(wait_vm(ASL));
   __builtin_amdgcn_s_barrier();
   Frags fa, fb;
-  if (computes) {
+  if (HEXMI_EITHER(copies_w)) issue_w(WS - 1, w_lds + (WS - 1) * kWStage);
+  if (HEXMI_EITHER(computes)) {
     issue_a(2, a_lds + 2 * kAStage);
     read_frags(fa, a_lds, w_lds);
-  } else if (copies_w) {
-    issue_w(WS - 1, w_lds + (WS - 1) * kWStage);
   }
   // The loop is unrolled by two only (the two register buffers alternate); the LDS stages are counted at run time
   // in scalar registers. A kernel's instruction cache starts cold and a jump to code not yet fetched costs about
@@ -542,6 +550,9 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   }
+  // the scale is first used here: without this the compiler converts it to fp32 where it is loaded and makes wave 0
+  // wait for an HBM access before its first copies
+  asm volatile("" : "+v"(my_scale));
   if (computes) {
     if (threadIdx.x < kMidCh) sc_s[threadIdx.x] = (float)my_scale;
 #pragma unroll
@@ -578,6 +589,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     }
   }
 }
+#undef HEXMI_EITHER
 #undef HEXMI_LDS
 #undef HEXMI_GLB
 
