@@ -918,7 +918,7 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     if (M <= 16) {
       if (paired) HEXMI_MID_KC(1, 2, 256); else HEXMI_MID(1)
     } else if (M <= 32) HEXMI_MID(2) else if (M <= 48) HEXMI_MID(3) else if (M <= 64) HEXMI_MID(4)
-    else HEXMI_MID(8)
+    else if (M <= 96) HEXMI_MID(6) else HEXMI_MID(8)
 #undef HEXMI_MID
 #undef HEXMI_MID_NT
 #undef HEXMI_MID_KC
@@ -941,12 +941,18 @@ namespace {
 // N in 1024 .. 28672 and K in 2048 .. 14336 on 256 CUs. Those kernels give every workgroup all of K and up to 48
 // channels (M <= 128) or a 128 x 128 tile (M > 128): they fall behind when that leaves CUs idle or oversubscribed
 // (N > 48 channels per CU, twice that up to 32 rows; fewer tiles than a third of the CUs, or than half of them with
-// a long K) and when K is long (every workgroup pulls M x K of activations through L2; up to 64 rows only when K is
-// also longer than N: N = K = 8192 takes 26.4 us against 28.8 at M = 64, 44.6 against 35.4 at M = 128).
+// a long K) and when K is long, since every workgroup pulls M x K of activations through L2: up to 96 rows from
+// K = 8192 on and only when K is more than twice N (N = 4096, K = 8192, M = 64: 23.4 us against 26.0; K = 11008:
+// 29.4 against 28.9), above 96 rows from K = 4608 + 64 per channel of a CU's share on (N = 4096: 27.6 against 28.6 us
+// at K = 5120, 31.7 against 29.7 at 6144; N = 11008: 41.4 against 42.5 at K = 7168, 47.6 against 44.6 at 8192).
 bool prefer_split(int64_t M, int64_t N, int64_t K, int cus) {
   if (M < 32 || M > 256) return false;
   if (M <= 32) return N > 96 * (int64_t)cus;
-  if (M <= 128) return N > 48 * (int64_t)cus || (K >= 8192 && (M > 64 || K > N));
+  if (M <= 128) {
+    if (N > 48 * (int64_t)cus) return true;
+    if (M <= 96) return K >= 8192 && K > 2 * N;
+    return K >= 4608 + 64 * ((N + cus - 1) / cus);
+  }
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
   return tiles * 3 <= cus || (tiles * 2 <= cus && K >= 8192);
 }

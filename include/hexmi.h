@@ -211,9 +211,10 @@ int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void *A,
 /* hexmi_gemm_w8a16 with a caller-owned scratch buffer, for the shapes whose
  * kernels of choice split K over several workgroups and add the fp32 partial
  * tiles up afterwards: 32 < M <= 128 with more than 48 output channels per
- * compute unit (M = 32: more than 96) or with K >= 8192 (up to M = 64 only when
- * also K > N), and 128 < M <= 256 with fewer 128 x 128 tiles than a third of
- * the compute units (than half of them when K >= 8192)
+ * compute unit (M = 32: more than 96) or with a long K (up to M = 96: K >= 8192
+ * and K > 2 N; above: K >= 4608 + 64 per output channel of a compute unit's
+ * share), and 128 < M <= 256 with fewer 128 x 128 tiles than a third of the
+ * compute units (than half of them when K >= 8192)
  * (the down projection N = 4096, K = 11008 of
  * the model whose up projection is the benchmark shape is one: M = 256 in 40 us
  * where hexmi_gemm_w8a16 takes 75). hexmi_gemm_w8a16_workspace returns the bytes

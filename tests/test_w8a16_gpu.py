@@ -68,7 +68,7 @@ def test_scale_selection_and_indexing(hexmi, oracle):
     assert c1[1, 37] == w[37, 7] and c1[:, :37].abs().sum() == 0 and c1[:, 38:].abs().sum() == 0
 
 
-@pytest.mark.parametrize("M", [1, 2, 15, 16, 17, 33, 64, 100, 129, 200, 256])
+@pytest.mark.parametrize("M", [1, 2, 15, 16, 17, 33, 64, 65, 96, 100, 129, 200, 256])
 @pytest.mark.parametrize("N,K", [(96, 512), (1000, 256), (16, 64), (11, 4096), (200, 7936)])
 def test_w8a16_parity(hexmi, oracle, M, N, K):
     a, w, s = _inputs(M, N, K, seed=3)
@@ -78,7 +78,7 @@ def test_w8a16_parity(hexmi, oracle, M, N, K):
     assert (got.float() - want.float()).abs().max() / math.sqrt(K) <= 2e-2
 
 
-@pytest.mark.parametrize("M", [3, 8, 9, 16, 32, 48, 64, 100, 128])
+@pytest.mark.parametrize("M", [3, 8, 9, 16, 32, 48, 64, 80, 96, 100, 128])
 @pytest.mark.parametrize("chunks", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 13])
 def test_w8a16_every_tail_of_the_chunked_kernel(hexmi, oracle, M, chunks):
     # the chunked kernel (M <= 128) stops copying ahead and lowers its waits by the number of chunks left: every
