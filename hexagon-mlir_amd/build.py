@@ -27,6 +27,20 @@ FLAGS = [
 ]
 
 
+# amdgpu-kernarg-preload-count: the kernel arguments arrive in scalar registers when a wave starts instead of being
+# loaded by its first instructions. About 0.1 us per launch for the W8A16 kernels (9.19 -> 9.08 us at one row,
+# 11.8 -> 11.7 at sixteen, A/B under graph replay); the row kernels, which start tens of thousands of waves, lose by
+# it (softmax fp32 [4096, 1024] 6.55 -> 6.89 us), so it is set per file.
+EXTRA_FLAGS = {
+    "w8a16.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "w8a16_split.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+}
+
+
+def flags_for(src):
+    return FLAGS + EXTRA_FLAGS.get(src, [])
+
+
 def _sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
@@ -43,7 +57,7 @@ def _compile(src, force, hdr_mtime):
     if (not force and os.path.exists(obj)
             and os.path.getmtime(obj) > max(os.path.getmtime(path), hdr_mtime)):
         return obj, False
-    cmd = [HIPCC] + FLAGS + ["-c", path, "-o", obj]
+    cmd = [HIPCC] + flags_for(src) + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))

@@ -166,7 +166,7 @@ CVT_SOURCES = ("gemm.hip", "calibrate.hip", "w8a16.hip", "w8a16_split.hip")   # 
 
 def _assembly(name, tmp):
     out = os.path.join(tmp, name[:-4] + ".s")
-    cmd = [_build.HIPCC] + _build.FLAGS + ["--cuda-device-only", "-S", os.path.join(_build.CSRC, name), "-o", out]
+    cmd = [_build.HIPCC] + _build.flags_for(name) + ["--cuda-device-only", "-S", os.path.join(_build.CSRC, name), "-o", out]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         sys.exit("hipcc failed:\n" + r.stderr)
