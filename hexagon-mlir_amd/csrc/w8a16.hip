@@ -286,10 +286,13 @@ template <int CH> __device__ __forceinline__ int mid_w_pos(int c, int row) {
 // path for them costs the kernel registers it does not have.
 // KC: K per chunk. With up to 32 rows (MB <= 2) K need not be a multiple of it: copies of a last, shorter chunk are
 // clamped to the row and the 64-k units past K are multiplied as zeros.
-template <int MB, int NT = 3, int KC = mid_kc(MB, NT)>
+// ZP: a zero point is subtracted from the widened weights (exact in fp16), as in w8a16_kernel above; per_tensor
+// reads scale and zero point at index 0 for every channel (with or without ZP).
+template <int MB, int NT = 3, int KC = mid_kc(MB, NT), bool ZP = false>
 __global__ __launch_bounds__(1024, (MB == 1 && NT == 2 && KC == 256) ? 8 : 4)
 void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
-                      f16* __restrict__ C, int M, int N, int K, int chan_per_wg, int rotate) {
+                      f16* __restrict__ C, int M, int N, int K, int chan_per_wg, int rotate,
+                      const int8_t* __restrict__ zero_points = nullptr, int per_tensor = 0) {
   constexpr int KU = KC / 64;                               // 64-k units per chunk
   // channel-tile slots the twelve compute waves are laid out for: the tiles in use when their units and whole
   // groups of row blocks take all twelve, else three (the waves of a slot without channels run along)
@@ -329,7 +332,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   f16 my_scale = (f16)0.0f;
   if (threadIdx.x < kMidCh) {
     const int gn = n_begin + (int)threadIdx.x;
-    my_scale = scales[gn < n_end ? gn : n_end - 1];
+    my_scale = scales[per_tensor ? 0 : (gn < n_end ? gn : n_end - 1)];
   }
 
   // ---- copy slots: every copy moves 1 KiB (1024 / row bytes whole rows); lane positions are permuted inside a row
@@ -410,6 +413,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   f32x4 acc[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  f16 zp_h = (f16)0.0f;                                     // ZP: set in the prologue
   // The fragment reads are written as inline assembly: the compiler cannot tell which stage an in-flight
   // global_load_lds writes and would make every LDS read wait for all of them (vmcnt(0)), which undoes the
   // pipelining. The waits this kernel needs are the explicit ones around the barrier.
@@ -440,13 +444,20 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   };
   auto multiply = [&](const Frags& f, int chunk) __attribute__((always_inline)) {
     f16x8 w0, w1;
+    f16 z = zp_h;
     if constexpr (TAIL) {
       // a unit past the end of K holds the bytes its copies were clamped to: its weights count as zeros
+      // (and so does its zero point)
       const unsigned keep = k_chunk(chunk) * KC + ku * 64 < K ? 0xffffffffu : 0u;
       const u32x4 raw = {f.raw[0] & keep, f.raw[1] & keep, f.raw[2] & keep, f.raw[3] & keep};
       cvt16(raw, w0, w1);
+      if constexpr (ZP) z = __builtin_bit_cast(f16, (unsigned short)(__builtin_bit_cast(unsigned short, zp_h) & keep));
     } else {
       cvt16(f.raw, w0, w1);                                 // converted once, used for every row block
+    }
+    if constexpr (ZP) {
+      w0 -= z;                                              // exact: integers of magnitude <= 255
+      w1 -= z;
     }
     // D[i = channel][j = activation row]: lane holds row j = lane%16, channels 4*(lane/16) + 0..3
 #pragma unroll
@@ -464,6 +475,17 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   if (HEXMI_EITHER(computes)) {
     issue_a(0, a_lds);
     issue_a(1, a_lds + kAStage);
+    if constexpr (ZP) {
+      // The zero point of the channel whose weights this lane converts (lane % 16 of the wave's tile), requested
+      // behind the first activation copies and waited for, with them, before the first barrier: it comes from HBM
+      // like the first weights everybody waits for there, and once it is a plain register value the compiler has no
+      // load to wait for inside the loop, where its wait would cover every copy in flight in every round. (Weight
+      // waves must not take part: the same wait would cover all their copies.)
+      const int gn = n_begin + (nt < NT ? nt : 0) * 16 + r16;
+      int my_zp = zero_points[per_tensor ? 0 : (gn < n_end ? gn : n_end - 1)];
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(my_zp) :: "memory");
+      zp_h = (f16)(float)my_zp;
+    }
   }
   // Round u: chunk u+1 has landed for every wave after the barrier (each role waited for its own copies of it) and
   // every wave has the fragments of chunk u in registers, so the stages of chunk u are free: the copies of chunk
@@ -599,17 +621,24 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
 // row) sit in registers as fp16 pairs. Products are v_dot2_f32_f16 (two exact fp16 products added into an fp32
 // accumulator), the 64 lane partials are summed with a butterfly, and lane 0 applies the channel scale.
 // NW waves per workgroup share the activation rows through LDS.
-template <int MR, int RPW, int KJ, int NW = 4>              // KJ = K / 1024: 16-byte loads per lane per row
+// ZP / per_tensor: as in the kernels above (the zero point is subtracted from the widened weights).
+template <int MR, int RPW, int KJ, int NW = 4, bool ZP = false>   // KJ = K / 1024: 16-byte loads per lane per row
 __global__ __launch_bounds__(NW * 64)
 void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
-                       f16* __restrict__ C, int M, int N, int K) {
+                       f16* __restrict__ C, int M, int N, int K, const int8_t* __restrict__ zero_points = nullptr,
+                       int per_tensor = 0) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n0 = (blockIdx.x * NW + wave) * RPW;           // may lie past N in the last workgroup: loads clamp, stores check
 
   // the channel scales first: they come from HBM and would otherwise be waited for after everything else
-  f16 sc[RPW];
+  f16 sc[RPW], zp[RPW];
 #pragma unroll
-  for (int r = 0; r < RPW; ++r) sc[r] = scales[n0 + r < N ? n0 + r : N - 1];
+  for (int r = 0; r < RPW; ++r) {
+    const int at = per_tensor ? 0 : (n0 + r < N ? n0 + r : N - 1);
+    sc[r] = scales[at];
+    zp[r] = (f16)0.0f;
+    if constexpr (ZP) zp[r] = (f16)(float)zero_points[at];
+  }
   // activations: lane needs k in [1024*j + 16*lane, +16) for every j. The four waves of the workgroup need the same
   // rows, so each fetches a quarter of them (requested before the weights: their wait then leaves the weight loads in
   // flight) and all read their fragments back from LDS.
@@ -658,6 +687,10 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
     for (int j = 0; j < KJ; ++j) {
       f16x8 w0, w1;
       cvt16(wv[r][j], w0, w1);
+      if constexpr (ZP) {
+        w0 -= zp[r];
+        w1 -= zp[r];
+      }
 #pragma unroll
       for (int m = 0; m < MR; ++m) {
 #pragma unroll
@@ -683,13 +716,16 @@ void w8a16_gemv_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, 
 // activation rows are staged in LDS once per workgroup and read back piece by piece, so the
 // registers hold the row's weight loads (all in flight at once) and little else. Sixteen waves per workgroup (N = 4096,
 // K = 11008: 11.5 us against 11.9 with eight and 12.0 with four: fewer workgroups stage the activation row).
-template <int MR, int NJ, int NW = 16>
+template <int MR, int NJ, int NW = 16, bool ZP = false>
 __global__ __launch_bounds__(NW * 64)
 void w8a16_gemv_any_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
-                           f16* __restrict__ C, int M, int N, int K) {
+                           f16* __restrict__ C, int M, int N, int K, const int8_t* __restrict__ zero_points = nullptr,
+                           int per_tensor = 0) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = blockIdx.x * NW + wave;                     // may lie past N in the last workgroup: loads clamp
-  const f16 sc = scales[n < N ? n : N - 1];
+  const f16 sc = scales[per_tensor ? 0 : (n < N ? n : N - 1)];
+  f16 zp = (f16)0.0f;
+  if constexpr (ZP) zp = (f16)(float)zero_points[per_tensor ? 0 : (n < N ? n : N - 1)];
   const int pieces = K / 16;                                // 16-byte pieces of a weight row
   u32x4 wv[NJ];
   {
@@ -717,6 +753,11 @@ void w8a16_gemv_any_kernel(const f16* __restrict__ A, const int8_t* __restrict__
     if (j * 64 < pieces) {                                  // wave-uniform: rounds past the row do nothing
       f16x8 w0, w1;
       cvt16(wv[j], w0, w1);
+      if constexpr (ZP) {
+        const f16 z = pc < pieces ? zp : (f16)0.0f;         // a masked lane's weights stay zero
+        w0 -= z;
+        w1 -= z;
+      }
       const int at = (pc < pieces ? pc : 0) * 16;           // masked lanes hold zero weights; any valid address
 #pragma unroll
       for (int m = 0; m < MR; ++m) {
@@ -829,8 +870,12 @@ int launch_pass_zp(const f16* A, const int8_t* W, const f16* s, f16* C, int M, i
 
 using namespace hexmi;
 
-extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
-                                void* C, hexmi_stream_t stream) {
+namespace {
+// hexmi_gemm_w8a16 (zp == nullptr, pt == 0) and hexmi_gemm_w8a16_ex: one choice of kernels for both. The decode
+// kernels and the chunked kernel have a zero-point instantiation; the 128 x 128 tile kernel does not, so more than
+// 128 rows with a zero point or a per-tensor scale run in passes of 64 rows, one workgroup per 16-channel tile.
+int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
+                   const int8_t* zp, int pt, void* C, hexmi_stream_t stream) {
   if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
   if (M == 0 || N == 0) return HEXMI_OK;
   if (!C || (K > 0 && (!A || !W || !scales))) return HEXMI_EINVAL;
@@ -849,7 +894,8 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     // any other row length: the masked form of the same kernel, instantiated per KiB of row
     const unsigned blocks = (unsigned)((N + 15) / 16);
     const int nj = (int)((K + 1023) / 1024);
-#define HEXMI_GEMV_ANY(MR, NJ) hipLaunchKernelGGL((w8a16_gemv_any_kernel<MR, NJ>), dim3(blocks), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K)
+#define HEXMI_GEMV_ANY(MR, NJ) { if (zp) hipLaunchKernelGGL((w8a16_gemv_any_kernel<MR, NJ, 16, true>), dim3(blocks), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, zp, pt); \
+    else hipLaunchKernelGGL((w8a16_gemv_any_kernel<MR, NJ, 16, false>), dim3(blocks), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, zp, pt); }
 #define HEXMI_GEMV_ANY_NJ(MR) switch (nj) { \
     case 1: HEXMI_GEMV_ANY(MR, 1); break; case 2: HEXMI_GEMV_ANY(MR, 2); break; case 3: HEXMI_GEMV_ANY(MR, 3); break; \
     case 4: HEXMI_GEMV_ANY(MR, 4); break; case 5: HEXMI_GEMV_ANY(MR, 5); break; case 6: HEXMI_GEMV_ANY(MR, 6); break; \
@@ -868,7 +914,7 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     const int64_t gy = (M + MR - 1) / MR;
     if (gy > 65535) return HEXMI_ENOTSUP;
     hipLaunchKernelGGL(w8a16_generic_kernel<MR>, dim3((unsigned)((N + 3) / 4), (unsigned)gy), dim3(256), 0, st, a, W, s,
-                       c, (int)M, (int)N, (int)K);
+                       c, (int)M, (int)N, (int)K, zp, pt);
     return launch_status();
   }
   if (M <= 2 && !chunked_pair && (K == 1024 || K == 2048 || K == 4096 || K == 8192)) {
@@ -877,8 +923,9 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     // channels x four waves on the same box)
     constexpr int RPW = 1, NW = 8;
     const unsigned blocks = (unsigned)((N + NW * RPW - 1) / (NW * RPW));
-#define HEXMI_GEMV(MR, KJ) hipLaunchKernelGGL((w8a16_gemv_kernel<MR, RPW, KJ, NW>), dim3(blocks), dim3(NW * 64), 0, st, a, W, s, c, (int)M, (int)N, (int)K)
-#define HEXMI_GEMV_K(MR) { if (K == 1024) HEXMI_GEMV(MR, 1); else if (K == 2048) HEXMI_GEMV(MR, 2); else if (K == 4096) HEXMI_GEMV(MR, 4); else HEXMI_GEMV(MR, 8); }
+#define HEXMI_GEMV(MR, KJ) { if (zp) hipLaunchKernelGGL((w8a16_gemv_kernel<MR, RPW, KJ, NW, true>), dim3(blocks), dim3(NW * 64), 0, st, a, W, s, c, (int)M, (int)N, (int)K, zp, pt); \
+    else hipLaunchKernelGGL((w8a16_gemv_kernel<MR, RPW, KJ, NW, false>), dim3(blocks), dim3(NW * 64), 0, st, a, W, s, c, (int)M, (int)N, (int)K, zp, pt); }
+#define HEXMI_GEMV_K(MR) { if (K == 1024) HEXMI_GEMV(MR, 1) else if (K == 2048) HEXMI_GEMV(MR, 2) else if (K == 4096) HEXMI_GEMV(MR, 4) else HEXMI_GEMV(MR, 8) }
     if (M == 1) HEXMI_GEMV_K(1) else HEXMI_GEMV_K(2)
 #undef HEXMI_GEMV_K
 #undef HEXMI_GEMV
@@ -911,12 +958,13 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
     const int grid = (int)grid64;
     const int tiles = (chan_per_wg + 15) / 16;              // channel tiles of a workgroup that hold channels
 #define HEXMI_MID_KC(MB, NT, KC) \
-  hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT, KC>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg, paired ? 0 : 1)
+  { if (zp) hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT, KC, true>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg, paired ? 0 : 1, zp, pt); \
+    else hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT, KC, false>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg, paired ? 0 : 1, zp, pt); }
 #define HEXMI_MID_NT(MB, NT) HEXMI_MID_KC(MB, NT, mid_kc(MB, NT))
 #define HEXMI_MID(MB) \
-  { if (tiles == 1) HEXMI_MID_NT(MB, 1); else if (tiles == 2) HEXMI_MID_NT(MB, 2); else HEXMI_MID_NT(MB, 3); }
+  { if (tiles == 1) HEXMI_MID_NT(MB, 1) else if (tiles == 2) HEXMI_MID_NT(MB, 2) else HEXMI_MID_NT(MB, 3) }
     if (M <= 16) {
-      if (paired) HEXMI_MID_KC(1, 2, 256); else HEXMI_MID(1)
+      if (paired) HEXMI_MID_KC(1, 2, 256) else HEXMI_MID(1)
     } else if (M <= 32) HEXMI_MID(2) else if (M <= 48) HEXMI_MID(3) else if (M <= 64) HEXMI_MID(4)
     else if (M <= 96) HEXMI_MID(6) else HEXMI_MID(8)
 #undef HEXMI_MID
@@ -924,16 +972,26 @@ extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, 
 #undef HEXMI_MID_KC
     return launch_status();
   }
-  if (M > 64 && K % 32 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8))
+  if (!zp && !pt && M > 64 && K % 32 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8))
     return gemm_w8a16_tiled(M, N, K, a, W, s, c, st);
   int rc = HEXMI_OK;
   for (int64_t m = 0; m < M && rc == HEXMI_OK; m += 64) {
     const int64_t left = M - m;
-    if (left > 32) rc = launch_pass<4>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
+    if (zp || pt) {
+      if (left > 32) rc = launch_pass_zp<4>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zp, pt, st);
+      else if (left > 16) rc = launch_pass_zp<2>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zp, pt, st);
+      else rc = launch_pass_zp<1>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zp, pt, st);
+    } else if (left > 32) rc = launch_pass<4>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
     else if (left > 16) rc = launch_pass<2>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
     else rc = launch_pass<1>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, st);
   }
   return rc;
+}
+}  // namespace
+
+extern "C" int hexmi_gemm_w8a16(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
+                                void* C, hexmi_stream_t stream) {
+  return gemm_w8a16_any(M, N, K, A, W, scales, nullptr, 0, C, stream);
 }
 
 namespace {
@@ -1063,32 +1121,5 @@ extern "C" int hexmi_dequant_w8_ex(int64_t N, int64_t K, const int8_t* W, const 
 
 extern "C" int hexmi_gemm_w8a16_ex(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
                                    const int8_t* zero_points, int per_tensor, void* C, hexmi_stream_t stream) {
-  if (!zero_points && !per_tensor) return hexmi_gemm_w8a16(M, N, K, A, W, scales, C, stream);   // the symmetric per-channel form
-  if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
-  if (M == 0 || N == 0) return HEXMI_OK;
-  if (!C || (K > 0 && (!A || !W || !scales))) return HEXMI_EINVAL;
-  if (M > 0x7fffffff || N > 0x7fffffff - 16 || K > 0x7fffffff) return HEXMI_ENOTSUP;
-  hipStream_t st = as_stream(stream);
-  const f16* a = static_cast<const f16*>(A);
-  const f16* s = static_cast<const f16*>(scales);
-  f16* c = static_cast<f16*>(C);
-  const int pt = per_tensor ? 1 : 0;
-  begin_call();
-  if (K == 0) return fill_zero_2d(C, M, N, N, 2, st);
-  if (K % 64 != 0 || !aligned_to(A, 16) || !aligned_to(W, 16)) {
-    constexpr int MR = 4;
-    const int64_t gy = (M + MR - 1) / MR;
-    if (gy > 65535) return HEXMI_ENOTSUP;
-    hipLaunchKernelGGL(w8a16_generic_kernel<MR>, dim3((unsigned)((N + 3) / 4), (unsigned)gy), dim3(256), 0, st, a, W, s,
-                       c, (int)M, (int)N, (int)K, zero_points, pt);
-    return launch_status();
-  }
-  int rc = HEXMI_OK;
-  for (int64_t m = 0; m < M && rc == HEXMI_OK; m += 64) {
-    const int64_t left = M - m;
-    if (left > 32) rc = launch_pass_zp<4>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zero_points, pt, st);
-    else if (left > 16) rc = launch_pass_zp<2>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zero_points, pt, st);
-    else rc = launch_pass_zp<1>(a, W, s, c, (int)M, (int)N, (int)K, (int)m, zero_points, pt, st);
-  }
-  return rc;
+  return gemm_w8a16_any(M, N, K, A, W, scales, zero_points, per_tensor ? 1 : 0, C, stream);
 }

@@ -374,7 +374,14 @@ def test_dequant_with_zero_point_bit_exact(hexmi, oracle, per_tensor):
 
 @pytest.mark.parametrize("per_tensor", [False, True])
 @pytest.mark.parametrize("M,N,K", [(1, 96, 512), (16, 1000, 256), (70, 130, 128), (33, 40, 4096), (5, 33, 100),
-                                   (3, 64, 72)])
+                                   (3, 64, 72),
+                                   # the decode kernels and every form of the chunked kernel (chunks of 768, 384, 256
+                                   # and 128 k, short last chunks, two workgroups per CU), which subtract the zero
+                                   # point in registers
+                                   (1, 500, 4096), (2, 300, 2048), (1, 200, 11008), (2, 4100, 8192), (4, 100, 832),
+                                   (16, 5000, 1536), (9, 10000, 4096), (32, 5000, 832), (48, 100, 768),
+                                   (64, 10000, 1024), (96, 100, 512), (128, 5000, 256), (16, 14336, 512),
+                                   (200, 136, 256)])
 def test_w8a16_with_zero_point_parity(hexmi, oracle, per_tensor, M, N, K):
     g = _gen(19)
     a = torch.randn(M, K, generator=g).half()
