@@ -223,7 +223,7 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
   }
 }
 
-// 2 < M <= 128 (MB = 1..8 blocks of 16 activation rows; K % 256 == 0, or any multiple of 64 with MB <= 2): persistent
+// 2 < M <= 128 (MB = 1..8 blocks of 16 activation rows; K any multiple of 64): persistent
 // workgroups of 16 waves, each owning an equal contiguous range of at most 48 output channels, so the weights cross
 // HBM once, in contiguous row segments. K is walked in chunks of KC = 256 (MB <= 4) or 128 (MB = 8): an activation
 // chunk is at most 32 KiB; with MB <= 2 and one or two channel tiles the chunks are 768 or 384 k long (mid_kc()). The raw int8 weight chunk [48][KC] and the activation chunk [MB*16][KC] fp16 are copied
@@ -284,11 +284,13 @@ template <int CH> __device__ __forceinline__ int mid_w_pos(int c, int row) {
 // are copied. The compute waves of the other tiles run the same code on whatever their part of the stage holds
 // (their sums are never stored): they are needed for the activation copies and the barriers, and a second code
 // path for them costs the kernel registers it does not have.
-// KC: K per chunk. With up to 32 rows (MB <= 2) K need not be a multiple of it: copies of a last, shorter chunk are
+// KC: K per chunk. K need not be a multiple of it: copies of a last, shorter chunk are
 // clamped to the row and the 64-k units past K are multiplied as zeros.
 // ZP: a zero point is subtracted from the widened weights (exact in fp16), as in w8a16_kernel above; per_tensor
 // reads scale and zero point at index 0 for every channel (with or without ZP).
-template <int MB, int NT = 3, int KC = mid_kc(MB, NT), bool ZP = false>
+// TAIL: K % KC != 0 allowed. Without it the copies take a uniform chunk offset and the weights go unmasked, which
+// the forms with more than 32 rows, short of registers and issue slots, run 5 % faster (M = 64: 17.0 against 18.0 us).
+template <int MB, int NT = 3, int KC = mid_kc(MB, NT), bool ZP = false, bool TAIL = true>
 __global__ __launch_bounds__(1024, (MB == 1 && NT == 2 && KC == 256) ? 8 : 4)
 void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, const f16* __restrict__ scales,
                       f16* __restrict__ C, int M, int N, int K, int chan_per_wg, int rotate,
@@ -298,7 +300,6 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   // groups of row blocks take all twelve, else three (the waves of a slot without channels run along)
   constexpr int TS = kMidCompute % (NT * KU) == 0 && MB % (kMidCompute / (NT * KU)) == 0 ? NT : 3;
   constexpr int RG = kMidCompute / TS / KU;                 // row-block groups
-  constexpr bool TAIL = MB <= 2;                            // K % KC != 0 allowed
   static_assert(TS * KU * RG == kMidCompute && KC % 64 == 0, "every compute wave has a tile slot, a unit and a group");
   constexpr int RB = MB / RG;                               // row blocks per compute wave
   static_assert(MB % RG == 0 && RB >= 1 && RB <= 4, "row blocks split evenly over the groups");
@@ -314,7 +315,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   const int r16 = lane % 16, kg = lane / 16;
   const int n_begin = blockIdx.x * chan_per_wg;
   const int n_end = n_begin + chan_per_wg < N ? n_begin + chan_per_wg : N;
-  const int n_chunks = TAIL ? (K + KC - 1) / KC : K / KC;
+  const int n_chunks = (K + KC - 1) / KC;                   // TAIL: the last one may be short (K % 64 == 0)
   // Workgroup b walks K from chunk b % n_chunks on and wraps round. With every workgroup at the same k at the
   // same time, all the addresses in flight on the chip agree in their low bits when the weight rows are a power of
   // two long, and the memory channels those bits select take the whole load (N = 8192, M = 16: 20.9 us at
@@ -376,7 +377,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   const unsigned a_lds = (unsigned)(size_t)(lds_ptr)(&a_s[0][0]);
   const unsigned w_lds = (unsigned)(size_t)(lds_ptr)(&w_s[0][0]);
   constexpr unsigned kAStage = MB * 16 * KC * 2, kWStage = NT * 16 * KC;
-  // With TAIL a lane whose piece of the last chunk lies past K fetches the last 16 bytes of its row instead (never
+  // A lane whose piece of the last chunk lies past K fetches the last 16 bytes of its row instead (never
   // multiplied: see the mask in multiply()).
   auto issue_a = [&](int chunk, unsigned dst) __attribute__((always_inline)) {
     const int ck = k_chunk(chunk < n_chunks ? chunk : n_chunks - 1);
@@ -444,18 +445,17 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   };
   auto multiply = [&](const Frags& f, int chunk) __attribute__((always_inline)) {
     f16x8 w0, w1;
-    f16 z = zp_h;
+    // a unit past the end of K holds the bytes its copies were clamped to: its weights count as zeros (and so does
+    // its zero point)
+    const unsigned keep = !TAIL || k_chunk(chunk) * KC + ku * 64 < K ? 0xffffffffu : 0u;
     if constexpr (TAIL) {
-      // a unit past the end of K holds the bytes its copies were clamped to: its weights count as zeros
-      // (and so does its zero point)
-      const unsigned keep = k_chunk(chunk) * KC + ku * 64 < K ? 0xffffffffu : 0u;
       const u32x4 raw = {f.raw[0] & keep, f.raw[1] & keep, f.raw[2] & keep, f.raw[3] & keep};
-      cvt16(raw, w0, w1);
-      if constexpr (ZP) z = __builtin_bit_cast(f16, (unsigned short)(__builtin_bit_cast(unsigned short, zp_h) & keep));
+      cvt16(raw, w0, w1);                                   // converted once, used for every row block
     } else {
-      cvt16(f.raw, w0, w1);                                 // converted once, used for every row block
+      cvt16(f.raw, w0, w1);
     }
     if constexpr (ZP) {
+      const f16 z = __builtin_bit_cast(f16, (unsigned short)(__builtin_bit_cast(unsigned short, zp_h) & keep));
       w0 -= z;                                              // exact: integers of magnitude <= 255
       w1 -= z;
     }
@@ -931,8 +931,8 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
 #undef HEXMI_GEMV
     return launch_status();
   }
-  // the chunked kernel: K in whole chunks of 256, or any K (a multiple of 64 here) with up to 32 rows
-  if (M <= kMidMaxM && (K % 256 == 0 || M <= 32) && K <= (1 << 29)) {
+  // the chunked kernel: any K (a multiple of 64 here)
+  if (M <= kMidMaxM && K <= (1 << 29)) {
     const int cus = hexmi_num_cus();
     if (cus <= 0) return HEXMI_ELAUNCH;
     const int64_t per_cu = (N + cus - 1) / cus;
@@ -957,9 +957,12 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
     if (grid64 > 0x7fffffff) return HEXMI_ENOTSUP;
     const int grid = (int)grid64;
     const int tiles = (chan_per_wg + 15) / 16;              // channel tiles of a workgroup that hold channels
+#define HEXMI_MID_T(MB, NT, KC, ZP, TAIL) \
+  hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT, KC, ZP, TAIL>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg, paired ? 0 : 1, zp, pt)
+  // up to 32 rows the form that takes any K is the only one (its masks and clamps cost nothing there)
 #define HEXMI_MID_KC(MB, NT, KC) \
-  { if (zp) hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT, KC, true>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg, paired ? 0 : 1, zp, pt); \
-    else hipLaunchKernelGGL((w8a16_mid_kernel<MB, NT, KC, false>), dim3(grid), dim3(1024), 0, st, a, W, s, c, (int)M, (int)N, (int)K, chan_per_wg, paired ? 0 : 1, zp, pt); }
+  { if (MB <= 2 || K % KC != 0) { if (zp) HEXMI_MID_T(MB, NT, KC, true, true); else HEXMI_MID_T(MB, NT, KC, false, true); } \
+    else { if (zp) HEXMI_MID_T(MB, NT, KC, true, (MB <= 2)); else HEXMI_MID_T(MB, NT, KC, false, (MB <= 2)); } }
 #define HEXMI_MID_NT(MB, NT) HEXMI_MID_KC(MB, NT, mid_kc(MB, NT))
 #define HEXMI_MID(MB) \
   { if (tiles == 1) HEXMI_MID_NT(MB, 1) else if (tiles == 2) HEXMI_MID_NT(MB, 2) else HEXMI_MID_NT(MB, 3) }
@@ -970,6 +973,7 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
 #undef HEXMI_MID
 #undef HEXMI_MID_NT
 #undef HEXMI_MID_KC
+#undef HEXMI_MID_T
     return launch_status();
   }
   if (!zp && !pt && M > 64 && K % 32 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8))

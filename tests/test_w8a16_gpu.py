@@ -90,12 +90,12 @@ def test_w8a16_every_tail_of_the_chunked_kernel(hexmi, oracle, M, chunks):
     assert close16(got, want, max_ulp=1, atol=2e-4)
 
 
-@pytest.mark.parametrize("M", [3, 9, 16, 17, 32])
+@pytest.mark.parametrize("M", [3, 9, 16, 17, 32, 48, 64, 96, 128])
 @pytest.mark.parametrize("N", [100, 5000, 10000])
 @pytest.mark.parametrize("K", [64, 192, 320, 448, 704, 768, 832, 1536, 1600, 2368, 4096])
-def test_w8a16_up_to_32_rows_take_any_k(hexmi, oracle, M, N, K):
-    # up to 32 rows: chunks of 768, 384 or 256 k for one, two or three channel tiles per workgroup (N = 100, 5000,
-    # 10000 on 256 CUs), K any multiple of 64: a last chunk that is short, a single short chunk, whole chunks
+def test_w8a16_chunked_kernel_takes_any_k(hexmi, oracle, M, N, K):
+    # chunks of 768, 384, 256 or 128 k by the rows and the channel tiles per workgroup (one, two, three at N = 100,
+    # 5000, 10000 on 256 CUs), K any multiple of 64: a last chunk that is short, a single short chunk, whole chunks
     a, w, s = _inputs(M, N, K, seed=K + M)
     got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
     want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w.numpy(), s.numpy()))
