@@ -873,7 +873,7 @@ using namespace hexmi;
 namespace {
 // hexmi_gemm_w8a16 (zp == nullptr, pt == 0) and hexmi_gemm_w8a16_ex: one choice of kernels for both. The decode
 // kernels and the chunked kernel have a zero-point instantiation; the 128 x 128 tile kernel does not, so more than
-// 128 rows with a zero point or a per-tensor scale run in passes of 64 rows, one workgroup per 16-channel tile.
+// 128 rows with a zero point or a per-tensor scale run the chunked kernel in passes of 128 rows.
 int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t* W, const void* scales,
                    const int8_t* zp, int pt, void* C, hexmi_stream_t stream) {
   if (M < 0 || N < 0 || K < 0) return HEXMI_EINVAL;
@@ -930,6 +930,16 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
 #undef HEXMI_GEMV_K
 #undef HEXMI_GEMV
     return launch_status();
+  }
+  // more than 128 rows with a zero point or a per-tensor scale: the chunked kernel in passes of 128 rows (the tile
+  // kernel has no such form; M = 256, N = 11008, K = 4096: 2 x 28 us against four passes of 20 through w8a16_kernel)
+  if ((zp || pt) && M > kMidMaxM && K <= (1 << 29)) {
+    int rc = HEXMI_OK;
+    for (int64_t m = 0; m < M && rc == HEXMI_OK; m += kMidMaxM) {
+      const int64_t rows = M - m < kMidMaxM ? M - m : kMidMaxM;
+      rc = gemm_w8a16_any(rows, N, K, a + m * K, W, scales, zp, pt, c + m * N, stream);
+    }
+    return rc;
   }
   // the chunked kernel: any K (a multiple of 64 here)
   if (M <= kMidMaxM && K <= (1 << 29)) {

@@ -259,7 +259,7 @@ int hexmi_dequant_w8(int64_t N, int64_t K, const int8_t *W, const void *scales,
  * from the widened weights (exact in fp16) inside the kernel, the scale
  * multiplies the finished fp32 sum. Up to 128 rows it runs the kernels of
  * hexmi_gemm_w8a16 (5-15 % slower with zero points, equal with a per-tensor
- * scale alone); more rows run in passes of 64. With zero_points NULL and
+ * scale alone); more rows run in passes of 128. With zero_points NULL and
  * per_tensor 0 both are the symmetric per-channel entry points above. */
 int hexmi_dequant_w8_ex(int64_t N, int64_t K, const int8_t *W,
                         const void *scales, const int8_t *zero_points,

@@ -381,7 +381,7 @@ def test_dequant_with_zero_point_bit_exact(hexmi, oracle, per_tensor):
                                    (1, 500, 4096), (2, 300, 2048), (1, 200, 11008), (2, 4100, 8192), (4, 100, 832),
                                    (16, 5000, 1536), (9, 10000, 4096), (32, 5000, 832), (48, 100, 768),
                                    (64, 10000, 1024), (96, 100, 512), (128, 5000, 256), (16, 14336, 512),
-                                   (200, 136, 256)])
+                                   (200, 136, 256), (300, 1000, 832)])
 def test_w8a16_with_zero_point_parity(hexmi, oracle, per_tensor, M, N, K):
     g = _gen(19)
     a = torch.randn(M, K, generator=g).half()
