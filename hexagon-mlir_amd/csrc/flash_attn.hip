@@ -14,6 +14,12 @@
 //
 // fp32 inputs with head size 64 or 128 run the fp32 matrix-core kernels of flash_attn_f32.hip; other head sizes and
 // unaligned operands take the plain one-wave-per-query-row kernel below.
+#include <algorithm>
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
 #include "flash_attn_tiles.h"
 
 namespace hexmi {
@@ -65,7 +71,7 @@ template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, i
 __global__ __launch_bounds__(NW * 64, NW == 4 ? (D == 64 && !GENERAL ? 3 : 2) : 1)
 void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                       OutT* __restrict__ O, int ZH, int S, float scale_log2e, const T* __restrict__ Mk = nullptr,
-                      int Skv_arg = 0, float mask_factor = 0.0f) {
+                      int Skv_arg = 0, float mask_factor = 0.0f, int group_heads = 0) {
   static_assert(!(CAUSAL && GENERAL), "the causal kernel has as many keys as queries and no mask");
   static_assert(!MASK_LDS || (GENERAL && NW == 8), "staged mask tiles: general kernel, 8 waves");
   const int Skv = GENERAL ? Skv_arg : S;
@@ -88,16 +94,33 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): every XCD gets a list of whole heads, longest
   // query blocks first, and its workgroups take the list in snake order (unit it*P + u, then it*P + P-1-u, ...),
   // so a workgroup's long and short units alternate and the head in progress stays in the XCD's L2.
+  // group_heads = G > 0 (causal, chosen by the host, see plan_causal_groups): the snake pairs a workgroup's long
+  // unit of one pass with a short one of the next only when a pass is whole heads, or a head whole passes: 16 query
+  // blocks on 32 workgroups per XCD are, 15 or 62 are not, and the causal kernel then ran 20-40 % below its rate at
+  // the next power of two (S = 15872: 763 TFLOP/s against 1139 at 16384). With G the XCD's heads are taken G at a
+  // time; a group's units are listed longest first across its heads (slot j: head j % G, query block
+  // nqb - 1 - j / G) and padded with empty slots at the short end to whole passes. G = 2 at 16 blocks is the list
+  // described above; 15 blocks run as 32 slots of which two are empty, 62 blocks as 64 of which two are.
   const int total = ZH * nqb;
   const bool by_xcd = ZH % 8 == 0 && gridDim.x % 8 == 0;
   const int P = by_xcd ? gridDim.x / 8 : gridDim.x;             // workgroups sharing one list
   const int u = by_xcd ? blockIdx.x / 8 : blockIdx.x;
-  const int list_len = by_xcd ? total / 8 : total;
+  const int G = by_xcd ? group_heads : 0;
+  const int heads = ZH / 8;                                     // of an XCD's list
+  const int gs = G > 0 ? (G * nqb + P - 1) / P * P : 0;         // slots of a full group
+  const int full = G > 0 ? heads / G : 0, rem = G > 0 ? heads % G : 0;
+  const int list_len = G > 0 ? full * gs + (rem * nqb + P - 1) / P * P : (by_xcd ? total / 8 : total);
   for (int it = 0; it * P < list_len; ++it) {
     const int unit = it * P + ((it & 1) ? P - 1 - u : u);
-    if (unit >= list_len) continue;                             // workgroup-uniform
+    if (unit >= list_len) continue;                             // workgroup-uniform, like the one below
     int zh, qb;
-    if (by_xcd) {
+    if (G > 0) {
+      const int grp = unit < full * gs ? unit / gs : full;
+      const int j = unit - grp * gs, gh = grp < full ? G : rem;
+      qb = nqb - 1 - j / gh;
+      if (qb < 0) continue;                                     // padding
+      zh = blockIdx.x % 8 + 8 * (grp * G + j % gh);
+    } else if (by_xcd) {
       zh = blockIdx.x % 8 + 8 * (unit / nqb);
       qb = nqb - 1 - unit % nqb;
     } else {
@@ -447,6 +470,59 @@ inline int64_t resident_grid(int64_t units, int per_cu) {
   return units < resident || resident == 0 ? units : resident;
 }
 
+// Heads per group for the causal kernel's unit lists (0: the plain list of whole heads): the candidate whose
+// busiest workgroup has the least to do, counted in key blocks plus two per unit, with the lists walked exactly as
+// the kernel walks them; of equal candidates the largest group. Up to eight heads: more heads in flight per XCD
+// than their keys and values fit its L2 cost nothing measurable ([4, 32, S, 128]: S = 3840 514 / 506 / 491 us with
+// 2 / 4 / 8 heads, all equal in this count; S = 4096 567 / 574 / 552; S = 4352 842 / 644 / 632), balance decides.
+inline int plan_causal_groups(int64_t ZH, int64_t nqb, int64_t grid) {
+  if (ZH % 8 != 0 || grid % 8 != 0 || nqb > (1 << 20)) return 0;
+  const int64_t P = grid / 8, heads = ZH / 8;
+  if (heads * nqb <= P) return 0;                               // one unit per workgroup at most
+  const int64_t gmax = heads < 8 ? heads : 8;
+  // the answer depends on four integers: remembered, so that a launch does not pay for the walk
+  static std::mutex mu;
+  static std::map<std::tuple<int64_t, int64_t, int64_t, int64_t>, int> known;
+  const auto key = std::make_tuple(ZH, nqb, grid, gmax);
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    const auto it = known.find(key);
+    if (it != known.end()) return it->second;
+  }
+  std::vector<int64_t> load((size_t)P);
+  int best = 0;
+  int64_t best_span = -1;
+  for (int G = 0; G <= (int)gmax; ++G) {
+    std::fill(load.begin(), load.end(), 0);
+    const int64_t gs = G > 0 ? (G * nqb + P - 1) / P * P : 0;
+    const int64_t full = G > 0 ? heads / G : 0, rem = G > 0 ? heads % G : 0;
+    const int64_t list_len = G > 0 ? full * gs + (rem * nqb + P - 1) / P * P : heads * nqb;
+    for (int64_t it = 0; it * P < list_len; ++it)
+      for (int64_t u = 0; u < P; ++u) {
+        const int64_t unit = it * P + ((it & 1) ? P - 1 - u : u);
+        if (unit >= list_len) continue;
+        int64_t qb;
+        if (G > 0) {
+          const int64_t grp = unit < full * gs ? unit / gs : full;
+          const int64_t j = unit - grp * gs, gh = grp < full ? G : rem;
+          qb = nqb - 1 - j / gh;
+          if (qb < 0) continue;
+        } else {
+          qb = nqb - 1 - unit % nqb;
+        }
+        load[(size_t)u] += qb + 2;
+      }
+    const int64_t span = *std::max_element(load.begin(), load.end());
+    if (best_span < 0 || span <= best_span) {
+      best_span = span;
+      best = G;
+    }
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  known[key] = best;
+  return best;
+}
+
 template <typename T, typename OutT, int D, bool CAUSAL, int NW>
 int launch_mfma_nw(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
                    hipStream_t st, int per_cu = NW == 4 ? 2 : 1) {
@@ -455,9 +531,11 @@ int launch_mfma_nw(const void* Q, const void* K, const void* V, void* O, int64_t
   if (units > 0x7fffffff) return HEXMI_ENOTSUP;
   const int64_t blocks = resident_grid(units, per_cu);
   if (blocks <= 0) return HEXMI_ELAUNCH;
+  const int groups = CAUSAL ? plan_causal_groups(ZH, nqb, blocks) : 0;
   hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, CAUSAL, false, NW>), dim3((unsigned)blocks), dim3(NW * 64), 0, st,
                      static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
-                     static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e);
+                     static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e, static_cast<const T*>(nullptr), 0, 0.0f,
+                     groups);
   return launch_status();
 }
 

@@ -369,3 +369,19 @@ def test_attention_more_units_than_resident_workgroups(hexmi, case, causal):
     want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal,
                                                             scale=scale)
     assert (got - want).abs().max() <= 5e-3
+
+
+@pytest.mark.parametrize("case", [(1, 32, 3840, 128), (1, 32, 2176, 128), (1, 24, 5120, 128), (1, 64, 2176, 64)])
+def test_causal_attention_block_counts_off_the_power_of_two(hexmi, case):
+    # causal units of unequal length are dealt to the persistent workgroups in groups of heads, longest first and
+    # padded to whole passes (15, 9, 20 query blocks of 256 rows on 32 workgroups per XCD; 17 blocks of 128 rows on
+    # 96): every unit must be visited exactly once, so the output starts as NaN. Oracle: the PyTorch CPU call the
+    # reference's test uses (test/python/triton/test_flash_attention.py:212).
+    Z, H, S, D = case
+    q, k, v = _qkv(Z, H, S, D, torch.float16, seed=21)
+    scale = 1.0 / math.sqrt(D)
+    out = torch.full((Z, H, S, D), float("nan"), dtype=torch.float32, device="cuda")
+    got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, True, out=out).cpu()
+    assert not torch.isnan(got).any()
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True, scale=scale)
+    assert (got - want).abs().max() <= 5e-3
