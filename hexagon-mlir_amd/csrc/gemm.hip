@@ -1115,6 +1115,22 @@ int launch_tiled(const T* A, const T* B, OutT* C, int64_t M, int64_t N, int64_t 
   return launch_status();
 }
 
+// 256 x 256 or 128 x 128 tiles. Either kind runs one workgroup per CU at a time, so a launch is whole rounds over
+// the CUs and the last round may be nearly empty. With every round full the large tiles run about 1.3 times the
+// rate of the small ones (fp16 K = 4096: 1.4 against 1.08 PFLOP/s; int8 weights: 1.2 against 0.93), and a round
+// that is not full runs its tiles somewhat faster: the large tiles are taken when 1.48 times the fill of their
+// rounds is at least the fill of the small tiles' rounds. (fp16, K = 4096, 256 CUs: 128 large tiles 825 TFLOP/s
+// against 1074 with small ones, 289 tiles 920 against 1019, 192 tiles 1152 against 1077, 324 tiles 1020 against 965;
+// int8 weights, N = 11008: M = 512 518 against 680, M = 768 739 against 687.)
+inline bool prefer_large_tiles(int64_t M, int64_t N) {
+  const int64_t cus = hexmi_num_cus();
+  if (cus <= 0) return false;
+  const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), small = ((M + 127) / 128) * ((N + 127) / 128);
+  const int64_t rounds_big = (big + cus - 1) / cus, rounds_small = (small + cus - 1) / cus;
+  if (big > (int64_t)1 << 40) return true;
+  return 148 * big * rounds_small >= 100 * small * rounds_big;
+}
+
 template <typename T, typename OutT, bool TRANS_B>
 int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldb, int64_t ldc, hipStream_t s, const void* bias_v, const void* resid_v, int64_t ldr) {
@@ -1131,10 +1147,10 @@ int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N
                     aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(C, 16) && (!bias || aligned_to(bias, run)) &&
                     (!resid || (aligned_to(resid, run) && ldr % 4 == 0));
   if (fast) {
-    const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    const bool large = prefer_large_tiles(M, N);
     // the large-tile kernels sit at the register limit and carry no epilogue operands: a product with bias or
     // residual runs on the 128x128 tiles at any size
-    if (big_tiles >= 128 && !bias && !resid)
+    if (large && !bias && !resid)
       return launch_tiled<T, OutT, 4, 4, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s, nullptr, nullptr, 0);
     return launch_tiled<T, OutT, 2, 2, TRANS_B>(A, B, C, M, N, K, lda, ldb, ldc, s, bias, resid, ldr);
   }
@@ -1200,8 +1216,7 @@ int fill_zero_2d(void* C, int64_t rows, int64_t cols, int64_t ld, int elem_size,
 // K % 32 == 0, N % 8 == 0, 16-byte aligned A / W / C / scales (checked by the caller).
 int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,
                      hipStream_t stream) {
-  const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= 128) return launch_w8a16<4, 4>(A, W, scales, C, M, N, K, stream);
+  if (prefer_large_tiles(M, N)) return launch_w8a16<4, 4>(A, W, scales, C, M, N, K, stream);
   return launch_w8a16<2, 2>(A, W, scales, C, M, N, K, stream);
 }
 
