@@ -519,6 +519,7 @@ inline int plan_causal_groups(int64_t ZH, int64_t nqb, int64_t grid) {
     }
   }
   std::lock_guard<std::mutex> lock(mu);
+  if (known.size() >= 1024) known.clear();                      // a caller with ever new shapes: start over
   known[key] = best;
   return best;
 }
