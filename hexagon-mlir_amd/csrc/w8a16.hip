@@ -223,17 +223,18 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
   }
 }
 
-// 2 < M <= 128 (MB = 1..8 blocks of 16 activation rows; K any multiple of 64): persistent
+// 2 < M <= 128 (MB = 1, 2, 3, 4, 6 or 8 blocks of 16 activation rows; K any multiple of 64): persistent
 // workgroups of 16 waves, each owning an equal contiguous range of at most 48 output channels, so the weights cross
-// HBM once, in contiguous row segments. K is walked in chunks of KC = 256 (MB <= 4) or 128 (MB = 8): an activation
-// chunk is at most 32 KiB; with MB <= 2 and one or two channel tiles the chunks are 768 or 384 k long (mid_kc()). The raw int8 weight chunk [48][KC] and the activation chunk [MB*16][KC] fp16 are copied
+// HBM once, in contiguous row segments. K is walked in chunks of KC = 256 (MB <= 4) or 128 (MB = 6, 8): an
+// activation chunk is at most 32 KiB; with MB <= 2 and one or two channel tiles the chunks are 768 or 384 k long
+// (mid_kc()). The raw int8 weight chunk [48][KC] and the activation chunk [MB*16][KC] fp16 are copied
 // global -> LDS (global_load_lds, no registers) by different waves: waves 12..15 copy weights, four chunks ahead
 // (five stages: three or four measured the same, seven and nine 5-10 % slower), waves 0..11 copy activations, two
 // chunks ahead (three stages; L2 hits). A wave's outstanding-copy counter only sees its own copies, so each role
 // waits with its own count and the workgroup barrier publishes both.
 // Compute wave w < 12 owns channel tile w % 3 and, of every chunk, one unit of 64 k for one group of row blocks
-// (four K units and all row blocks at KC = 256; two units and two groups of four row blocks at KC = 128; twelve
-// units of one tile at KC = 768 and six of each of two tiles at KC = 384, where no wave is left over). It converts
+// (four K units and all row blocks at KC = 256; two units and two groups of three or four row blocks at KC = 128;
+// twelve units of one tile at KC = 768 and six of each of two tiles at KC = 384, where no wave is left over). It converts
 // its 16 x 64 int8 weights to fp16 once per chunk (16 vector instructions) and multiplies them into its RB
 // accumulators (2 * RB MFMAs). A SIMD issues one instruction at a time and a 16x16x32 MFMA hides only two vector
 // instructions, so the conversions per MFMA set the pace: with one 16 x 16 tile per wave (every row-block wave
@@ -242,16 +243,16 @@ void w8a16_persist_kernel(const f16* __restrict__ A, const int8_t* __restrict__ 
 // permuted inside their row through the copies' source addresses (conflict-free). The K units of a tile are summed
 // through LDS after the K loop, in a fixed order, and the tile is stored row by row (one wave, one row's channels).
 // What a launch of this kernel costs besides the stream, from wall-clock stamps inside it (N = 11008, K = 4096,
-// weights from HBM, median workgroup): 0.2-0.4 us to the first copy, 1.3-1.8 us until its data is there, then a
-// chunk every 0.45 us at 16 rows (6.3 TB/s: the HBM rate), 0.73 us at 64 (activations through L2); 0.3 us from the
-// last chunk's barrier to the end of the loop and 0.7 us (16 rows) to 1.9 us (64, 128 rows) for the sum of the K
-// units and the stores.
+// weights from HBM, median workgroup): 0.5-0.7 us to the first copies (a weight wave needs another 0.5-0.8 us to
+// get its twelve issued), the first chunk there 2.4 us after the start, then a chunk every 0.45-0.5 us at 16 rows
+// (6.0-6.3 TB/s: the HBM rate), 0.73 us at 64 (activations through L2); 0.3 us from the last chunk's barrier to the
+// end of the loop and 0.5 us (16 rows) to 1.0 us (64, 128 rows) for the sum of the K units and the stores.
 // With every CU fetching all of A the kernel moves M * 8 KiB per CU through L2: 29 us at M = 128 (the 128 x 128
 // tile kernel, 86 tiles: 34), but 47 us at M = 256 with 64-k chunks (tile kernel: 37), so it stops at 128 rows.
 constexpr int kMidWeightPolicy = 2;                         // nt: weights are read once (12.4 against 13.0 us at M = 16)
 constexpr int kMidCh = 48;                                  // channels per workgroup (three tiles of 16)
 constexpr int kMidAStages = 3, kMidWStages = 5;
-constexpr int kMidCompute = 12;                             // compute waves: three channel tiles x four (unit, group)
+constexpr int kMidCompute = 12;                             // compute waves: (channel tile, K unit, row-block group)
 constexpr int kMidWWave0 = 12;                              // first of the four weight-copy waves
 constexpr int kMidMaxM = 128;
 // K per chunk. Sixteen rows leave LDS for longer chunks, and a workgroup with one or two channel tiles needs them:
@@ -336,8 +337,9 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     my_scale = scales[per_tensor ? 0 : (gn < n_end ? gn : n_end - 1)];
   }
 
-  // ---- copy slots: every copy moves 1 KiB (1024 / row bytes whole rows); lane positions are permuted inside a row
-  //      (see the fragment side). Slots past the last real copy repeat one (same bytes, rewritten).
+  // ---- copy slots: every copy moves 1 KiB, 64 consecutive 16-byte pieces of the stage (a row may end inside it);
+  //      lane positions are permuted inside a row (see the fragment side). Slots past the last real copy repeat one
+  //      (same bytes, rewritten).
   const char* slot_src[SL];                                 // source of this lane for chunk 0
   int slot_dst[SL];                                         // byte offset of the copy inside its stage
   int slot_lim[SL];                                         // largest chunk offset that keeps this lane inside its row
