@@ -613,6 +613,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     }
   }
 }
+
 #undef HEXMI_EITHER
 #undef HEXMI_LDS
 #undef HEXMI_GLB

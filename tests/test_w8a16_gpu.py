@@ -119,7 +119,11 @@ def test_w8a16_short_last_chunk_ignores_what_lies_behind_the_row(hexmi):
 
 
 @pytest.mark.parametrize("M,N,K", [(4, 14336, 512), (16, 14336, 4096), (9, 28672, 768), (16, 22016, 1024),
-                                   (64, 14336, 1024), (128, 22016, 512), (32, 13824, 5120)])
+                                   (64, 14336, 1024), (128, 22016, 512), (32, 13824, 5120),
+                                   # up to 16 rows, two workgroups per CU at a time: one chunk, short last chunks,
+                                   # a last workgroup with fewer channels, several rounds
+                                   (16, 14336, 256), (3, 13000, 832), (16, 13000, 64), (8, 40000, 640),
+                                   (16, 22016, 1984), (5, 52000, 320), (16, 12300, 1280)])
 def test_w8a16_more_than_a_workgroup_of_channels_per_cu(hexmi, oracle, M, N, K):
     # N beyond 48 channels per CU: equal workgroups in whole rounds, two at a time per CU with up to 16 rows;
     # the oracle covers every 29th output channel and the first and last 64
