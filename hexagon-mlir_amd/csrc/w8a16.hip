@@ -536,6 +536,10 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
     if (computes) {
       if (togo > 3) issue_a(chunk + 3, sa);
       if (reads) read_frags(nxt, sa1, sw1);
+      // With one row block the round is short and the order of its few instructions shows: the next chunk's reads
+      // go out whole before the first MFMA (2-3 % at sixteen rows under graph replay). With more row blocks the
+      // compiler's own interleaving is as good or better.
+      if constexpr (MB == 1) __builtin_amdgcn_sched_barrier(0);
       multiply(cur, chunk);
     } else if (copies_w) {
       if (togo > WS) issue_w(chunk + WS, sw);
