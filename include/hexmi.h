@@ -148,6 +148,11 @@ int hexmi_matmul_f16f16_f32(int64_t n_row, int64_t n_col, int64_t n_inner,
  *     test/python/torch-mlir/test_hexkl_macro_matmul.py:24-28).
  * in_dtype: HEXMI_F16 or HEXMI_BF16 (A and B). out_dtype: in_dtype or HEXMI_F32
  * (the fp16 x fp16 -> fp32 form of docs/tutorials/triton/matmul_hexkl.md:61-97).
+ * Any shape, leading dimension and alignment of the element type is taken.
+ * Fastest: K % 64 == 0, operand rows on 16-byte boundaries (lda, ldb
+ * multiples of 8, aligned bases), B as [K,N] with N % 8 == 0; K % 8 == 0 or an
+ * odd N with B as [N,K] costs up to half the rate, unaligned operand rows about
+ * two thirds.
  * in_dtype == out_dtype == HEXMI_F32: fp32 operands multiplied in fp32 (no
  * rounding of the operands): the fp32 matmuls of the reference's torch-mlir
  * graphs (test/python/torch-mlir/test_add_matmul_softmax.py:25-29). K % 32 == 0

@@ -45,7 +45,11 @@ SHAPES = [
     (100, 72, 64), (300, 264, 128),          # ragged M / N on the tiled path
     (256, 256, 96), (300, 264, 160),         # K % 64 == 32: the four-stage 32-wide-slab kernel
     (384, 256, 320),                         # odd number of 64-wide slabs
-    (33, 17, 40), (1, 8, 8), (65, 130, 24), (7, 5, 3),   # generic path
+    (33, 17, 40), (1, 8, 8), (65, 130, 24), (7, 5, 3),   # any-shape kernel (and, [N,K] weights, the ragged-K one)
+    (300, 264, 1000), (130, 136, 72),        # K % 8 == 0 only: the 32-wide-slab kernel with a masked last slab
+    (200, 257, 96), (260, 1003, 72),         # ... with an odd N: rows leave through LDS ([N,K]); any-shape ([K,N])
+    (300, 1001, 256), (129, 70, 64),         # odd N, whole 64-wide slabs: the paired-slab kernel, element stores
+    (130, 136, 2049), (257, 129, 333),       # K % 8 != 0: unaligned rows, the any-shape kernel
 ]
 
 
@@ -101,6 +105,45 @@ def test_gemm_large_ragged_tiles(hexmi, dtype, trans_b):
     assert ((got[rows].double() - want).abs() <= 1e-5 * mag + 1e-30).all()
     got16 = hexmi.matmul(a.cuda(), b.cuda(), trans_b=trans_b).cpu()
     assert torch.equal(got16, got.to(dtype))          # the 16-bit result is the rounded fp32 result, staged or not
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gemm_odd_width_on_large_tiles(hexmi, dtype):
+    # [N,K] weights with an odd N and enough tiles for the 256x256 form (a vocabulary-sized projection): the same
+    # kernel as with the weight padded to a multiple of 8 rows, only the way out differs -- bit for bit
+    M, N, K = 4096, 8193, 128
+    a, b = _inputs(M, N, K, dtype, True, seed=13)
+    got = hexmi.matmul(a.cuda(), b.cuda(), trans_b=True)
+    b_pad = torch.cat([b, torch.zeros(7, K, dtype=dtype)])
+    want = hexmi.matmul(a.cuda(), b_pad.cuda(), trans_b=True)
+    assert torch.equal(got, want[:, :N])
+    rows = torch.arange(0, M, 97)
+    ref = a[rows].double() @ b.double().t()
+    assert (got.cpu()[rows].double() - ref).abs().max() <= 2e-2 * math.sqrt(K)
+
+
+def test_gemm_unaligned_views(hexmi):
+    # operands and result that start 2 bytes into their buffers, odd leading dimensions (C ABI only): the any-shape
+    # kernel; nothing outside the result's window is written
+    from hexmi import _lib
+    L = _lib.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    g = _gen(14)
+    for trans_b in (0, 1):
+        for M, N, K in ((200, 136, 264), (130, 77, 100), (64, 64, 64)):
+            lda, ldb, ldc = K + 3, (K if trans_b else N) + 5, N + 1
+            a_buf = (2 * torch.rand(M * lda + 1, generator=g) - 1).half().cuda()
+            b_buf = (2 * torch.rand((N if trans_b else K) * ldb + 1, generator=g) - 1).half().cuda()
+            c_buf = torch.full((M * ldc + 1,), 7.0, dtype=torch.float16, device="cuda")
+            rc = L.hexmi_gemm(M, N, K, a_buf.data_ptr() + 2, lda, b_buf.data_ptr() + 2, ldb, c_buf.data_ptr() + 2, ldc,
+                              1, 1, trans_b, st)
+            assert rc == 0
+            a = a_buf[1:].view(M, lda)[:, :K].contiguous()
+            b = b_buf[1:].view(-1, ldb)[:, :(K if trans_b else N)].contiguous()
+            want = hexmi.matmul(a, b, trans_b=bool(trans_b))
+            c = c_buf[1:].view(M, ldc)
+            assert close16(c[:, :N].contiguous(), want, max_ulp=1, atol=1e-4)
+            assert float(c_buf[0]) == 7.0 and (c[:, N:] == 7.0).all()
 
 
 def test_gemm_strided_operands(hexmi):
@@ -295,7 +338,8 @@ def _linear_ref(a, b, bias, resid, trans_b):
                                              (torch.float16, torch.float32), (torch.float32, torch.float32)])
 @pytest.mark.parametrize("shape", [(512, 2304, 768), (512, 768, 3072),      # GPT-2 small layers (64-k tiled kernel)
                                    (256, 256, 96),                           # 32-k tiled kernel
-                                   (100, 72, 40), (33, 50, 17),              # generic kernel (ragged, unaligned)
+                                   (100, 72, 40), (33, 50, 17),              # any-shape kernel (ragged, unaligned)
+                                   (260, 1003, 72), (130, 136, 1000),        # ragged-K kernel: rows through LDS / runs
                                    (1024, 1024, 1024)])
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_gemm_ex_bias_and_residual(hexmi, dtype, out_dtype, shape, trans_b):
