@@ -316,7 +316,7 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   const int r16 = lane % 16, kg = lane / 16;
   const int n_begin = blockIdx.x * chan_per_wg;
   const int n_end = n_begin + chan_per_wg < N ? n_begin + chan_per_wg : N;
-  const int n_chunks = (K + KC - 1) / KC;                   // TAIL: the last one may be short (K % 64 == 0)
+  const int n_chunks = (K + KC - 1) / KC;                   // TAIL: the last one may be short (K % 16 == 0)
   // Workgroup b walks K from chunk b % n_chunks on and wraps round. With every workgroup at the same k at the
   // same time, all the addresses in flight on the chip agree in their low bits when the weight rows are a power of
   // two long, and the memory channels those bits select take the whole load (N = 8192, M = 16: 20.9 us at
@@ -447,9 +447,9 @@ void w8a16_mid_kernel(const f16* __restrict__ A, const int8_t* __restrict__ W, c
   };
   auto multiply = [&](const Frags& f, int chunk) __attribute__((always_inline)) {
     f16x8 w0, w1;
-    // a unit past the end of K holds the bytes its copies were clamped to: its weights count as zeros (and so does
-    // its zero point)
-    const unsigned keep = !TAIL || k_chunk(chunk) * KC + ku * 64 < K ? 0xffffffffu : 0u;
+    // a lane's sixteen weights past the end of K (K % 16 == 0) are the bytes its copy was clamped to: they count as
+    // zeros (and so does their zero point)
+    const unsigned keep = !TAIL || k_chunk(chunk) * KC + (ku * 4 + kg) * 16 < K ? 0xffffffffu : 0u;
     if constexpr (TAIL) {
       const u32x4 raw = {f.raw[0] & keep, f.raw[1] & keep, f.raw[2] & keep, f.raw[3] & keep};
       cvt16(raw, w0, w1);                                   // converted once, used for every row block
@@ -915,8 +915,10 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
 #undef HEXMI_GEMV_ANY
     return launch_status();
   }
-  // the fast kernels read 16 bytes of a weight row per lane in 64-wide K steps; other shapes take the generic one
-  if (K % 64 != 0 || !aligned_to(A, 16) || !aligned_to(W, 16)) {
+  // the fast kernels copy 16 bytes of a weight row per lane: K % 16 == 0 and aligned bases; other shapes take the
+  // generic one. (K % 64 != 0 runs the chunked kernel, in passes of 128 rows where the tile kernel does not apply.)
+  const bool tile_kernel = !zp && !pt && M > 64 && K % 64 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8);
+  if (K % 16 != 0 || !aligned_to(A, 16) || !aligned_to(W, 16) || (K % 64 != 0 && K > (1 << 29))) {
     constexpr int MR = 4;
     const int64_t gy = (M + MR - 1) / MR;
     if (gy > 65535) return HEXMI_ENOTSUP;
@@ -940,7 +942,7 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
   }
   // more than 128 rows with a zero point or a per-tensor scale: the chunked kernel in passes of 128 rows (the tile
   // kernel has no such form; M = 256, N = 11008, K = 4096: 2 x 28 us against four passes of 20 through w8a16_kernel)
-  if ((zp || pt) && M > kMidMaxM && K <= (1 << 29)) {
+  if (((zp || pt) || (K % 64 != 0 && !tile_kernel)) && M > kMidMaxM && K <= (1 << 29)) {
     int rc = HEXMI_OK;
     for (int64_t m = 0; m < M && rc == HEXMI_OK; m += kMidMaxM) {
       const int64_t rows = M - m < kMidMaxM ? M - m : kMidMaxM;
@@ -948,7 +950,7 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
     }
     return rc;
   }
-  // the chunked kernel: any K (a multiple of 64 here)
+  // the chunked kernel: any K (a multiple of 16 here)
   if (M <= kMidMaxM && K <= (1 << 29)) {
     const int cus = hexmi_num_cus();
     if (cus <= 0) return HEXMI_ELAUNCH;
@@ -993,8 +995,7 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
 #undef HEXMI_MID_T
     return launch_status();
   }
-  if (!zp && !pt && M > 64 && K % 32 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8))
-    return gemm_w8a16_tiled(M, N, K, a, W, s, c, st);
+  if (tile_kernel) return gemm_w8a16_tiled(M, N, K, a, W, s, c, st);
   int rc = HEXMI_OK;
   for (int64_t m = 0; m < M && rc == HEXMI_OK; m += 64) {
     const int64_t left = M - m;

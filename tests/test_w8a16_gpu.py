@@ -102,6 +102,41 @@ def test_w8a16_chunked_kernel_takes_any_k(hexmi, oracle, M, N, K):
     assert close16(got, want, max_ulp=1, atol=2e-4)
 
 
+@pytest.mark.parametrize("M", [3, 16, 17, 64, 100, 128, 130, 300])
+@pytest.mark.parametrize("N", [100, 5000, 10000])
+@pytest.mark.parametrize("K", [16, 48, 80, 272, 1008, 1040, 4048])
+@pytest.mark.parametrize("zero_points", [False, True])
+def test_w8a16_inner_dimension_in_sixteens(hexmi, oracle, M, N, K, zero_points):
+    # K a multiple of 16 but not of 64: the chunked kernel masks a lane's sixteen weights past K (its copies are
+    # clamped to the row's end); more than 128 rows run it in passes
+    if zero_points and (M in (17, 100, 130) or K in (48, 1040)):
+        pytest.skip("zero points: a subset of the shapes")
+    a, w, s = _inputs(M, N, K, seed=K + M + 1)
+    zp = torch.randint(-128, 128, (N,), generator=_gen(K + M), dtype=torch.int8) if zero_points else None
+    got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda(), zero_points=None if zp is None else zp.cuda()).cpu()
+    if zp is None:
+        want = torch.from_numpy(oracle.matmul_w8a16(a.numpy(), w.numpy(), s.numpy()))
+    else:
+        want = torch.from_numpy(oracle.matmul_w8a16_ex(a.numpy(), w.numpy(), s.numpy(), zero_points=zp.numpy()))
+    assert close16(got, want, max_ulp=1, atol=2e-4)
+
+
+def test_w8a16_sixteen_wide_tail_ignores_what_lies_behind_the_row(hexmi):
+    # K = 784 = 768 + 16: of the last chunk one sixteenth is inside the row; the copies of the rest are clamped to the
+    # row's end, where the largest weights and activations sit (their true products are zero)
+    M, N, K = 16, 64, 784
+    a = torch.zeros(M, K, dtype=torch.float16)
+    a[:, -8:] = 60000.0
+    a[:, 0] = 1.0
+    w = torch.zeros(N, K, dtype=torch.int8)
+    w[:, -16:] = 127
+    w[:, -8:] = 0
+    w[:, 0] = torch.arange(N, dtype=torch.int8)
+    s = torch.ones(N, dtype=torch.float16)
+    c = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda()).cpu()
+    assert torch.equal(c.float(), torch.arange(N).float().repeat(M, 1))
+
+
 def test_w8a16_short_last_chunk_ignores_what_lies_behind_the_row(hexmi):
     # K = 832 = 768 + 64: the copies of the last chunk are clamped to the row's end and their units count as zeros,
     # whatever the bytes there are: the largest weights and activations in the last 16 bytes of every row
