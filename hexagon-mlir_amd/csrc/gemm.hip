@@ -261,7 +261,8 @@ template <typename OutT> struct RaggedStage {
 template <typename OutT, int WM, int WN, int NW, int BM, int BN>
 __device__ __forceinline__ void store_tile_by_rows(const f32x16 (&acc)[WM][WN], OutT* c_s, OutT* C, int64_t ldc,
                                                    const OutT* bias, const OutT* resid, int64_t ldr, int M, int N, int m0,
-                                                   int n0, int wm, int wn, int wave, int lane) {
+                                                   int n0, int wm, int wn, int wave, int lane,
+                                                   const f16* scales = nullptr, int per_tensor = 0) {
   constexpr int PR = RaggedStage<OutT>::kRows, PITCH = RaggedStage<OutT>::pitch(BN);
 #pragma unroll
   for (int p = 0; p < BM / PR; ++p) {
@@ -276,6 +277,11 @@ __device__ __forceinline__ void store_tile_by_rows(const f32x16 (&acc)[WM][WN], 
           const int col = (wn * WN + j) * 32 + 8 * q + 4 * (lane / 32);
           f32x4 c = {acc[t % WM][j][q * 4 + 0], acc[t % WM][j][q * 4 + 1], acc[t % WM][j][q * 4 + 2],
                      acc[t % WM][j][q * 4 + 3]};
+          if (scales) {                                  // weight-only quantised B: the channel scale on the finished sum
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (n0 + col + r < N) c[r] *= (float)scales[per_tensor ? 0 : n0 + col + r];
+          }
           if (bias || resid) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -1084,12 +1090,33 @@ __device__ __forceinline__ u32x4 load_chunk_any(const T* p, int valid) {
   return v;
 }
 
-template <typename T, typename OutT, bool TRANS_B>
+// Eight int8 weights (any alignment, `valid` of them inside the row) minus the zero point, as eight fp16: exact.
+__device__ __forceinline__ u32x4 load_chunk_i8(const int8_t* p, int valid, int zero_point) {
+  int8_t b[kChunk];
+  if (valid >= kChunk) {
+    __builtin_memcpy(b, p, kChunk);                 // one global_load_dwordx2
+  } else {
+#pragma unroll
+    for (int t = 0; t < kChunk; ++t) b[t] = t < valid ? p[t] : (int8_t)0;
+  }
+  union { f16 h[kChunk]; u32x4 v; } u;
+#pragma unroll
+  for (int t = 0; t < kChunk; ++t) u.h[t] = t < valid ? (f16)(float)((int)b[t] - zero_point) : (f16)0.0f;
+  return u.v;
+}
+
+// B_I8: B is int8 [N,K] (needs TRANS_B, fp16 A and C): (W - zero_point) is formed in fp16 on the way into LDS and the
+// finished sums are multiplied by scales[column] (one scale and zero point for the tensor with per_tensor).
+template <typename T, typename OutT, bool TRANS_B, bool B_I8 = false>
 __global__ __launch_bounds__(256)
-void gemm_kernel_any(const T* __restrict__ A, const T* __restrict__ B, OutT* C, int M, int N, int K, int64_t lda,
+void gemm_kernel_any(const T* __restrict__ A, const void* __restrict__ Bv, OutT* C, int M, int N, int K, int64_t lda,
                      int64_t ldb, int64_t ldc, int tiles_m, int tiles_n, const OutT* __restrict__ bias = nullptr,
-                     const OutT* resid = nullptr, int64_t ldr = 0) {
+                     const OutT* resid = nullptr, int64_t ldr = 0, const f16* __restrict__ scales = nullptr,
+                     const int8_t* __restrict__ zero_points = nullptr, int per_tensor = 0) {
   static_assert(sizeof(T) == 2, "16-bit operands");
+  static_assert(!B_I8 || (TRANS_B && std::is_same<T, f16>::value), "int8 B is [N,K] and multiplies fp16 A");
+  const T* B = static_cast<const T*>(Bv);
+  const int8_t* B8 = static_cast<const int8_t*>(Bv);
   typedef typename Mfma<T>::Frag Frag;
   constexpr int WM = 2, WN = 2, NW = 4, BM = 128, BN = 128;
   __shared__ __attribute__((aligned(16))) T a_s[2][BM * BK];
@@ -1113,7 +1140,8 @@ void gemm_kernel_any(const T* __restrict__ A, const T* __restrict__ B, OutT* C, 
   // [K,N] tile: chunk e -> slab row e / 16, source chunk e % 16. LDS positions as in KMajorLoader / NMajorLoader.
   const T* a_ptr[2];
   const T* b_ptr[2];
-  int a_k[2], b_k[2], a_pos[2], b_pos[2], b_valid_n[2];
+  const int8_t* b8_ptr[2];
+  int a_k[2], b_k[2], a_pos[2], b_pos[2], b_valid_n[2], b_zero[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int e = j * 256 + tid;
@@ -1129,10 +1157,12 @@ void gemm_kernel_any(const T* __restrict__ A, const T* __restrict__ B, OutT* C, 
       const int row = e / 4, c = e % 4;
       int grow = n0 + row;
       grow = grow < N - 1 ? grow : N - 1;
-      b_ptr[j] = B + (int64_t)grow * ldb + c * kChunk;
+      if constexpr (B_I8) b8_ptr[j] = B8 + (int64_t)grow * ldb + c * kChunk;
+      else b_ptr[j] = B + (int64_t)grow * ldb + c * kChunk;
       b_k[j] = c * kChunk;
       b_pos[j] = row * BK + ((c ^ swz_k(row)) * kChunk);
       b_valid_n[j] = kChunk;
+      b_zero[j] = B_I8 && zero_points ? (int)zero_points[per_tensor ? 0 : grow] : 0;
     } else {
       constexpr int CPR = BN / kChunk;
       const int k = e / CPR, c = e % CPR;
@@ -1150,7 +1180,10 @@ void gemm_kernel_any(const T* __restrict__ A, const T* __restrict__ B, OutT* C, 
     for (int j = 0; j < 2; ++j) {
       const int left = K - (k0 + a_k[j]);                    // elements of this chunk before the end of K
       ra[j] = load_chunk_any<T>(a_ptr[j] + k0, left < 0 ? 0 : left);
-      if constexpr (TRANS_B) {
+      if constexpr (B_I8) {
+        const int leftb = K - (k0 + b_k[j]);
+        rb[j] = load_chunk_i8(b8_ptr[j] + k0, leftb < 0 ? 0 : leftb, b_zero[j]);
+      } else if constexpr (TRANS_B) {
         const int leftb = K - (k0 + b_k[j]);
         rb[j] = load_chunk_any<T>(b_ptr[j] + k0, leftb < 0 ? 0 : leftb);
       } else {
@@ -1190,7 +1223,8 @@ void gemm_kernel_any(const T* __restrict__ A, const T* __restrict__ B, OutT* C, 
     if (kt + 1 < KT) stash(stage ^ 1);
     __syncthreads();
   }
-  store_tile_by_rows<OutT, WM, WN, NW, BM, BN>(acc, c_s, C, ldc, bias, resid, ldr, M, N, m0, n0, wm, wn, wave, lane);
+  store_tile_by_rows<OutT, WM, WN, NW, BM, BN>(acc, c_s, C, ldc, bias, resid, ldr, M, N, m0, n0, wm, wn, wave, lane,
+                                               B_I8 ? scales : nullptr, per_tensor);
 }
 
 // fp32 inputs (the reference's torch-mlir graphs multiply fp32 matrices, e.g.
@@ -1452,6 +1486,17 @@ int fill_zero_2d(void* C, int64_t rows, int64_t cols, int64_t ld, int elem_size,
   if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
   hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, static_cast<char*>(C), rows, cols,
                      ld, elem_size);
+  return launch_status();
+}
+
+// Any K and alignment: the register-staged 128x128 kernel with int8 B (zero points and a per-tensor scale included).
+int gemm_w8a16_any_shape(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales,
+                         const int8_t* zero_points, int per_tensor, f16* C, hipStream_t stream) {
+  const int64_t tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
+  if (tiles_m * tiles_n > 0x7fffffff || K > 0x7fffffff - 64) return HEXMI_ENOTSUP;
+  hipLaunchKernelGGL((gemm_kernel_any<f16, f16, true, true>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, stream, A,
+                     static_cast<const void*>(W), C, (int)M, (int)N, (int)K, K, K, N, (int)tiles_m, (int)tiles_n, nullptr,
+                     nullptr, 0, scales, zero_points, per_tensor);
   return launch_status();
 }
 

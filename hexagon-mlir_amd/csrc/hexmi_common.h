@@ -223,6 +223,8 @@ int block_sum_any(const void* x, void* out, int64_t n, int64_t block, int dtype,
 // Tiled W8A16 GEMM for many activation rows (gemm.hip): C[M,N] = (A[M,K] * W[N,K]^T) * scales[N].
 int gemm_w8a16_tiled(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales, f16* C,
                      hipStream_t stream);
+int gemm_w8a16_any_shape(int64_t M, int64_t N, int64_t K, const f16* A, const int8_t* W, const f16* scales,
+                         const int8_t* zero_points, int per_tensor, f16* C, hipStream_t stream);
 
 // W8A16 on a (channel range x K part) decomposition with the K parts summed through a caller workspace
 // (w8a16_split.hip). w8a16_split_workspace: bytes the shape needs (0: one K part, or a shape the kernel does not

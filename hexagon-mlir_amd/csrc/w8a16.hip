@@ -919,6 +919,11 @@ int gemm_w8a16_any(int64_t M, int64_t N, int64_t K, const void* A, const int8_t*
   // generic one. (K % 64 != 0 runs the chunked kernel, in passes of 128 rows where the tile kernel does not apply.)
   const bool tile_kernel = !zp && !pt && M > 64 && K % 64 == 0 && N % 8 == 0 && aligned_to(C, 16) && aligned_to(scales, 8);
   if (K % 16 != 0 || !aligned_to(A, 16) || !aligned_to(W, 16) || (K % 64 != 0 && K > (1 << 29))) {
+    // Enough output for it: 128x128 tiles on the matrix cores, the slabs staged through registers at any alignment
+    // (N = 11008, K = 4040: M = 64 1.43 -> 0.14 ms, M = 1024 22.5 -> 0.23 ms). With few tiles that kernel waits out a
+    // memory latency per slab (about 110 us at K = 4040 whatever the rows), and the kernel below, a wave per channel
+    // with lanes striding over k, is ahead while M * N stays small (M = 16: 76 us at N = 4096, 371 at N = 11008).
+    if (M > 8 && M * N >= 98304) return gemm_w8a16_any_shape(M, N, K, a, W, s, zp, pt, c, st);
     constexpr int MR = 4;
     const int64_t gy = (M + MR - 1) / MR;
     if (gy > 65535) return HEXMI_ENOTSUP;

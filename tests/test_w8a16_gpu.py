@@ -121,6 +121,27 @@ def test_w8a16_inner_dimension_in_sixteens(hexmi, oracle, M, N, K, zero_points):
     assert close16(got, want, max_ulp=1, atol=2e-4)
 
 
+@pytest.mark.parametrize("M", [9, 64, 130, 300])
+@pytest.mark.parametrize("N", [100, 1000, 1027])
+@pytest.mark.parametrize("K", [1, 17, 100, 1001, 4040])
+@pytest.mark.parametrize("mode", ["plain", "zero_points", "per_tensor"])
+def test_w8a16_unaligned_rows_on_the_matrix_cores(hexmi, oracle, M, N, K, mode):
+    # K not a multiple of 16: weight rows start at any byte; more than 8 activation rows run 128x128 tiles whose slabs
+    # come through registers (8-byte weight loads at any alignment, guarded bytes at the end of a row)
+    a, w, s = _inputs(M, N, K, seed=K + M + N)
+    zp = None
+    if mode == "zero_points":
+        zp = torch.randint(-128, 128, (N,), generator=_gen(K + N), dtype=torch.int8)
+    elif mode == "per_tensor":
+        s = s[:1].contiguous()
+        zp = torch.tensor([-7], dtype=torch.int8)
+    got = hexmi.w8a16_matmul(a.cuda(), w.cuda(), s.cuda(), zero_points=None if zp is None else zp.cuda()).cpu()
+    want = torch.from_numpy(oracle.matmul_w8a16_ex(a.numpy(), w.numpy(), s.numpy(),
+                                                   zero_points=None if zp is None else zp.numpy(),
+                                                   per_tensor=mode == "per_tensor"))
+    assert close16(got, want, max_ulp=1, atol=2e-4)
+
+
 def test_w8a16_sixteen_wide_tail_ignores_what_lies_behind_the_row(hexmi):
     # K = 784 = 768 + 16: of the last chunk one sixteenth is inside the row; the copies of the rest are clamped to the
     # row's end, where the largest weights and activations sit (their true products are zero)
