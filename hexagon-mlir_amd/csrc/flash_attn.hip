@@ -67,12 +67,16 @@ struct MaskTileLoader {
 // MASK_LDS (GENERAL, 8 waves, a mask with Skv % 8 == 0): the mask tiles are copied global -> LDS one key block ahead
 // like K and V (no registers, whole 128-byte rows), instead of being loaded into registers in 8-byte runs at the
 // top of the block that uses them.
-template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, int NW = 4, bool MASK_LDS = false>
+// PADDED: the head is head_dim < D wide (a multiple of 8): Q, K, V and O rows are head_dim elements apart, the tiles
+// carry zero columns from head_dim to D (they add nothing to Q K^T; the output columns there are not stored).
+template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, int NW = 4, bool MASK_LDS = false,
+          bool PADDED = false>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? (D == 64 && !GENERAL ? 3 : 2) : 1)
 void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                       OutT* __restrict__ O, int ZH, int S, float scale_log2e, const T* __restrict__ Mk = nullptr,
-                      int Skv_arg = 0, float mask_factor = 0.0f, int group_heads = 0) {
+                      int Skv_arg = 0, float mask_factor = 0.0f, int group_heads = 0, int head_dim = D) {
   static_assert(!(CAUSAL && GENERAL), "the causal kernel has as many keys as queries and no mask");
+  const int dh = PADDED ? head_dim : D;                 // elements between rows in memory
   static_assert(!MASK_LDS || (GENERAL && NW == 8), "staged mask tiles: general kernel, 8 waves");
   const int Skv = GENERAL ? Skv_arg : S;
   typedef typename MfmaT<T>::Frag Frag;
@@ -89,6 +93,18 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   constexpr int kBlockM = NW * 32;                  // query rows per workgroup
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int nqb = (S + kBlockM - 1) / kBlockM;
+  if constexpr (PADDED) {
+    // the zero columns of both stages of K and V, once: no copy ever writes there (the first barrier of the key loop
+    // lies between these writes and the first fragment read)
+    KvTileLoader<T, D, false, NW, true> kz;
+    KvTileLoader<T, D, true, NW, true> vz;
+    kz.init(wave, lane, dh);
+    vz.init(wave, lane, dh);
+    kz.zero_padding(k_lds0, lane);
+    kz.zero_padding(k_lds1, lane);
+    vz.zero_padding(v_lds0, lane);
+    vz.zero_padding(v_lds1, lane);
+  }
   // Persistent workgroups: the grid is at most what the chip holds at once, and a workgroup walks several (head,
   // query block) units, which takes the per-unit launch cost and the idle tail out of short causal units.
   // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): every XCD gets a list of whole heads, longest
@@ -127,8 +143,8 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       zh = unit % ZH;
       qb = nqb - 1 - unit / ZH;
     }
-    const int64_t base = (int64_t)zh * S * D;
-    const int64_t kv_base = (int64_t)zh * Skv * D;
+    const int64_t base = (int64_t)zh * S * dh;
+    const int64_t kv_base = (int64_t)zh * Skv * dh;
     const T* q_g = Q + base;
     const T* k_g = K + kv_base;
     const T* v_g = V + kv_base;
@@ -142,8 +158,10 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     {
       const int qr = qrow < S ? qrow : S - 1;
 #pragma unroll
-      for (int ds = 0; ds < DS; ++ds)
-        qf[ds] = *reinterpret_cast<const Frag*>(q_g + (int64_t)qr * D + ds * 16 + half * 8);
+      for (int ds = 0; ds < DS; ++ds) {
+        if (!PADDED || ds * 16 + half * 8 < dh) qf[ds] = *reinterpret_cast<const Frag*>(q_g + (int64_t)qr * dh + ds * 16 + half * 8);
+        else qf[ds] = Frag{};
+      }
     }
 
     f32x16 o_acc[DT];
@@ -157,10 +175,10 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     const int key_end = CAUSAL ? ((qb + 1) * kBlockM < S ? (qb + 1) * kBlockM : S) : Skv;
     const int n_steps = (key_end + kBlockN - 1) / kBlockN;
 
-    KvTileLoader<T, D, false, NW> k_loader;
-    KvTileLoader<T, D, true, NW> v_loader;
-    k_loader.init(wave, lane);
-    v_loader.init(wave, lane);
+    KvTileLoader<T, D, false, NW, PADDED> k_loader;
+    KvTileLoader<T, D, true, NW, PADDED> v_loader;
+    k_loader.init(wave, lane, dh);
+    v_loader.init(wave, lane, dh);
     MaskTileLoader<T> m_loader;
     const T* mask_wg = nullptr;
     if constexpr (MASK_LDS) {
@@ -393,14 +411,15 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     const float l_tot = l_i + other_half(l_i);
     const float inv_l = 1.0f / l_tot;
     if (qrow < S) {
-      OutT* o_row = O + base + (int64_t)qrow * D;
+      OutT* o_row = O + base + (int64_t)qrow * dh;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
           const int d = dt * 32 + 8 * q4 + 4 * half;
-          store4o<OutT>(o_row + d, o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l,
-                        o_acc[dt][q4 * 4 + 2] * inv_l, o_acc[dt][q4 * 4 + 3] * inv_l);
+          if (!PADDED || d < dh)
+            store4o<OutT>(o_row + d, o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l,
+                          o_acc[dt][q4 * 4 + 2] * inv_l, o_acc[dt][q4 * 4 + 3] * inv_l);
         }
     }
     __syncthreads();                                            // the next unit's copies reuse both stages
@@ -540,6 +559,23 @@ int launch_mfma_nw(const void* Q, const void* K, const void* V, void* O, int64_t
   return launch_status();
 }
 
+// A head of head_dim < D columns (a multiple of 8) on the kernel for D: 128-row workgroups, two per CU.
+template <typename T, typename OutT, int D, bool CAUSAL>
+int launch_mfma_padded(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, int head_dim,
+                       float scale_log2e, hipStream_t st) {
+  const int64_t nqb = (S + 127) / 128;
+  const int64_t units = nqb * ZH;
+  if (units > 0x7fffffff) return HEXMI_ENOTSUP;
+  const int64_t blocks = resident_grid(units, 2);
+  if (blocks <= 0) return HEXMI_ELAUNCH;
+  const int groups = CAUSAL ? plan_causal_groups(ZH, nqb, blocks) : 0;
+  hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, CAUSAL, false, 4, false, true>), dim3((unsigned)blocks), dim3(256), 0, st,
+                     static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                     static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e, static_cast<const T*>(nullptr), 0, 0.0f,
+                     groups, head_dim);
+  return launch_status();
+}
+
 template <typename T, typename OutT, int D>
 int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
                 bool causal, hipStream_t st) {
@@ -621,6 +657,16 @@ int dispatch_half(const void* Q, const void* K, const void* V, const void* mask,
   const bool plain = !mask && Skv == S;
   if (ok && plain && D == 128) return launch_mfma<T, OutT, 128>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
   if (ok && plain && D == 64) return launch_mfma<T, OutT, 64>(Q, K, V, O, ZH, S, scale_log2e, causal, st);
+  // other head sizes up to 128 in multiples of 8 (rows on 16-byte boundaries): the same kernels on tiles padded with
+  // zero columns to 64 or 128 ([2,16,2048,80] causal: 9.9 ms on the row-wise kernel)
+  if (ok && plain && D % 8 == 0 && D < 128) {
+    if (D < 64) {
+      if (causal) return launch_mfma_padded<T, OutT, 64, true>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
+      return launch_mfma_padded<T, OutT, 64, false>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
+    }
+    if (causal) return launch_mfma_padded<T, OutT, 128, true>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
+    return launch_mfma_padded<T, OutT, 128, false>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
+  }
   const bool general_ok = ok && !causal && Skv % 4 == 0 && Skv >= 4 && (!mask || aligned_to(mask, 8));
   if (general_ok && D == 128) return launch_mfma_general<T, OutT, 128>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
   if (general_ok && D == 64) return launch_mfma_general<T, OutT, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);

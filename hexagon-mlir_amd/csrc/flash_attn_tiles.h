@@ -57,7 +57,10 @@ template <int D> __device__ __forceinline__ int swz_vtile(int row) {
 // global -> LDS copy of one [64 keys][D] tile: 64*D/8/64/4 wave-wide instructions per wave. The per-lane element
 // offsets inside a tile do not change from tile to tile, so they are computed once; only a ragged last tile
 // (keys past the end of the sequence) needs its rows clamped.
-template <typename T, int D, bool IS_V, int NW = 4>
+// PADDED: the head is narrower than the tile (d % 8 == 0, d < D): rows are d elements apart in memory, and a lane
+// whose chunk lies past column d copies nothing -- its LDS positions, which no other lane ever writes, are zeroed
+// once by the kernel (zero_padding), so the tile reads as the head padded with zero columns.
+template <typename T, int D, bool IS_V, int NW = 4, bool PADDED = false>
 struct KvTileLoader {
   static constexpr int CPR = D / 8;                       // chunks per row
   static constexpr int NI = kBlockN * CPR / 64 / NW;      // instructions per wave
@@ -69,17 +72,29 @@ struct KvTileLoader {
   int off0;                                               // element offset of this lane's chunk inside a tile, j = 0
   int row0, col0;
   int lds_off0;
-  __device__ __forceinline__ void init(int wave, int lane) {
+  int d;                                                  // elements between rows in memory (D unless PADDED)
+  bool live;                                              // this lane's chunk is inside the head
+  __device__ __forceinline__ void init(int wave, int lane, int head_dim = D) {
     const int lin = wave * 64 + lane;
     row0 = lin / CPR;
     col0 = ((lin % CPR) ^ (IS_V ? swz_vtile<D>(row0) : swz_ktile<D>(row0))) * 8;
-    off0 = row0 * D + col0;
+    d = PADDED ? head_dim : D;
+    live = !PADDED || col0 < d;
+    off0 = row0 * d + col0;
     lds_off0 = wave * 64 * 8;
+  }
+  // PADDED: zeros where this lane would have copied, in one stage
+  __device__ __forceinline__ void zero_padding(T* lds, int lane) const {
+    if (!live) {
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+        *reinterpret_cast<u32x4*>(lds + lds_off0 + j * (NW * 64 * 8) + lane * 8) = u32x4{0u, 0u, 0u, 0u};
+    }
   }
   // instruction j of this wave's share of a tile that lies wholly inside the sequence
   __device__ __forceinline__ void issue_one_whole(int j, const T* __restrict__ g, int key0, T* lds) const {
-    const char* base = reinterpret_cast<const char*>(g + ((int64_t)key0 + j * kRowStep) * D);
-    copy_to_lds(base, off0 * (int)sizeof(T), lds + lds_off0 + j * (NW * 64 * 8));
+    const char* base = reinterpret_cast<const char*>(g + ((int64_t)key0 + j * kRowStep) * d);
+    if (live) copy_to_lds(base, off0 * (int)sizeof(T), lds + lds_off0 + j * (NW * 64 * 8));
   }
   // instruction j of this wave's share of the tile
   __device__ __forceinline__ void issue_one(int j, const T* __restrict__ g, int key0, int S, T* lds) const {
@@ -91,7 +106,7 @@ struct KvTileLoader {
       const char* base = reinterpret_cast<const char*>(g);
       int key = key0 + row0 + j * kRowStep;
       key = key < S ? key : S - 1;
-      copy_to_lds(base, (key * D + col0) * (int)sizeof(T), dst);
+      if (live) copy_to_lds(base, (key * d + col0) * (int)sizeof(T), dst);
     }
   }
   __device__ __forceinline__ void issue(const T* __restrict__ g, int key0, int S, T* lds) const {

@@ -54,6 +54,41 @@ def test_attention_parity_half(hexmi, oracle, case, dtype, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", [(1, 2, 300, 80), (2, 1, 129, 96), (1, 3, 64, 32), (1, 1, 513, 8), (2, 8, 200, 48),
+                                  (1, 1, 1000, 120), (1, 2, 77, 16), (1, 1, 260, 112), (1, 16, 384, 40), (1, 1, 1, 72)])
+def test_attention_other_head_sizes(hexmi, oracle, case, dtype, causal):
+    # head sizes below 128 in multiples of 8 run the matrix-core kernel for 64 or 128 on tiles padded with zero
+    # columns; the output buffer starts as NaN and has one row more than the result, which must stay as it is
+    Z, H, S, D = case
+    q, k, v = _qkv(Z, H, S, D, dtype, seed=D + S)
+    scale = 1.0 / math.sqrt(D)
+    buf = torch.full((Z * H * S + 1, D), float("nan"), dtype=dtype, device="cuda")
+    out = buf[:Z * H * S].view(Z, H, S, D)
+    hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal, out=out)
+    want = _oracle(oracle, q, k, v, scale, causal)
+    tol = 2e-2 if dtype == torch.float16 else 4e-2
+    assert (out.cpu().float() - want).abs().max() <= tol
+    assert torch.isnan(buf[-1]).all()
+    got32 = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal, out_dtype=torch.float32).cpu()
+    assert (got32 - want).abs().max() <= (5e-3 if dtype == torch.float16 else 3e-2)
+
+
+def test_attention_padded_head_equals_the_zero_padded_problem(hexmi):
+    # head size 80 on the kernel for 128 is the 128-wide problem with 48 zero columns in Q, K and V (and 1/sqrt(80)):
+    # the same kernel, the same arithmetic -- bit for bit
+    Z, H, S, D = 2, 8, 700, 80
+    q, k, v = _qkv(Z, H, S, D, torch.float16, seed=31)
+    scale = 1.0 / math.sqrt(D)
+    for causal in (False, True):
+        got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal).cpu()
+        qp, kp, vp = (torch.nn.functional.pad(t, (0, 48)) for t in (q, k, v))
+        want = hexmi.flash_attention(qp.cuda(), kp.cuda(), vp.cuda(), scale, causal).cpu()
+        assert torch.equal(got, want[..., :D])
+        assert (want[..., D:] == 0).all()
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("case", [(1, 1, 1024, 64), (1, 2, 100, 128), (2, 2, 65, 32), (1, 1, 130, 80),
                                   # head sizes 64 and 128 run on the fp32 matrix cores: ragged query and key blocks,
                                   # several workgroups per head, a single row
