@@ -597,10 +597,22 @@ int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH
   return launch_mfma_nw<T, OutT, D, false, 4>(Q, K, V, O, ZH, S, scale_log2e, st);
 }
 
+// head_dim < D: the 128-row form on padded tiles (the mask comes straight from global memory)
 template <typename T, typename OutT, int D>
 int launch_mfma_general(const void* Q, const void* K, const void* V, const void* mask, void* O, int64_t ZH, int64_t S,
-                        int64_t Skv, float scale_log2e, hipStream_t st) {
+                        int64_t Skv, float scale_log2e, hipStream_t st, int head_dim = D) {
   const float mask_factor = 1.44269504088896340736f / scale_log2e;     // mask / sm_scale
+  if (head_dim < D) {
+    const int64_t units = (S + 127) / 128 * ZH;
+    if (units > 0x7fffffff) return HEXMI_ENOTSUP;
+    const int64_t blocks = resident_grid(units, 2);
+    if (blocks <= 0) return HEXMI_ELAUNCH;
+    hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, D, false, true, 4, false, true>), dim3((unsigned)blocks), dim3(256), 0, st,
+                       static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                       static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e, static_cast<const T*>(mask), (int)Skv,
+                       mask_factor, 0, head_dim);
+    return launch_status();
+  }
   // a mask whose rows are whole 16-byte chunks is staged through LDS by 256-row workgroups (one per CU); the
   // copies address a workgroup's 256 mask rows with 32-bit byte offsets
   if (mask != nullptr && Skv % 8 == 0 && aligned_to(mask, 16) && S > 128 && Skv <= (1 << 21)) {
@@ -670,6 +682,8 @@ int dispatch_half(const void* Q, const void* K, const void* V, const void* mask,
   const bool general_ok = ok && !causal && Skv % 4 == 0 && Skv >= 4 && (!mask || aligned_to(mask, 8));
   if (general_ok && D == 128) return launch_mfma_general<T, OutT, 128>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
   if (general_ok && D == 64) return launch_mfma_general<T, OutT, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
+  if (general_ok && D % 8 == 0 && D < 64) return launch_mfma_general<T, OutT, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st, (int)D);
+  if (general_ok && D % 8 == 0 && D < 128) return launch_mfma_general<T, OutT, 128>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st, (int)D);
   return launch_rowwise<T, OutT>(Q, K, V, mask, O, ZH, S, Skv, D, scale_log2e, causal, st);
 }
 

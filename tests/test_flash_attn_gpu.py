@@ -259,7 +259,9 @@ MASKED_CASES = [(2, 128, 128, 128), (3, 200, 72, 64), (1, 1, 64, 128), (2, 77, 5
                 (1, 130, 1024, 128), (2, 65, 66, 64), (1, 40, 100, 80),   # the last two: Skv % 4 != 0 / other D
                 # more than 128 queries and Skv % 8 == 0: mask tiles staged through LDS by 256-row workgroups
                 # (ragged last row block, ragged last key block, several row blocks, many batch entries)
-                (3, 300, 520, 128), (2, 513, 72, 64), (1, 257, 2048 + 8, 128), (40, 129, 136, 64)]
+                (3, 300, 520, 128), (2, 513, 72, 64), (1, 257, 2048 + 8, 128), (40, 129, 136, 64),
+                # head sizes below 128 in multiples of 8: the 128-row kernel on tiles padded with zero columns
+                (2, 200, 72, 80), (1, 300, 520, 96), (3, 129, 136, 32), (1, 77, 516, 40), (2, 64, 64, 112)]
 
 
 @pytest.mark.parametrize("with_mask", [True, False])
