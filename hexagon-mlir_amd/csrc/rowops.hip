@@ -40,6 +40,31 @@ __device__ __forceinline__ void store16_stream(T* p, const Vec16<T>& r) {
   __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(r.v), reinterpret_cast<u32x4*>(p));
 }
 
+// Rows that do not start on 16-byte boundaries or do not end on a chunk boundary (RAGGED tiles): a whole chunk is one
+// 16-byte access at the alignment of the element type, which the hardware takes; the row's last, partial chunk goes
+// element by element (n of them; the rest of a loaded chunk is zero bits).
+template <typename T>
+__device__ __forceinline__ Vec16<T> load16_any(const T* p, int n) {
+  Vec16<T> r;
+  if (n >= Vec16<T>::N) {
+    __builtin_memcpy(r.v, p, 16);
+  } else {
+#pragma unroll
+    for (int i = 0; i < Vec16<T>::N; ++i) r.v[i] = i < n ? p[i] : T(0.0f);
+  }
+  return r;
+}
+template <typename T>
+__device__ __forceinline__ void store16_any(T* p, const Vec16<T>& r, int n) {
+  if (n >= Vec16<T>::N) {
+    __builtin_memcpy(p, r.v, 16);
+  } else {
+#pragma unroll
+    for (int i = 0; i < Vec16<T>::N; ++i)
+      if (i < n) p[i] = r.v[i];
+  }
+}
+
 // Reduce across the WAVES waves that share a row through LDS. `red` holds one float per wave and must not be
 // reused by another reduction of the same kernel (each reduction gets its own slots, so one barrier suffices);
 // every thread returns the combined value.
@@ -100,12 +125,14 @@ __device__ __forceinline__ float rsqrt_newton(float x) {
 // per-row mean / rstd (one lane stores them) are written one group late, between the wait for the loads and the
 // issue of the next ones.
 // Without PIPE a workgroup handles exactly one row group (gridDim.x == number of groups) and accesses are masked.
-template <typename T, int OP, int CHUNKS, int THREADS, int ROWS_PER_BLOCK, bool PIPE>
+// RAGGED (never with PIPE): rows at any alignment and of any length; the masks are per element.
+template <typename T, int OP, int CHUNKS, int THREADS, int ROWS_PER_BLOCK, bool PIPE, bool RAGGED = false>
 __global__ __launch_bounds__(THREADS * ROWS_PER_BLOCK)
 void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict__ w,
                 const T* __restrict__ b, float* __restrict__ mean_out, float* __restrict__ rstd_out,
                 int64_t rows, int cols, int64_t ld_x, int64_t ld_y, float eps) {
   constexpr bool FULL = PIPE;
+  static_assert(!(PIPE && RAGGED), "the pipelined walk is for exact tiles");
   // MIX (fp16 norms, pipelined walk): the row is kept as loaded and every first use converts it inside the
   // arithmetic (v_fma_mix_f32 reads an fp16 half of a register as one operand of an fp32 fma, at the issue cost of
   // a plain fma), instead of sixteen conversions per thread and row up front. The norms issue vector instructions
@@ -153,11 +180,16 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
   int load_col[CHUNKS];
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) load_col[c] = (c * THREADS + t) * N < cols ? (c * THREADS + t) * N : 0;
+  // RAGGED: elements of chunk c inside the row (a chunk past the end stands in for column 0's, as above)
+  auto left = [&](int c) { return cols - load_col[c]; };
   Vec16<T> raw_a[CHUNKS];
   {
     const T* xr = x + row_of(blockIdx.x) * ld_x;
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) raw_a[c] = load16_stream(xr + load_col[c]);
+    for (int c = 0; c < CHUNKS; ++c) {
+      if constexpr (RAGGED) raw_a[c] = load16_any(xr + load_col[c], left(c));
+      else raw_a[c] = load16_stream(xr + load_col[c]);
+    }
   }
   float one = 1.0f, zero = 0.0f;                       // opaque, so that x * one + y and x * y + zero stay fused
   if constexpr (MIX) asm volatile("" : "+v"(one), "+v"(zero));   // multiply-adds (the form that converts on the fly)
@@ -191,7 +223,9 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
       for (int c = 0; c < CHUNKS; ++c) {
         const bool in = FULL || (c * THREADS + t) * N < cols;
 #pragma unroll
-        for (int i = 0; i < N; ++i) v[c][i] = in ? to_f32<T>(raw[c].v[i]) : (OP == kSoftmax ? -INFINITY : 0.0f);
+        for (int i = 0; i < N; ++i)
+          v[c][i] = in && (!RAGGED || (c * THREADS + t) * N + i < cols) ? to_f32<T>(raw[c].v[i])
+                                                                         : (OP == kSoftmax ? -INFINITY : 0.0f);
       }
     }
     flush_stats();
@@ -222,7 +256,8 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
           Vec16<T> o;
 #pragma unroll
           for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i] * inv);
-          store16_stream(yr + col, o);
+          if constexpr (RAGGED) store16_any(yr + col, o, cols - col);
+          else store16_stream(yr + col, o);
         }
       }
     } else {
@@ -253,7 +288,7 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
               q = fmaf(v[c][i], v[c][i], q);
             } else if constexpr (MIX) {
               q = fmaf(to_f32<T>(raw[c].v[i]), to_f32<T>(raw[c].v[i]), q);
-            } else {
+            } else if (!RAGGED || (c * THREADS + t) * N + i < cols) {
               v[c][i] -= mean;
               q += v[c][i] * v[c][i];
             }
@@ -290,7 +325,8 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
             }
           } else {
             if (w) {
-              wv[c] = load16(w + col);
+              if constexpr (RAGGED) wv[c] = load16_any(w + col, cols - col);
+              else wv[c] = load16(w + col);
 #pragma unroll
               for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd * to_f32<T>(wv[c].v[i]);
             } else {
@@ -298,14 +334,16 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
               for (int i = 0; i < N; ++i) v[c][i] = v[c][i] * rstd;
             }
             if (OP == kLayerNorm && b) {
-              bv[c] = load16(b + col);
+              if constexpr (RAGGED) bv[c] = load16_any(b + col, cols - col);
+              else bv[c] = load16(b + col);
 #pragma unroll
               for (int i = 0; i < N; ++i) v[c][i] += to_f32<T>(bv[c].v[i]);
             }
           }
 #pragma unroll
           for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i]);
-          store16_stream(yr + col, o);
+          if constexpr (RAGGED) store16_any(yr + col, o, cols - col);
+          else store16_stream(yr + col, o);
         }
       }
     }
@@ -662,6 +700,23 @@ int dispatch_rows(const void* xv, void* yv, const void* wv, const void* bv, floa
     if (chunks <= 1024 * 8) HEXMI_TILE(8, 1024, 1, false);
   }
 #undef HEXMI_TILE
+  // Rows that are not whole aligned chunks (an odd number of columns, a view that starts anywhere): the same tiles
+  // with per-element masks and accesses at the alignment of the element type; one pass over the row instead of the
+  // three sweeps of the kernel below ([8192, 4097] fp16: softmax 62 us on that one, 24 us at 4096 columns).
+#define HEXMI_RAGGED(C, TH, RPB) \
+  { hipLaunchKernelGGL((row_kernel<T, OP, C, TH, RPB, false, true>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(TH * RPB), 0, s, \
+                       x, y, w, b, mean, rstd, rows, (int)cols, ld_x, ld_y, eps); return launch_status(); }
+  if (!vec_ok && rows <= 0x7fffffff) {
+    if (chunks <= 64 * 1) HEXMI_RAGGED(1, 64, 4);
+    if (chunks <= 64 * 2) HEXMI_RAGGED(2, 64, 4);
+    if (chunks <= 64 * 4) HEXMI_RAGGED(4, 64, 4);
+    if (chunks <= 256 * 2) HEXMI_RAGGED(2, 256, 1);
+    if (chunks <= 256 * 4) HEXMI_RAGGED(4, 256, 1);
+    if (chunks <= 512 * 4) HEXMI_RAGGED(4, 512, 1);
+    if (chunks <= 1024 * 4) HEXMI_RAGGED(4, 1024, 1);
+    if (chunks <= 1024 * 8) HEXMI_RAGGED(8, 1024, 1);
+  }
+#undef HEXMI_RAGGED
   if (rows > 0x7fffffff) return HEXMI_ENOTSUP;
   hipLaunchKernelGGL((row_kernel_generic<T, OP>), dim3((unsigned)rows), dim3(256), 0, s, x, y, w, b, mean, rstd, rows,
                      cols, ld_x, ld_y, eps);

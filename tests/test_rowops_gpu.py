@@ -351,3 +351,43 @@ def test_norm_statistics_at_the_edges_of_the_range(hexmi):
         assert torch.allclose(got[1:], want[1:], rtol=1e-5, atol=1e-6, equal_nan=True)
         var = x.double().var(-1, unbiased=False)
         assert torch.allclose(r.cpu()[1:].double(), 1.0 / torch.sqrt(var + eps)[1:], rtol=1e-5, equal_nan=True)
+
+
+RAGGED_COLS = [1, 7, 9, 63, 513, 1001, 2049, 4097, 8200 + 3, 12289, 32001, 50257]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("cols", RAGGED_COLS)
+def test_rows_that_are_not_whole_chunks(hexmi, oracle, dtype, cols):
+    # every tile of the one-pass kernel with per-element masks: rows of any length that start at any alignment of the
+    # element type (row r starts r * cols elements in), against the oracle; the output is a window between margins
+    rows = 9 if cols < 20000 else 3
+    g = _gen(cols)
+    x = (torch.randn(rows, cols, generator=g) * 2 + 0.3).to(dtype)
+    w = (1 + 0.1 * torch.randn(cols, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(cols, generator=g)).to(dtype)
+    a, tag = to_np(x)
+    wn, bn = to_np(w)[0], to_np(b)[0]
+
+    def window():
+        buf = torch.full((rows * cols + 64,), 5.0, dtype=dtype, device="cuda")
+        return buf, buf[32:32 + rows * cols].view(rows, cols)
+
+    buf, out = window()
+    hexmi.softmax(x.cuda(), out=out)
+    _check(out, from_np(oracle.softmax(a, dtype=tag), dtype), dtype, atol16=1e-7)
+    assert (buf[:32] == 5.0).all() and (buf[32 + rows * cols:] == 5.0).all()
+    buf, out = window()
+    hexmi.rms_norm(x.cuda(), w.cuda(), 1e-5, out=out)
+    _check(out, from_np(oracle.rms_norm(a, wn, 1e-5, dtype=tag), dtype), dtype)
+    assert (buf[:32] == 5.0).all() and (buf[32 + rows * cols:] == 5.0).all()
+    buf, out = window()
+    mean = torch.empty(rows, device="cuda")
+    rstd = torch.empty(rows, device="cuda")
+    hexmi.layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-5, out=out, mean=mean, rstd=rstd)
+    want, want_mean, want_rstd = oracle.layer_norm(a, wn, bn, 1e-5, dtype=tag)
+    _check(out, from_np(want, dtype), dtype, atol16=2e-6, atol32=2e-6)
+    assert (buf[:32] == 5.0).all() and (buf[32 + rows * cols:] == 5.0).all()
+    assert torch.allclose(mean.cpu(), torch.from_numpy(want_mean), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(rstd.cpu(), torch.from_numpy(want_rstd), rtol=1e-5)
+
