@@ -204,8 +204,10 @@ int hexmi_add_matmul_softmax(int64_t M, int64_t N, int64_t K, const void *x,
  * [N], one per output channel. Results are reproducible bit for bit; the order
  * of a channel's sum over k may depend on where the channel stands in W (for
  * 2 <= M <= 128 the workgroup that owns it sets the k it starts at), so moving a
- * channel can change its outputs in the last place. The reference has no such
- * kernel; this is the
+ * channel can change its outputs in the last place. Any K: multiples of 64
+ * are fastest, multiples of 16 cost little up to 128 rows (passes of 128 rows
+ * beyond), other K and unaligned bases run a register-staged tile kernel.
+ * The reference has no such kernel; this is the
  * fusion of quant.dcast lowering
  * (qcom_hexagon_backend/lib/Conversion/LinalgToLLVM/LinalgToLLVMPass.cpp:224-230)
  * with the transposed-weight matmul of test_hexkl_macro_matmul.py:24-28. */
@@ -304,6 +306,9 @@ int hexmi_gemm_w8a16_packed(int64_t M, int64_t N, int64_t K, const void *A,
  * test/python/triton/test_flash_attention.py:37-168 (STAGE=1 is causal == 0)
  * and tm_tensor.attention (include/hexagon/Dialect/TmTensor/IR/TmTensorOps.td:28-56).
  * in_dtype: HEXMI_F16 / HEXMI_BF16 (MFMA path) or HEXMI_F32.
+ * D: 64 and 128 are the kernels' own sizes; 16-bit heads below 128 in
+ * multiples of 8 run them on zero-padded tiles; anything else a slow
+ * row-wise kernel (D <= 256).
  * out_dtype: in_dtype, or HEXMI_F32 with fp16 inputs (the fp16 QKV -> fp32 O
  * form of test/python/mlir/hexkl_attention/input.mlir:1-169). */
 int hexmi_flash_attn_fwd(const void *Q, const void *K, const void *V, void *O,
