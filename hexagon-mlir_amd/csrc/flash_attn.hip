@@ -69,13 +69,17 @@ struct MaskTileLoader {
 // top of the block that uses them.
 // PADDED: the head is head_dim < D wide (a multiple of 8): Q, K, V and O rows are head_dim elements apart, the tiles
 // carry zero columns from head_dim to D (they add nothing to Q K^T; the output columns there are not stored).
+// WIDE (with PADDED, D = 128, four waves): a head of 128 < head_dim <= 256 columns as two 128-wide halves. The
+// scores are the sum over both halves' K tiles, the output two sets of accumulators, the second half's tiles padded
+// like a narrow head's; twice the LDS and about 100 registers more, so one workgroup per CU.
 template <typename T, typename OutT, int D, bool CAUSAL, bool GENERAL = false, int NW = 4, bool MASK_LDS = false,
-          bool PADDED = false>
-__global__ __launch_bounds__(NW * 64, NW == 4 ? (D == 64 && !GENERAL ? 3 : 2) : 1)
+          bool PADDED = false, bool WIDE = false>
+__global__ __launch_bounds__(NW * 64, NW == 4 && !WIDE ? (D == 64 && !GENERAL ? 3 : 2) : 1)
 void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                       OutT* __restrict__ O, int ZH, int S, float scale_log2e, const T* __restrict__ Mk = nullptr,
                       int Skv_arg = 0, float mask_factor = 0.0f, int group_heads = 0, int head_dim = D) {
   static_assert(!(CAUSAL && GENERAL), "the causal kernel has as many keys as queries and no mask");
+  static_assert(!WIDE || (PADDED && D == 128 && NW == 4 && !GENERAL), "two halves of 128 columns, four waves, no mask");
   const int dh = PADDED ? head_dim : D;                 // elements between rows in memory
   static_assert(!MASK_LDS || (GENERAL && NW == 8), "staged mask tiles: general kernel, 8 waves");
   const int Skv = GENERAL ? Skv_arg : S;
@@ -87,6 +91,11 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
   __shared__ __attribute__((aligned(16))) T k_lds1[kBlockN * D];
   __shared__ __attribute__((aligned(16))) T v_lds0[kBlockN * D];
   __shared__ __attribute__((aligned(16))) T v_lds1[kBlockN * D];
+  // WIDE: the tiles of columns 128 .. 255
+  __shared__ __attribute__((aligned(16))) T kb_lds0[WIDE ? kBlockN * D : 8];
+  __shared__ __attribute__((aligned(16))) T kb_lds1[WIDE ? kBlockN * D : 8];
+  __shared__ __attribute__((aligned(16))) T vb_lds0[WIDE ? kBlockN * D : 8];
+  __shared__ __attribute__((aligned(16))) T vb_lds1[WIDE ? kBlockN * D : 8];
   __shared__ __attribute__((aligned(16))) T m_lds0[MASK_LDS ? NW * 32 * kBlockN : 8];
   __shared__ __attribute__((aligned(16))) T m_lds1[MASK_LDS ? NW * 32 * kBlockN : 8];
 
@@ -98,12 +107,12 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     // lies between these writes and the first fragment read)
     KvTileLoader<T, D, false, NW, true> kz;
     KvTileLoader<T, D, true, NW, true> vz;
-    kz.init(wave, lane, dh);
-    vz.init(wave, lane, dh);
-    kz.zero_padding(k_lds0, lane);
-    kz.zero_padding(k_lds1, lane);
-    vz.zero_padding(v_lds0, lane);
-    vz.zero_padding(v_lds1, lane);
+    kz.init(wave, lane, dh, WIDE ? dh - D : dh);
+    vz.init(wave, lane, dh, WIDE ? dh - D : dh);
+    kz.zero_padding(WIDE ? kb_lds0 : k_lds0, lane);
+    kz.zero_padding(WIDE ? kb_lds1 : k_lds1, lane);
+    vz.zero_padding(WIDE ? vb_lds0 : v_lds0, lane);
+    vz.zero_padding(WIDE ? vb_lds1 : v_lds1, lane);
   }
   // Persistent workgroups: the grid is at most what the chip holds at once, and a workgroup walks several (head,
   // query block) units, which takes the per-unit launch cost and the idle tail out of short causal units.
@@ -163,12 +172,25 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
         else qf[ds] = Frag{};
       }
     }
+    Frag qfb[WIDE ? DS : 1];                            // WIDE: columns 128 .. 255 of the query row
+    if constexpr (WIDE) {
+      const int qr = qrow < S ? qrow : S - 1;
+#pragma unroll
+      for (int ds = 0; ds < DS; ++ds) {
+        if (D + ds * 16 + half * 8 < dh) qfb[ds] = *reinterpret_cast<const Frag*>(q_g + (int64_t)qr * dh + D + ds * 16 + half * 8);
+        else qfb[ds] = Frag{};
+      }
+    }
 
     f32x16 o_acc[DT];
+    f32x16 o_accb[WIDE ? DT : 1];                       // WIDE: output columns 128 .. 255
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.0f;
+      for (int r = 0; r < 16; ++r) {
+        o_acc[dt][r] = 0.0f;
+        if constexpr (WIDE) o_accb[dt][r] = 0.0f;
+      }
     float m_i = -INFINITY;                              // running max (already multiplied by scale*log2e)
     float l_i = 0.0f;                                   // this lane's share of the running sum
 
@@ -177,27 +199,40 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
 
     KvTileLoader<T, D, false, NW, PADDED> k_loader;
     KvTileLoader<T, D, true, NW, PADDED> v_loader;
-    k_loader.init(wave, lane, dh);
-    v_loader.init(wave, lane, dh);
+    k_loader.init(wave, lane, dh, dh);
+    v_loader.init(wave, lane, dh, dh);
+    KvTileLoader<T, D, false, NW, PADDED> kb_loader;   // WIDE: the second halves, from 128 columns into the rows
+    KvTileLoader<T, D, true, NW, PADDED> vb_loader;
+    if constexpr (WIDE) {
+      kb_loader.init(wave, lane, dh, dh - D);
+      vb_loader.init(wave, lane, dh, dh - D);
+    }
     MaskTileLoader<T> m_loader;
     const T* mask_wg = nullptr;
     if constexpr (MASK_LDS) {
       mask_wg = Mk + ((int64_t)zh * S + qb * kBlockM) * Skv;
       m_loader.init(wave, lane, S - qb * kBlockM, Skv);
     }
-    auto load_kv = [&](int step, T* k_dst, T* v_dst, T* m_dst) __attribute__((always_inline)) {
+    auto load_kv = [&](int step, T* k_dst, T* v_dst, T* m_dst, T* kb_dst, T* vb_dst) __attribute__((always_inline)) {
       k_loader.issue(k_g, step * kBlockN, Skv, k_dst);
       v_loader.issue(v_g, step * kBlockN, Skv, v_dst);
+      if constexpr (WIDE) {
+        kb_loader.issue(k_g + D, step * kBlockN, Skv, kb_dst);
+        vb_loader.issue(v_g + D, step * kBlockN, Skv, vb_dst);
+      }
       if constexpr (MASK_LDS) m_loader.issue(mask_wg, step * kBlockN, Skv, m_dst + wave * (32 * kBlockN));
     };
     // The same copies one instruction at a time (c = 0 .. kCopies-1: K, then V, then the mask), for issuing
     // them between the score MFMAs of the block before. Whole tiles only: a ragged last tile is copied by load_kv.
     constexpr int kNI = KvTileLoader<T, D, false, NW>::NI;
-    constexpr int kCopies = 2 * kNI + (MASK_LDS ? 4 : 0);
-    auto load_one = [&](int c, int step, T* k_dst, T* v_dst, T* m_dst) __attribute__((always_inline)) {
+    constexpr int kCopies = (WIDE ? 4 : 2) * kNI + (MASK_LDS ? 4 : 0);
+    auto load_one = [&](int c, int step, T* k_dst, T* v_dst, T* m_dst, T* kb_dst, T* vb_dst) __attribute__((always_inline)) {
       if (c < kNI) k_loader.issue_one_whole(c, k_g, step * kBlockN, k_dst);
       else if (c < 2 * kNI) v_loader.issue_one_whole(c - kNI, v_g, step * kBlockN, v_dst);
-      else if constexpr (MASK_LDS) m_loader.issue_one(c - 2 * kNI, mask_wg, step * kBlockN, Skv, m_dst + wave * (32 * kBlockN));
+      else if constexpr (WIDE) {
+        if (c < 3 * kNI) kb_loader.issue_one_whole(c - 2 * kNI, k_g + D, step * kBlockN, kb_dst);
+        else vb_loader.issue_one_whole(c - 3 * kNI, v_g + D, step * kBlockN, vb_dst);
+      } else if constexpr (MASK_LDS) m_loader.issue_one(c - 2 * kNI, mask_wg, step * kBlockN, Skv, m_dst + wave * (32 * kBlockN));
     };
 
     // Online softmax of one 64-key block (two 32-key score tiles): mask, row max, (rare) rescale; the exponentials
@@ -235,7 +270,10 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+          for (int r = 0; r < 16; ++r) {
+            o_acc[dt][r] *= alpha;
+            if constexpr (WIDE) o_accb[dt][r] *= alpha;
+          }
         // a row with every key masked so far keeps m_i = -inf and neg_m = 0: its scores are all -inf and give
         // exp2(-inf) = 0, not exp2(-inf + inf)
         neg_m = m_i == -INFINITY ? 0.0f : -m_i;
@@ -283,6 +321,12 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o_acc[dt] = MfmaT<T>::run(vf.f[hf][dt], pf[hf], o_acc[dt]);
     };
+    auto pv_tile_b = [&](const VFrags& vf, const Frag* pf) __attribute__((always_inline)) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int dt = 0; dt < (WIDE ? DT : 1); ++dt) o_accb[dt] = MfmaT<T>::run(vf.f[hf][dt], pf[hf], o_accb[dt]);
+    };
 
     // mask row of this lane's query (GENERAL with a mask only)
     const T* mask_row = nullptr;
@@ -295,12 +339,12 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
     // CU's vector memory pipe busy for about 500 cycles, during which every wave sits in its copy instructions
     // and the matrix cores have nothing queued.
     auto process = [&](int step, const T* k_src, const T* v_src, const T* m_src, int next, T* k_dst, T* v_dst,
-                       T* m_dst) __attribute__((always_inline)) {
+                       T* m_dst, const T* kb_src, const T* vb_src, T* kb_dst, T* vb_dst) __attribute__((always_inline)) {
       const int n0 = step * kBlockN;
       // causal: a key block wholly past this wave's 32 rows contributes nothing (wave-uniform; the workgroup's
       // barriers are outside)
       const bool spread = next >= 0 && (next + 1) * kBlockN <= Skv && !(CAUSAL && n0 > q0 + 31);
-      if (next >= 0 && !spread) load_kv(next, k_dst, v_dst, m_dst);
+      if (next >= 0 && !spread) load_kv(next, k_dst, v_dst, m_dst, kb_dst, vb_dst);
       if (CAUSAL && n0 > q0 + 31) return;
       // mask values of this lane's 32 scores: four runs of four consecutive keys per 32-key tile
       typedef T MaskRun __attribute__((ext_vector_type(4)));
@@ -350,9 +394,31 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
           if (spread) {
 #pragma unroll
             for (int c = 0; c < kCopies; ++c)
-              if (c * DS / kCopies == ds) load_one(c, next, k_dst, v_dst, m_dst);
+              if (c * DS / kCopies == ds) load_one(c, next, k_dst, v_dst, m_dst, kb_dst, vb_dst);
           }
           __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (WIDE) {                           // the second halves of Q and K add to the same scores
+          auto read_kb = [&](int jt, int ds) __attribute__((always_inline)) {
+            const int row = jt * 32 + krow;
+            const int c = (ds * 2 + half) ^ swz_ktile<D>(row);
+            return *reinterpret_cast<const Frag*>(kb_src + (row * CPR + c) * 8);
+          };
+#pragma unroll
+          for (int ds = 0; ds < kAhead && ds < DS; ++ds) {
+            kf[0][ds] = read_kb(0, ds);
+            kf[1][ds] = read_kb(1, ds);
+          }
+#pragma unroll
+          for (int ds = 0; ds < DS; ++ds) {
+            if (ds + kAhead < DS) {
+              kf[0][ds + kAhead] = read_kb(0, ds + kAhead);
+              kf[1][ds + kAhead] = read_kb(1, ds + kAhead);
+            }
+            s[0] = MfmaT<T>::run(kf[0][ds], qfb[ds], s[0]);
+            s[1] = MfmaT<T>::run(kf[1][ds], qfb[ds], s[1]);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       }
       VFrags vf0, vf1;
@@ -389,22 +455,29 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
       pv_tile(vf0, &pf[0]);
       exp_tile(s[1], &pf[2]);
       pv_tile(vf1, &pf[2]);
+      if constexpr (WIDE) {                             // the same probabilities on the second half of V
+        read_v(vb_src, 0, vf0);
+        read_v(vb_src, 1, vf1);
+        pv_tile_b(vf0, &pf[0]);
+        pv_tile_b(vf1, &pf[2]);
+      }
     };
 
-    load_kv(0, k_lds0, v_lds0, m_lds0);
+    load_kv(0, k_lds0, v_lds0, m_lds0, kb_lds0, vb_lds0);
     int step = 0;
     for (; step + 1 < n_steps; step += 2) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      process(step, k_lds0, v_lds0, m_lds0, step + 1, k_lds1, v_lds1, m_lds1);
+      process(step, k_lds0, v_lds0, m_lds0, step + 1, k_lds1, v_lds1, m_lds1, kb_lds0, vb_lds0, kb_lds1, vb_lds1);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      process(step + 1, k_lds1, v_lds1, m_lds1, step + 2 < n_steps ? step + 2 : -1, k_lds0, v_lds0, m_lds0);
+      process(step + 1, k_lds1, v_lds1, m_lds1, step + 2 < n_steps ? step + 2 : -1, k_lds0, v_lds0, m_lds0, kb_lds1,
+              vb_lds1, kb_lds0, vb_lds0);
     }
     if (step < n_steps) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      process(step, k_lds0, v_lds0, m_lds0, -1, k_lds1, v_lds1, m_lds1);
+      process(step, k_lds0, v_lds0, m_lds0, -1, k_lds1, v_lds1, m_lds1, kb_lds0, vb_lds0, kb_lds1, vb_lds1);
     }
 
     // ---- epilogue: o_acc[dt][r] is O[qrow][dt*32 + 8*(r/4) + 4*half + r%4] * l
@@ -420,6 +493,11 @@ void flash_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K, const T*
           if (!PADDED || d < dh)
             store4o<OutT>(o_row + d, o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l,
                           o_acc[dt][q4 * 4 + 2] * inv_l, o_acc[dt][q4 * 4 + 3] * inv_l);
+          if constexpr (WIDE) {
+            if (D + d < dh)
+              store4o<OutT>(o_row + D + d, o_accb[dt][q4 * 4 + 0] * inv_l, o_accb[dt][q4 * 4 + 1] * inv_l,
+                            o_accb[dt][q4 * 4 + 2] * inv_l, o_accb[dt][q4 * 4 + 3] * inv_l);
+          }
         }
     }
     __syncthreads();                                            // the next unit's copies reuse both stages
@@ -576,6 +654,24 @@ int launch_mfma_padded(const void* Q, const void* K, const void* V, void* O, int
   return launch_status();
 }
 
+// A head of 128 < head_dim <= 256 columns (a multiple of 8) as two halves on the kernel for 128: one 128-row
+// workgroup per CU.
+template <typename T, typename OutT, bool CAUSAL>
+int launch_mfma_wide(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, int head_dim,
+                     float scale_log2e, hipStream_t st) {
+  const int64_t nqb = (S + 127) / 128;
+  const int64_t units = nqb * ZH;
+  if (units > 0x7fffffff) return HEXMI_ENOTSUP;
+  const int64_t blocks = resident_grid(units, 1);
+  if (blocks <= 0) return HEXMI_ELAUNCH;
+  const int groups = CAUSAL ? plan_causal_groups(ZH, nqb, blocks) : 0;
+  hipLaunchKernelGGL((flash_fwd_kernel<T, OutT, 128, CAUSAL, false, 4, false, true, true>), dim3((unsigned)blocks), dim3(256), 0,
+                     st, static_cast<const T*>(Q), static_cast<const T*>(K), static_cast<const T*>(V),
+                     static_cast<OutT*>(O), (int)ZH, (int)S, scale_log2e, static_cast<const T*>(nullptr), 0, 0.0f,
+                     groups, head_dim);
+  return launch_status();
+}
+
 template <typename T, typename OutT, int D>
 int launch_mfma(const void* Q, const void* K, const void* V, void* O, int64_t ZH, int64_t S, float scale_log2e,
                 bool causal, hipStream_t st) {
@@ -678,6 +774,11 @@ int dispatch_half(const void* Q, const void* K, const void* V, const void* mask,
     }
     if (causal) return launch_mfma_padded<T, OutT, 128, true>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
     return launch_mfma_padded<T, OutT, 128, false>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
+  }
+  // ... and up to 256 as two halves of 128
+  if (ok && plain && D % 8 == 0 && D > 128 && D <= 256) {
+    if (causal) return launch_mfma_wide<T, OutT, true>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
+    return launch_mfma_wide<T, OutT, false>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
   }
   const bool general_ok = ok && !causal && Skv % 4 == 0 && Skv >= 4 && (!mask || aligned_to(mask, 8));
   if (general_ok && D == 128) return launch_mfma_general<T, OutT, 128>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);

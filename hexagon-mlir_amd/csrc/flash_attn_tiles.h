@@ -74,12 +74,14 @@ struct KvTileLoader {
   int lds_off0;
   int d;                                                  // elements between rows in memory (D unless PADDED)
   bool live;                                              // this lane's chunk is inside the head
-  __device__ __forceinline__ void init(int wave, int lane, int head_dim = D) {
+  // live_cols: columns of the tile that exist in memory (the head itself, or what is left of it for a tile that
+  // starts at a column offset: the caller then passes the offset pointer)
+  __device__ __forceinline__ void init(int wave, int lane, int head_dim = D, int live_cols = D) {
     const int lin = wave * 64 + lane;
     row0 = lin / CPR;
     col0 = ((lin % CPR) ^ (IS_V ? swz_vtile<D>(row0) : swz_ktile<D>(row0))) * 8;
     d = PADDED ? head_dim : D;
-    live = !PADDED || col0 < d;
+    live = !PADDED || col0 < live_cols;
     off0 = row0 * d + col0;
     lds_off0 = wave * 64 * 8;
   }

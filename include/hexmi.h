@@ -306,9 +306,9 @@ int hexmi_gemm_w8a16_packed(int64_t M, int64_t N, int64_t K, const void *A,
  * test/python/triton/test_flash_attention.py:37-168 (STAGE=1 is causal == 0)
  * and tm_tensor.attention (include/hexagon/Dialect/TmTensor/IR/TmTensorOps.td:28-56).
  * in_dtype: HEXMI_F16 / HEXMI_BF16 (MFMA path) or HEXMI_F32.
- * D: 64 and 128 are the kernels' own sizes; 16-bit heads below 128 in
- * multiples of 8 run them on zero-padded tiles; anything else a slow
- * row-wise kernel (D <= 256).
+ * D: 64 and 128 are the kernels' own sizes; other 16-bit heads up to 256 in
+ * multiples of 8 run them on zero-padded tiles (above 128 as two halves);
+ * anything else a slow row-wise kernel (D <= 256).
  * out_dtype: in_dtype, or HEXMI_F32 with fp16 inputs (the fp16 QKV -> fp32 O
  * form of test/python/mlir/hexkl_attention/input.mlir:1-169). */
 int hexmi_flash_attn_fwd(const void *Q, const void *K, const void *V, void *O,

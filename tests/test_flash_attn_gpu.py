@@ -74,6 +74,27 @@ def test_attention_other_head_sizes(hexmi, oracle, case, dtype, causal):
     assert (got32 - want).abs().max() <= (5e-3 if dtype == torch.float16 else 3e-2)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", [(1, 2, 300, 256), (2, 1, 129, 192), (1, 3, 64, 136), (1, 8, 200, 160), (1, 1, 1000, 200),
+                                  (1, 1, 1, 256), (2, 8, 515, 144)])
+def test_attention_head_sizes_up_to_256(hexmi, oracle, case, dtype, causal):
+    # head sizes above 128 run the kernel for 128 on two halves of the head: the scores sum over both halves' K
+    # tiles, the second half is padded like a narrow head
+    Z, H, S, D = case
+    q, k, v = _qkv(Z, H, S, D, dtype, seed=D + S)
+    scale = 1.0 / math.sqrt(D)
+    buf = torch.full((Z * H * S + 1, D), float("nan"), dtype=dtype, device="cuda")
+    out = buf[:Z * H * S].view(Z, H, S, D)
+    hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal, out=out)
+    want = _oracle(oracle, q, k, v, scale, causal)
+    tol = 2e-2 if dtype == torch.float16 else 4e-2
+    assert (out.cpu().float() - want).abs().max() <= tol
+    assert torch.isnan(buf[-1]).all()
+    got32 = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal, out_dtype=torch.float32).cpu()
+    assert (got32 - want).abs().max() <= (5e-3 if dtype == torch.float16 else 3e-2)
+
+
 def test_attention_padded_head_equals_the_zero_padded_problem(hexmi):
     # head size 80 on the kernel for 128 is the 128-wide problem with 48 zero columns in Q, K and V (and 1/sqrt(80)):
     # the same kernel, the same arithmetic -- bit for bit
@@ -86,6 +107,15 @@ def test_attention_padded_head_equals_the_zero_padded_problem(hexmi):
         want = hexmi.flash_attention(qp.cuda(), kp.cuda(), vp.cuda(), scale, causal).cpu()
         assert torch.equal(got, want[..., :D])
         assert (want[..., D:] == 0).all()
+    # and head size 192 is the 256-wide problem with 64 zero columns (both on the two-halves form)
+    q, k, v = _qkv(1, 8, 400, 192, torch.float16, seed=32)
+    scale = 1.0 / math.sqrt(192)
+    for causal in (False, True):
+        got = hexmi.flash_attention(q.cuda(), k.cuda(), v.cuda(), scale, causal).cpu()
+        qp, kp, vp = (torch.nn.functional.pad(t, (0, 64)) for t in (q, k, v))
+        want = hexmi.flash_attention(qp.cuda(), kp.cuda(), vp.cuda(), scale, causal).cpu()
+        assert torch.equal(got, want[..., :192])
+        assert (want[..., 192:] == 0).all()
 
 
 @pytest.mark.parametrize("causal", [False, True])
