@@ -12,6 +12,9 @@
 // Causal: key blocks past the diagonal are skipped, the diagonal blocks are masked element-wise, and workgroups
 // are numbered so the longest (last) query blocks start first.
 //
+// Other 16-bit head sizes in multiples of 8: below 128 on tiles padded with zero columns (PADDED), above 128 up to
+// 256 as two 128-wide halves of the head (WIDE).
+//
 // fp32 inputs with head size 64 or 128 run the fp32 matrix-core kernels of flash_attn_f32.hip; other head sizes and
 // unaligned operands take the plain one-wave-per-query-row kernel below.
 #include <algorithm>
