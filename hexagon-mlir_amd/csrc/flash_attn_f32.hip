@@ -27,11 +27,15 @@ __device__ __forceinline__ float other_half_f32(float v) {
   return __builtin_bit_cast(float, (threadIdx.x & 32) ? lo : hi);
 }
 
-template <int D, int BN, bool CAUSAL, bool MASKED>
+// PADDED: the head is head_dim < D wide (a multiple of 4): rows are head_dim floats apart in memory and the tiles
+// carry zero columns from head_dim to D -- a copy lane whose chunk lies there issues nothing, its LDS positions (which
+// no other lane writes) are zeroed once; the Q chunks there are zero registers, the output columns are not stored.
+template <int D, int BN, bool CAUSAL, bool MASKED, bool PADDED = false>
 __global__ __launch_bounds__(256, D == 64 ? 2 : 1)
 void flash_fwd_f32_kernel(const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
                           float* __restrict__ O, int ZH, int S, int Skv, float scale_log2e,
-                          const float* __restrict__ Mk, float mask_factor) {
+                          const float* __restrict__ Mk, float mask_factor, int head_dim = D) {
+  const int dh = PADDED ? head_dim : D;             // floats between rows in memory
   constexpr int NT = BN / 32;                       // 32-key score tiles per key block
   constexpr int CPR = D / 4;                        // 16-byte chunks per row
   constexpr int DT = D / 32;                        // 32-wide output tiles over the head dimension
@@ -47,9 +51,9 @@ void flash_fwd_f32_kernel(const float* __restrict__ Q, const float* __restrict__
   const int nqb = (S + 127) / 128;
   const int zh = blockIdx.x % ZH;
   const int qb = nqb - 1 - blockIdx.x / ZH;         // longest (last) query blocks first
-  const float* q_g = Q + (int64_t)zh * S * D;
-  const float* k_g = K + (int64_t)zh * Skv * D;
-  const float* v_g = V + (int64_t)zh * Skv * D;
+  const float* q_g = Q + (int64_t)zh * S * dh;
+  const float* k_g = K + (int64_t)zh * Skv * dh;
+  const float* v_g = V + (int64_t)zh * Skv * dh;
   const int q0 = qb * 128 + wave * 32;
   const int r32 = lane % 32, kh = lane / 32;
   const int qrow = q0 + r32;
@@ -58,8 +62,10 @@ void flash_fwd_f32_kernel(const float* __restrict__ Q, const float* __restrict__
   // Q: chunk 2*dq + kh of the row: head dimensions 8*dq + 4*kh + e, the k slots of MFMA (dq, e)
   f32x4a qf[DQ];
 #pragma unroll
-  for (int dq = 0; dq < DQ; ++dq)
-    qf[dq] = *reinterpret_cast<const f32x4a*>(q_g + (int64_t)qr * D + (2 * dq + kh) * 4);
+  for (int dq = 0; dq < DQ; ++dq) {
+    if (!PADDED || (2 * dq + kh) * 4 < dh) qf[dq] = *reinterpret_cast<const f32x4a*>(q_g + (int64_t)qr * dh + (2 * dq + kh) * 4);
+    else qf[dq] = f32x4a{0.0f, 0.0f, 0.0f, 0.0f};
+  }
 
   f32x16 o_acc[DT];
 #pragma unroll
@@ -81,6 +87,21 @@ void flash_fwd_f32_kernel(const float* __restrict__ Q, const float* __restrict__
     kcol[j] = (pc ^ (row_c[j] & 15)) * 4;
     vcol[j] = (pc ^ (((row_c[j] >> 2) & 1) << 3)) * 4;
   }
+  if constexpr (PADDED) {
+    // the zero columns of both stages, once (the first barrier of the key loop lies before the first fragment read)
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const f32x4a z = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (kcol[j] >= dh) {
+        *reinterpret_cast<f32x4a*>(k_s0 + (j * 4 + wave) * 256 + lane * 4) = z;
+        *reinterpret_cast<f32x4a*>(k_s1 + (j * 4 + wave) * 256 + lane * 4) = z;
+      }
+      if (vcol[j] >= dh) {
+        *reinterpret_cast<f32x4a*>(v_s0 + (j * 4 + wave) * 256 + lane * 4) = z;
+        *reinterpret_cast<f32x4a*>(v_s1 + (j * 4 + wave) * 256 + lane * 4) = z;
+      }
+    }
+  }
   auto load_kv = [&](int step, float* k_dst, float* v_dst) __attribute__((always_inline)) {
     const char* kb = reinterpret_cast<const char*>(k_g);
     const char* vb = reinterpret_cast<const char*>(v_g);
@@ -88,8 +109,8 @@ void flash_fwd_f32_kernel(const float* __restrict__ Q, const float* __restrict__
     for (int j = 0; j < NI; ++j) {
       int key = step * BN + row_c[j];
       key = key < Skv ? key : Skv - 1;                // rows past the end repeat the last key (masked below)
-      copy_to_lds(kb, (key * D + kcol[j]) * (int)sizeof(float), k_dst + (j * 4 + wave) * 256);
-      copy_to_lds(vb, (key * D + vcol[j]) * (int)sizeof(float), v_dst + (j * 4 + wave) * 256);
+      if (!PADDED || kcol[j] < dh) copy_to_lds(kb, (key * dh + kcol[j]) * (int)sizeof(float), k_dst + (j * 4 + wave) * 256);
+      if (!PADDED || vcol[j] < dh) copy_to_lds(vb, (key * dh + vcol[j]) * (int)sizeof(float), v_dst + (j * 4 + wave) * 256);
     }
   };
 
@@ -219,14 +240,15 @@ void flash_fwd_f32_kernel(const float* __restrict__ Q, const float* __restrict__
   const float l_tot = l_i + other_half_f32(l_i);
   const float inv_l = 1.0f / l_tot;
   if (qrow < S) {
-    float* o_row = O + ((int64_t)zh * S + qrow) * D;
+    float* o_row = O + ((int64_t)zh * S + qrow) * dh;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4)
-        *reinterpret_cast<f32x4a*>(o_row + dt * 32 + 8 * q4 + 4 * kh) =
-            f32x4a{o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l, o_acc[dt][q4 * 4 + 2] * inv_l,
-                   o_acc[dt][q4 * 4 + 3] * inv_l};
+        if (!PADDED || dt * 32 + 8 * q4 + 4 * kh < dh)
+          *reinterpret_cast<f32x4a*>(o_row + dt * 32 + 8 * q4 + 4 * kh) =
+              f32x4a{o_acc[dt][q4 * 4 + 0] * inv_l, o_acc[dt][q4 * 4 + 1] * inv_l, o_acc[dt][q4 * 4 + 2] * inv_l,
+                     o_acc[dt][q4 * 4 + 3] * inv_l};
   }
 }
 
@@ -417,28 +439,35 @@ void flash_fwd_f32_split_kernel(const float* __restrict__ Q, const float* __rest
 
 template <int D, int BN>
 int launch(const float* Q, const float* K, const float* V, const float* mask, float* O, int64_t ZH, int64_t S,
-           int64_t Skv, float scale_log2e, bool causal, hipStream_t st) {
+           int64_t Skv, float scale_log2e, bool causal, hipStream_t st, int head_dim = D) {
   const int64_t blocks = (S + 127) / 128 * ZH;
   if (blocks > 0x7fffffff) return HEXMI_ENOTSUP;
   const float mask_factor = mask ? 1.44269504088896340736f / scale_log2e : 0.0f;      // mask / sm_scale
-#define HEXMI_FA32(CZ, MK) \
-  hipLaunchKernelGGL((flash_fwd_f32_kernel<D, BN, CZ, MK>), dim3((unsigned)blocks), dim3(256), 0, st, Q, K, V, O, \
-                     (int)ZH, (int)S, (int)Skv, scale_log2e, mask, mask_factor)
-  if (mask) HEXMI_FA32(false, true);
-  else if (causal) HEXMI_FA32(true, false);
-  else HEXMI_FA32(false, false);
+#define HEXMI_FA32(CZ, MK, PD) \
+  hipLaunchKernelGGL((flash_fwd_f32_kernel<D, BN, CZ, MK, PD>), dim3((unsigned)blocks), dim3(256), 0, st, Q, K, V, O, \
+                     (int)ZH, (int)S, (int)Skv, scale_log2e, mask, mask_factor, head_dim)
+  if (head_dim < D) {
+    if (mask) HEXMI_FA32(false, true, true);
+    else if (causal) HEXMI_FA32(true, false, true);
+    else HEXMI_FA32(false, false, true);
+  } else {
+    if (mask) HEXMI_FA32(false, true, false);
+    else if (causal) HEXMI_FA32(true, false, false);
+    else HEXMI_FA32(false, false, false);
+  }
 #undef HEXMI_FA32
   return launch_status();
 }
 
 }  // namespace
 
-// True (and the kernel launched, status in *status) for head sizes 64 and 128 with 16-byte aligned operands; a mask
+// True (and the kernel launched, status in *status) for head sizes up to 128 in multiples of 4 (64 and 128 are the
+// kernels' own; narrower heads run them on padded tiles) with 16-byte aligned operands; a mask
 // needs whole 16-byte runs (Skv % 4 == 0) and excludes causal.
 bool flash_attn_f32_mfma(const float* Q, const float* K, const float* V, const float* mask, float* O, int64_t ZH,
                          int64_t S, int64_t Skv, int64_t D, float scale_log2e, bool causal, hipStream_t st,
                          int* status) {
-  if (D != 64 && D != 128) return false;
+  if (D < 4 || D > 128 || D % 4 != 0) return false;     // 64 and 128, or a narrower head on padded tiles
   // the row maximum is taken on the raw scores and scaled afterwards: right for a positive scale only
   if (!(scale_log2e > 0.0f)) return false;
   if (!aligned_to(Q, 16) || !aligned_to(K, 16) || !aligned_to(V, 16) || !aligned_to(O, 16)) return false;
@@ -447,7 +476,8 @@ bool flash_attn_f32_mfma(const float* Q, const float* K, const float* V, const f
   if (mask && (Skv % 4 != 0 || Skv < 4 || !aligned_to(mask, 16))) return false;
   const int cus = hexmi_num_cus();
   const int64_t row_split_groups = (S + 127) / 128 * ZH;
-  if (!mask && Skv == S && row_split_groups * 2 < (cus > 0 ? cus : 256) && (S + 31) / 32 * ZH <= 0x7fffffff) {
+  if ((D == 64 || D == 128) && !mask && Skv == S && row_split_groups * 2 < (cus > 0 ? cus : 256) &&
+      (S + 31) / 32 * ZH <= 0x7fffffff) {
     // too few 128-row workgroups for the chip: 32-row workgroups whose waves split the keys
     const unsigned blocks = (unsigned)((S + 31) / 32 * ZH);
 #define HEXMI_FA32S(DD, NWW, CZ) \
@@ -459,8 +489,8 @@ bool flash_attn_f32_mfma(const float* Q, const float* K, const float* V, const f
     *status = launch_status();
     return true;
   }
-  *status = D == 64 ? launch<64, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, causal, st)
-                    : launch<128, 32>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, causal, st);
+  *status = D <= 64 ? launch<64, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, causal, st, (int)D)
+                    : launch<128, 32>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, causal, st, (int)D);
   return true;
 }
 

@@ -122,7 +122,9 @@ def test_attention_padded_head_equals_the_zero_padded_problem(hexmi):
 @pytest.mark.parametrize("case", [(1, 1, 1024, 64), (1, 2, 100, 128), (2, 2, 65, 32), (1, 1, 130, 80),
                                   # head sizes 64 and 128 run on the fp32 matrix cores: ragged query and key blocks,
                                   # several workgroups per head, a single row
-                                  (2, 3, 333, 64), (1, 2, 515, 128), (1, 1, 1, 64), (3, 1, 129, 128)])
+                                  (2, 3, 333, 64), (1, 2, 515, 128), (1, 1, 1, 64), (3, 1, 129, 128),
+                                  # narrower heads in multiples of 4: the same kernels on padded tiles
+                                  (1, 2, 300, 4), (2, 1, 257, 36), (1, 3, 200, 100), (1, 1, 640, 124), (2, 2, 129, 72)])
 def test_attention_parity_fp32(hexmi, oracle, case, causal):
     # (1,1,1024,64) rand inputs, scale 0.5, non-causal is test_flash_attention.py:20-34,171-213
     Z, H, S, D = case
@@ -315,7 +317,9 @@ def test_masked_attention_parity_half(hexmi, oracle, case, dtype, with_mask):
 
 @pytest.mark.parametrize("case", [(2, 50, 70, 32), (1, 64, 64, 128), (1, 33, 129, 64),
                                   # Skv % 4 == 0 with head size 64 / 128: the fp32 matrix-core kernel with a mask
-                                  (2, 200, 72, 64), (1, 130, 516, 128), (3, 129, 1028, 64)])
+                                  (2, 200, 72, 64), (1, 130, 516, 128), (3, 129, 1028, 64),
+                                  # ... and narrower heads on padded tiles
+                                  (2, 200, 72, 80), (1, 130, 516, 36), (2, 129, 132, 100)])
 def test_masked_attention_parity_fp32(hexmi, oracle, case):
     B, Sq, Skv, D = case
     g = _gen(23)
