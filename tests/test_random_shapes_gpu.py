@@ -191,8 +191,11 @@ def case_w8():
 
 def case_flash():
     dt = pick(torch.float16, torch.float16, torch.bfloat16, torch.float32)
-    D = pick(64, 128, 128) if dt != torch.float32 else pick(64, 128)
+    # the kernels' own head sizes, narrower and wider ones on padded tiles, and one for the row-wise kernel
+    D = pick(64, 128, 128, 8, 40, 80, 96, 160, 192, 256, 20) if dt != torch.float32 else pick(64, 128, 4, 36, 80, 100, 10)
     Z, H = pick(1, 2, 3), pick(1, 2, 3, 5, 8, 9)
+    if D > 128 or D in (10, 20):
+        H = min(H, 3)
     S = dim(1, 2600 if BIG else 900, (1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 383, 384, 512, 640, 1024, 1100))
     causal = rnd.random() < 0.6
     what = "flash %s Z=%d H=%d S=%d D=%d causal=%s" % (dt, Z, H, S, D, causal)
@@ -208,7 +211,7 @@ def case_flash():
 
 def case_attention():
     dt = pick(torch.float16, torch.bfloat16, torch.float32)
-    D = pick(64, 128) if dt != torch.float32 else pick(64, 128)
+    D = pick(64, 128, 32, 80, 112) if dt != torch.float32 else pick(64, 128, 36, 80)
     B = pick(1, 2, 5, 9)
     Sq = dim(1, 2000 if BIG else 600, (1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257))
     Skv = dim(1, 2000 if BIG else 600, (1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257))
