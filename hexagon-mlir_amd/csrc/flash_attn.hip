@@ -61,7 +61,7 @@ struct MaskTileLoader {
 
 // GENERAL: the number of keys (Skv) may differ from the number of queries (S) and an additive mask
 // [ZH, S, Skv] (same dtype as Q; may be null) is added to the scaled scores before the softmax, as
-// tm_tensor.attention does (qcom_hexagon_backend/lib/Transforms/LowerTmTensor.cpp:157-160); Skv % 4 == 0.
+// tm_tensor.attention does (qcom_hexagon_backend/lib/Transforms/LowerTmTensor.cpp:157-160); with a mask Skv % 4 == 0.
 // NW waves per workgroup (4 or 8), 32 query rows each: every K / V tile copied into LDS serves NW*32 query rows.
 // Eight waves halve the L2 -> LDS copy traffic (each query block streams the whole K and V of its head), worth
 // 1-9 % from 2048 keys on; short sequences and small grids prefer the larger number of 128-row workgroups. (Measured on random
@@ -783,7 +783,8 @@ int dispatch_half(const void* Q, const void* K, const void* V, const void* mask,
     if (causal) return launch_mfma_wide<T, OutT, true>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
     return launch_mfma_wide<T, OutT, false>(Q, K, V, O, ZH, S, (int)D, scale_log2e, st);
   }
-  const bool general_ok = ok && !causal && Skv % 4 == 0 && Skv >= 4 && (!mask || aligned_to(mask, 8));
+  // (a mask is read in runs of four keys; without one any key count goes: cross-attention over 77 keys, say)
+  const bool general_ok = ok && !causal && (!mask || (Skv % 4 == 0 && Skv >= 4 && aligned_to(mask, 8)));
   if (general_ok && D == 128) return launch_mfma_general<T, OutT, 128>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
   if (general_ok && D == 64) return launch_mfma_general<T, OutT, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st);
   if (general_ok && D % 8 == 0 && D < 64) return launch_mfma_general<T, OutT, 64>(Q, K, V, mask, O, ZH, S, Skv, scale_log2e, st, (int)D);

@@ -293,7 +293,9 @@ MASKED_CASES = [(2, 128, 128, 128), (3, 200, 72, 64), (1, 1, 64, 128), (2, 77, 5
                 # (ragged last row block, ragged last key block, several row blocks, many batch entries)
                 (3, 300, 520, 128), (2, 513, 72, 64), (1, 257, 2048 + 8, 128), (40, 129, 136, 64),
                 # head sizes below 128 in multiples of 8: the 128-row kernel on tiles padded with zero columns
-                (2, 200, 72, 80), (1, 300, 520, 96), (3, 129, 136, 32), (1, 77, 516, 40), (2, 64, 64, 112)]
+                (2, 200, 72, 80), (1, 300, 520, 96), (3, 129, 136, 32), (1, 77, 516, 40), (2, 64, 64, 112),
+                # key counts that are not multiples of 4 (matrix-core kernel without a mask, row-wise with one)
+                (4, 1024, 77, 64), (2, 300, 1, 128), (1, 129, 515, 80)]
 
 
 @pytest.mark.parametrize("with_mask", [True, False])
