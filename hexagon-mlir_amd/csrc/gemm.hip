@@ -1227,6 +1227,84 @@ void gemm_kernel_any(const T* __restrict__ A, const void* __restrict__ Bv, OutT*
                                                B_I8 ? scales : nullptr, per_tensor);
 }
 
+// Up to eight activation rows against weights given as [N,K] (x @ W^T, a decode step): the product is a stream of
+// the weights at the HBM rate, and tiles of 128 columns would leave most CUs without work (N = K = 4096: 32 tiles,
+// 24 us where the 32 MB of weights take 6). One wave per output channel, eight per workgroup: the wave reads its
+// weight row 16 bytes per lane (non-temporal, four chunks in flight), the activation rows come from LDS where the
+// workgroup staged 2048 columns of them, products accumulate in fp32 (v_dot2) and a butterfly sums the lanes.
+// K % 8 == 0, rows on 16-byte boundaries.
+template <typename T> struct Dot8;
+template <> struct Dot8<f16> {
+  static __device__ __forceinline__ float run(const u32x4& w, const u32x4& a, float acc) {
+    const f16x8 wf = __builtin_bit_cast(f16x8, w), af = __builtin_bit_cast(f16x8, a);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      acc = __builtin_amdgcn_fdot2(f16x2{wf[2 * e], wf[2 * e + 1]}, f16x2{af[2 * e], af[2 * e + 1]}, acc, false);
+    return acc;
+  }
+};
+template <> struct Dot8<bf16> {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ float run(const u32x4& w, const u32x4& a, float acc) {
+    const bf16x8 wf = __builtin_bit_cast(bf16x8, w), af = __builtin_bit_cast(bf16x8, a);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2_t{wf[2 * e], wf[2 * e + 1]}, bf16x2_t{af[2 * e], af[2 * e + 1]}, acc, false);
+    return acc;
+  }
+};
+
+constexpr int kGemvWaves = 8, kGemvBlockK = 2048;
+
+template <typename T, typename OutT, int MR>
+__global__ __launch_bounds__(kGemvWaves * 64)
+void gemv_nt_kernel(const T* __restrict__ A, const T* __restrict__ W, OutT* C, int M, int N, int K, int64_t lda,
+                    int64_t ldb, int64_t ldc, const OutT* __restrict__ bias, const OutT* resid, int64_t ldr) {
+  constexpr int KB = kGemvBlockK, CPB = KB / kChunk;  // chunks per row of a staged block
+  __shared__ __attribute__((aligned(16))) T a_s[MR][KB];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n = blockIdx.x * kGemvWaves + wave;
+  const T* wrow = W + (int64_t)(n < N ? n : N - 1) * ldb;   // past the end: the last channel again, not stored
+  float acc[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+  for (int kb = 0; kb < K; kb += KB) {
+    const int kn = K - kb < KB ? K - kb : KB;           // columns of this block, a multiple of 8
+    // the weight chunks of this block first: they come from HBM, the activations below from L2
+    u32x4 wv[CPB / kWave];
+#pragma unroll
+    for (int j = 0; j < CPB / kWave; ++j) {
+      const int k = (j * kWave + lane) * kChunk;
+      wv[j] = k < kn ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + kb + k)) : u32x4{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();                                    // every wave has read the block before
+    for (int c = threadIdx.x; c < MR * CPB; c += kGemvWaves * 64) {
+      const int m = c / CPB, k = (c % CPB) * kChunk;
+      if (k < kn)
+        *reinterpret_cast<u32x4*>(&a_s[m][k]) =
+            *reinterpret_cast<const u32x4*>(A + (int64_t)(m < M ? m : M - 1) * lda + kb + k);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < CPB / kWave; ++j) {
+      const int k = (j * kWave + lane) * kChunk;
+      if (k < kn) {
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[m] = Dot8<T>::run(wv[j], *reinterpret_cast<const u32x4*>(&a_s[m][k]), acc[m]);
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    float sum = wave_sum(acc[m]);
+    if (lane == 0 && n < N && m < M) {
+      if (bias) sum += to_f32<OutT>(bias[n]);
+      if (resid) sum += to_f32<OutT>(resid[(int64_t)m * ldr + n]);
+      C[(int64_t)m * ldc + n] = from_f32<OutT>(sum);
+    }
+  }
+}
+
 // fp32 inputs (the reference's torch-mlir graphs multiply fp32 matrices, e.g.
 // test/python/torch-mlir/test_add_matmul_softmax.py:25-29) whose shape or alignment the matrix-core kernel of
 // gemm_f32.hip does not take: 64x64 tile, K in steps of 16 through LDS, every thread a 4x4 block of fp32 FMAs.
@@ -1397,6 +1475,17 @@ int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N
   // chunks: K % 32 == 0, leading dimensions and N multiples of 8 elements, 16-byte aligned bases. Their epilogue
   // reads bias and residual in runs of four columns.
   const size_t run = 4 * sizeof(OutT);
+  // a few rows against [N,K] weights: the weight stream (see gemv_nt_kernel)
+  if (TRANS_B && M <= 8 && N >= 64 && K % kChunk == 0 && lda % 8 == 0 && ldb % 8 == 0 && aligned_to(A, 16) &&
+      aligned_to(B, 16)) {
+    const dim3 grid((unsigned)((N + kGemvWaves - 1) / kGemvWaves));
+#define HEXMI_GEMV(MR) \
+  hipLaunchKernelGGL((gemv_nt_kernel<T, OutT, MR>), grid, dim3(kGemvWaves * 64), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, \
+                     ldc, bias, resid, ldr)
+    if (M == 1) HEXMI_GEMV(1); else if (M == 2) HEXMI_GEMV(2); else if (M <= 4) HEXMI_GEMV(4); else HEXMI_GEMV(8);
+#undef HEXMI_GEMV
+    return launch_status();
+  }
   const bool fast = K % BK == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && N % 8 == 0 && N >= 8 &&
                     aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(C, 16) && (!bias || aligned_to(bias, run)) &&
                     (!resid || (aligned_to(resid, run) && ldr % 4 == 0));

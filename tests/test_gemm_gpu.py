@@ -71,6 +71,27 @@ def test_gemm_parity(hexmi, oracle, shape, dtype, trans_b):
     assert ((got.float() - want.float()).abs().max() / math.sqrt(K)) <= 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("N,K", [(64, 8), (100, 64), (4096, 2048), (1000, 2056), (257, 4096), (130, 11008)])
+def test_gemm_few_rows_against_transposed_weights(hexmi, oracle, dtype, M, N, K):
+    # up to eight rows with B as [N,K]: the weight-streaming kernel (a wave per output channel), with and without the
+    # epilogue operands, 16-bit and fp32 results
+    a, b = _inputs(M, N, K, dtype, True, seed=M + N)
+    got32 = hexmi.matmul(a.cuda(), b.cuda(), out_dtype=torch.float32, trans_b=True).cpu()
+    want32 = _oracle_mm(oracle, a, b, torch.float32, True)
+    mag = a.float().abs() @ b.float().t().abs()
+    assert ((got32 - want32).abs() <= 1e-5 * mag + 1e-30).all()
+    got = hexmi.matmul(a.cuda(), b.cuda(), trans_b=True).cpu()
+    want = _oracle_mm(oracle, a, b, dtype, True)
+    assert got.dtype == dtype and close16(got, want, max_ulp=1, atol=1e-5 * float(mag.max()))
+    g = _gen(K)
+    bias, resid = torch.randn(N, generator=g).to(dtype), torch.randn(M, N, generator=g).to(dtype)
+    fused = hexmi.matmul(a.cuda(), b.cuda(), trans_b=True, bias=bias.cuda(), residual=resid.cuda()).cpu()
+    ref = (want32.double() + bias.double() + resid.double()).to(dtype)
+    assert close16(fused, ref, max_ulp=1, atol=2e-5 * float(mag.max()))
+
+
 def test_gemm_closed_forms(hexmi):
     g = _gen(1)
     a = torch.randn(256, 128, generator=g).half()
