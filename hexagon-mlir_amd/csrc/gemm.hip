@@ -25,6 +25,7 @@
 // the last slab's chunks past K fetched from a zero chunk; an output side without runs of four columns (odd N with B
 // as [N,K], odd ldc, unaligned C) -> the same kernels with the tile leaving through LDS one element per lane;
 // anything else (unaligned operand rows, K % 8 != 0) -> gemm_kernel_any, which stages the slabs through registers.
+// Up to eight rows against B as [N,K] -> gemv_nt_kernel, a stream of the weights with one wave per output channel.
 #include <type_traits>
 
 #include "hexmi_common.h"
