@@ -92,6 +92,26 @@ def test_gemm_few_rows_against_transposed_weights(hexmi, oracle, dtype, M, N, K)
     assert close16(fused, ref, max_ulp=1, atol=2e-5 * float(mag.max()))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+@pytest.mark.parametrize("N,K", [(64, 8), (104, 64), (4096, 2048), (1000, 2056), (256, 4096), (136, 11008)])
+def test_gemm_few_rows_against_row_major_weights(hexmi, oracle, dtype, M, N, K):
+    # a few rows with B as [K,N] (these run on the tiles: a kernel that streams B in 64-byte pieces measured slower)
+    a, b = _inputs(M, N, K, dtype, False, seed=M + N)
+    got32 = hexmi.matmul(a.cuda(), b.cuda(), out_dtype=torch.float32).cpu()
+    want32 = _oracle_mm(oracle, a, b, torch.float32, False)
+    mag = a.float().abs() @ b.float().abs()
+    assert ((got32 - want32).abs() <= 1e-5 * mag + 1e-30).all()
+    got = hexmi.matmul(a.cuda(), b.cuda()).cpu()
+    want = _oracle_mm(oracle, a, b, dtype, False)
+    assert got.dtype == dtype and close16(got, want, max_ulp=1, atol=1e-5 * float(mag.max()))
+    g = _gen(K)
+    bias, resid = torch.randn(N, generator=g).to(dtype), torch.randn(M, N, generator=g).to(dtype)
+    fused = hexmi.matmul(a.cuda(), b.cuda(), bias=bias.cuda(), residual=resid.cuda()).cpu()
+    ref = (want32.double() + bias.double() + resid.double()).to(dtype)
+    assert close16(fused, ref, max_ulp=1, atol=2e-5 * float(mag.max()))
+
+
 def test_gemm_closed_forms(hexmi):
     g = _gen(1)
     a = torch.randn(256, 128, generator=g).half()
