@@ -228,6 +228,38 @@ class Gemm(Workload):
         return t * (n / rows), "rows 0..%d of A (of %d) x full B, fp32 torch.matmul on CPU, time scaled to the full GEMM" % (rows, n)
 
 
+class GemmNT(Workload):
+    """A[M,K] x W[N,K]^T fp16 off the square benchmark shapes: a decode step (one row: a stream of the weights, priced
+    against HBM) and a vocabulary projection with an odd N (priced against the matrix cores)."""
+    dtype = "f16"
+
+    def __init__(self, M, N, K):
+        self.M, self.N, self.K = M, N, K
+        self.name = "gemm_f16_nt_%dx%dx%d" % (M, N, K)
+        self.bound = "hbm" if M <= 8 else "mfma"
+        self.kernel = "gemv_nt_kernel" if M <= 8 else "gemm_kernel_k64"
+        self.desc = "C = A[%d,%d] . W[%d,%d]^T fp16 U(-1,1), fp32 accumulate, fp16 out" % (M, K, N, K)
+
+    def setup(self, torch, hexmi):
+        from hexmi.workloads import gemm_inputs, gemm_flops
+        self.hexmi, self.host = hexmi, gemm_inputs(self.M, self.N, self.K, torch.float16, trans_b=True)
+        bytes_ = 2 * (self.N * self.K + self.M * self.K + self.M * self.N)
+        self.work = bytes_ if self.bound == "hbm" else gemm_flops(self.M, self.N, self.K)
+        self.sets = _sets(torch, self.host, bytes_, rotate=self.bound == "hbm")
+        for s in self.sets:
+            s["out"] = torch.empty(self.M, self.N, dtype=torch.float16, device="cuda")
+
+    def step(self, i):
+        s = self.sets[i % len(self.sets)]
+        self.hexmi.matmul(s["a"], s["b"], out=s["out"], trans_b=True)
+
+    def cpu(self, torch):
+        a, b = self.host["a"].float(), self.host["b"].float()
+        rows = min(self.M, 512)
+        t = _time_cpu(lambda: torch.matmul(a[:rows], b.t()), 2)
+        return t * (self.M / rows), "rows 0..%d of %d, fp32 torch.matmul on CPU%s" % (rows, self.M, ", time scaled" if rows < self.M else "")
+
+
 class W8A16(Workload):
     bound, dtype = "hbm", "f16"
     # the kernel rocprofv3 names for each measured shape (the library picks by M, N, K)
@@ -574,6 +606,10 @@ def make_workloads():
         Gemm(8192, "bf16", packed=True), Gemm(4096, "f32"), W8A16(1), W8A16(16), W8A16Packed(16), W8A16(64), W8A16(256),
         W8A16(1, 4096, 11008), W8A16(16, 4096, 11008), W8A16(64, 4096, 11008), W8A16(256, 4096, 11008),
         Attention(4, 32, 4096, 128), Attention(1, 32, 16384, 128), AttentionF32(4, 32, 2048, 64),
+        # off the kernels' own shapes: head sizes on padded tiles / two halves, ragged rows, [N,K] weights with one
+        # row and with an odd N
+        Attention(2, 16, 2048, 80), Attention(2, 16, 2048, 256), Softmax(8192, 50257, "f16"),
+        GemmNT(1, 4096, 4096), GemmNT(4096, 50257, 768),
         MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
         Elementwise("sum"), LinearFused(), AddMatmulSoftmax(32, 32, 32, "f32"), AddMatmulSoftmax(512, 512, 64, "f16"),
         CopyCalibration())}
