@@ -1477,8 +1477,12 @@ int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N
   // reads bias and residual in runs of four columns.
   const size_t run = 4 * sizeof(OutT);
   // a few rows against [N,K] weights: the weight stream (see gemv_nt_kernel)
-  if (TRANS_B && M <= 8 && N >= 64 && K % kChunk == 0 && lda % 8 == 0 && ldb % 8 == 0 && aligned_to(A, 16) &&
-      aligned_to(B, 16)) {
+  // (Every workgroup stages the activation rows it multiplies, so their traffic grows with the rows while the
+  // weights' does not: up to two rows always, up to four from K = 1024, up to eight from K = 2048 on -- N = 50264,
+  // K = 768: 14.6 against 23 us on the tiles at one row, 32 against 23 at eight. Nine to sixteen rows as two passes
+  // of eight measured 21.5 against 24 us at N = K = 4096 but 48 against 26 at N = 11008: not taken.)
+  if (TRANS_B && (M <= 2 || (M <= 4 && K >= 1024) || (M <= 8 && K >= 2048)) && N >= 64 && K % kChunk == 0 &&
+      lda % 8 == 0 && ldb % 8 == 0 && aligned_to(A, 16) && aligned_to(B, 16)) {
     const dim3 grid((unsigned)((N + kGemvWaves - 1) / kGemvWaves));
 #define HEXMI_GEMV(MR) \
   hipLaunchKernelGGL((gemv_nt_kernel<T, OutT, MR>), grid, dim3(kGemvWaves * 64), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, \
