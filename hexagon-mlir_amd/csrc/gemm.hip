@@ -1257,29 +1257,39 @@ template <> struct Dot8<bf16> {
 
 constexpr int kGemvWaves = 8, kGemvBlockK = 2048;
 
-template <typename T, typename OutT, int MR>
-__global__ __launch_bounds__(kGemvWaves * 64)
+// RPW: output channels per wave (a chunk of activations read from LDS then serves RPW weight rows; measured, it did
+// not pay: see the launch).
+template <typename T, typename OutT, int MR, int NW = kGemvWaves, int RPW = 1>
+__global__ __launch_bounds__(NW * 64)
 void gemv_nt_kernel(const T* __restrict__ A, const T* __restrict__ W, OutT* C, int M, int N, int K, int64_t lda,
                     int64_t ldb, int64_t ldc, const OutT* __restrict__ bias, const OutT* resid, int64_t ldr) {
   constexpr int KB = kGemvBlockK, CPB = KB / kChunk;  // chunks per row of a staged block
+  constexpr int CPL = CPB / kWave;                    // chunks per lane, row and block
   __shared__ __attribute__((aligned(16))) T a_s[MR][KB];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int n = blockIdx.x * kGemvWaves + wave;
-  const T* wrow = W + (int64_t)(n < N ? n : N - 1) * ldb;   // past the end: the last channel again, not stored
-  float acc[MR];
+  const int n_first = (blockIdx.x * NW + wave) * RPW;
+  const T* wrow[RPW];
 #pragma unroll
-  for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+  for (int q = 0; q < RPW; ++q)                        // past the end: the last channel again, not stored
+    wrow[q] = W + (int64_t)(n_first + q < N ? n_first + q : N - 1) * ldb;
+  float acc[MR][RPW];
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int q = 0; q < RPW; ++q) acc[m][q] = 0.0f;
   for (int kb = 0; kb < K; kb += KB) {
     const int kn = K - kb < KB ? K - kb : KB;           // columns of this block, a multiple of 8
     // the weight chunks of this block first: they come from HBM, the activations below from L2
-    u32x4 wv[CPB / kWave];
+    u32x4 wv[RPW][CPL];
 #pragma unroll
-    for (int j = 0; j < CPB / kWave; ++j) {
-      const int k = (j * kWave + lane) * kChunk;
-      wv[j] = k < kn ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + kb + k)) : u32x4{0u, 0u, 0u, 0u};
-    }
+    for (int q = 0; q < RPW; ++q)
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        const int k = (j * kWave + lane) * kChunk;
+        wv[q][j] = k < kn ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[q] + kb + k)) : u32x4{0u, 0u, 0u, 0u};
+      }
     __syncthreads();                                    // every wave has read the block before
-    for (int c = threadIdx.x; c < MR * CPB; c += kGemvWaves * 64) {
+    for (int c = threadIdx.x; c < MR * CPB; c += NW * 64) {
       const int m = c / CPB, k = (c % CPB) * kChunk;
       if (k < kn)
         *reinterpret_cast<u32x4*>(&a_s[m][k]) =
@@ -1287,23 +1297,30 @@ void gemv_nt_kernel(const T* __restrict__ A, const T* __restrict__ W, OutT* C, i
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < CPB / kWave; ++j) {
+    for (int j = 0; j < CPL; ++j) {
       const int k = (j * kWave + lane) * kChunk;
       if (k < kn) {
 #pragma unroll
-        for (int m = 0; m < MR; ++m) acc[m] = Dot8<T>::run(wv[j], *reinterpret_cast<const u32x4*>(&a_s[m][k]), acc[m]);
+        for (int m = 0; m < MR; ++m) {
+          const u32x4 av = *reinterpret_cast<const u32x4*>(&a_s[m][k]);
+#pragma unroll
+          for (int q = 0; q < RPW; ++q) acc[m][q] = Dot8<T>::run(wv[q][j], av, acc[m][q]);
+        }
       }
     }
   }
 #pragma unroll
-  for (int m = 0; m < MR; ++m) {
-    float sum = wave_sum(acc[m]);
-    if (lane == 0 && n < N && m < M) {
-      if (bias) sum += to_f32<OutT>(bias[n]);
-      if (resid) sum += to_f32<OutT>(resid[(int64_t)m * ldr + n]);
-      C[(int64_t)m * ldc + n] = from_f32<OutT>(sum);
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int q = 0; q < RPW; ++q) {
+      float sum = wave_sum(acc[m][q]);
+      const int n = n_first + q;
+      if (lane == 0 && n < N && m < M) {
+        if (bias) sum += to_f32<OutT>(bias[n]);
+        if (resid) sum += to_f32<OutT>(resid[(int64_t)m * ldr + n]);
+        C[(int64_t)m * ldc + n] = from_f32<OutT>(sum);
+      }
     }
-  }
 }
 
 // fp32 inputs (the reference's torch-mlir graphs multiply fp32 matrices, e.g.
@@ -1483,11 +1500,14 @@ int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N
   // of eight measured 21.5 against 24 us at N = K = 4096 but 48 against 26 at N = 11008: not taken.)
   if (TRANS_B && (M <= 2 || (M <= 4 && K >= 1024) || (M <= 8 && K >= 2048)) && N >= 64 && K % kChunk == 0 &&
       lda % 8 == 0 && ldb % 8 == 0 && aligned_to(A, 16) && aligned_to(B, 16)) {
-    const dim3 grid((unsigned)((N + kGemvWaves - 1) / kGemvWaves));
-#define HEXMI_GEMV(MR) \
-  hipLaunchKernelGGL((gemv_nt_kernel<T, OutT, MR>), grid, dim3(kGemvWaves * 64), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, \
-                     ldc, bias, resid, ldr)
-    if (M == 1) HEXMI_GEMV(1); else if (M == 2) HEXMI_GEMV(2); else if (M <= 4) HEXMI_GEMV(4); else HEXMI_GEMV(8);
+#define HEXMI_GEMV(MR, NW, RPW) \
+  hipLaunchKernelGGL((gemv_nt_kernel<T, OutT, MR, NW, RPW>), dim3((unsigned)((N + NW * RPW - 1) / (NW * RPW))), dim3(NW * 64), 0, s, \
+                     A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, bias, resid, ldr)
+    // one channel per wave throughout: two for four rows measured equal to slower (N = 4096, K = 11008: 22.2 against
+    // 19.9 us), four for eight rows 38 against 22.5 us at N = 11008 (130 registers, four strided rows per load
+    // group); sixteen waves share the staged rows from five rows on (24 -> 22.5 us)
+    if (M == 1) HEXMI_GEMV(1, 8, 1); else if (M == 2) HEXMI_GEMV(2, 8, 1); else if (M <= 4) HEXMI_GEMV(4, 8, 1);
+    else HEXMI_GEMV(8, 16, 1);
 #undef HEXMI_GEMV
     return launch_status();
   }
