@@ -26,6 +26,7 @@
 // as [N,K], odd ldc, unaligned C) -> the same kernels with the tile leaving through LDS one element per lane;
 // anything else (unaligned operand rows, K % 8 != 0) -> gemm_kernel_any, which stages the slabs through registers.
 // Up to eight rows against B as [N,K] -> gemv_nt_kernel, a stream of the weights with one wave per output channel.
+#include <algorithm>
 #include <type_traits>
 
 #include "hexmi_common.h"
@@ -1323,6 +1324,92 @@ void gemv_nt_kernel(const T* __restrict__ A, const T* __restrict__ W, OutT* C, i
     }
 }
 
+// Nine to sixty-four rows against [N,K] weights: still a stream of the weights, now on the matrix cores. One workgroup
+// of four waves per tile of 16 output channels (N / 16 workgroups where 128-column tiles would be N / 128); the waves
+// split K four ways in runs of whole 128-byte lines and their partial tiles meet in LDS. A lane's 16-byte weight load
+// is its MFMA 16x16x32 operand as it stands (channel lane % 16, eight k from 8 * (lane / 16) on), all loads of a round
+// issued before the first MFMA; the activation fragments come through L1 / L2. K % 32 == 0, rows on 16-byte
+// boundaries. MT: 16-row tiles of activations.
+template <typename T> struct Mfma16Builtin;
+template <> struct Mfma16Builtin<f16> {
+  static __device__ __forceinline__ f32x4 run(const u32x4& w, const u32x4& a, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w), __builtin_bit_cast(f16x8, a), c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16Builtin<bf16> {
+  static __device__ __forceinline__ f32x4 run(const u32x4& w, const u32x4& a, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, a), c, 0, 0, 0);
+  }
+};
+
+template <typename T, typename OutT, int MT>
+__global__ __launch_bounds__(256)
+void gemm_nt_skinny_kernel(const T* __restrict__ A, const T* __restrict__ W, OutT* C, int M, int N, int K, int64_t lda,
+                           int64_t ldb, int64_t ldc, const OutT* __restrict__ bias, const OutT* resid, int64_t ldr) {
+  constexpr int NWV = 4;
+  __shared__ __attribute__((aligned(16))) float red[NWV * MT * 256];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int r16 = lane % 16, kg = lane / 16;
+  const int tile = blockIdx.x;
+  const int n = tile * 16 + r16;
+  const T* wrow = W + (int64_t)(n < N ? n : N - 1) * ldb + kg * kChunk;
+  const int steps = K / 32;
+  const int per_wave = (((steps + NWV - 1) / NWV) + 1) & ~1;      // an even number of 64-byte steps: whole lines
+  const int s_begin = wave * per_wave;
+  const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
+  const T* arow[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int gm = t * 16 + r16;
+    arow[t] = A + (int64_t)(gm < M ? gm : M - 1) * lda + kg * kChunk;   // past the end: the last row, not stored
+  }
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
+  for (int s0 = s_begin; s0 < s_end; s0 += U) {
+    u32x4 wv[U], av[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      wv[u] = u32x4{0u, 0u, 0u, 0u};
+      if (s0 + u < s_end) wv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + (int64_t)(s0 + u) * 32));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        av[u][t] = u32x4{0u, 0u, 0u, 0u};
+        if (s0 + u < s_end) av[u][t] = *reinterpret_cast<const u32x4*>(arow[t] + (int64_t)(s0 + u) * 32);
+      }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = Mfma16Builtin<T>::run(wv[u], av[u][t], acc[t]);   // a skipped step is zeros
+  }
+  // D[i = channel][j = activation row]: a lane holds row lane % 16, channels 4 * (lane / 16) + 0 .. 3
+#pragma unroll
+  for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4*>(red + ((wave * MT + t) * 64 + lane) * 4) = acc[t];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < MT * 64; idx += 256) {
+    const int t = idx / 64, l = idx % 64;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) sum += *reinterpret_cast<const f32x4*>(red + ((w * MT + t) * 64 + l) * 4);
+    const int gm = t * 16 + l % 16;
+    const int gn = tile * 16 + (l / 16) * 4;
+    if (gm < M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (gn + e < N) {
+          float v = sum[e];
+          if (bias) v += to_f32<OutT>(bias[gn + e]);
+          if (resid) v += to_f32<OutT>(resid[(int64_t)gm * ldr + gn + e]);
+          C[(int64_t)gm * ldc + gn + e] = from_f32<OutT>(v);
+        }
+    }
+  }
+}
+
 // fp32 inputs (the reference's torch-mlir graphs multiply fp32 matrices, e.g.
 // test/python/torch-mlir/test_add_matmul_softmax.py:25-29) whose shape or alignment the matrix-core kernel of
 // gemm_f32.hip does not take: 64x64 tile, K in steps of 16 through LDS, every thread a 4x4 block of fp32 FMAs.
@@ -1509,6 +1596,23 @@ int dispatch_gemm(const void* Av, const void* Bv, void* Cv, int64_t M, int64_t N
     if (M == 1) HEXMI_GEMV(1, 8, 1); else if (M == 2) HEXMI_GEMV(2, 8, 1); else if (M <= 4) HEXMI_GEMV(4, 8, 1);
     else HEXMI_GEMV(8, 16, 1);
 #undef HEXMI_GEMV
+    return launch_status();
+  }
+  // Every workgroup of the skinny kernel pulls all M x K activations through L2, N / 16 times over in total, where
+  // the tiles walk K with N / 128 workgroups: it wins while N is near sixteen channels per CU or K is long. Both
+  // sides as fitted on 256 CUs, in microseconds (N = K = 4096: 12.1 / 15.4 / 22.3 at 16 / 32 / 64 rows against
+  // 24 on the tiles; N = 4096, K = 11008: 27 / 36 / 56 against 57; N = 11008, K = 4096: 28 / 39 / 63 against 26).
+  const double nk = (double)N * (double)K;
+  const double skinny_us = 3.0 + 2.0 * nk / 6.0e6 + 1.27e-8 * nk * (double)M;
+  const double tiles_us = std::max(23.0, 4.0 + 5.2e-3 * (double)K * (double)((N + 128 * 512 - 1) / (128 * 512)));
+  if (TRANS_B && M <= 64 && N >= 64 && K % 32 == 0 && lda % 8 == 0 && ldb % 8 == 0 && aligned_to(A, 16) &&
+      aligned_to(B, 16) && skinny_us < 0.9 * tiles_us) {
+    const dim3 grid((unsigned)((N + 15) / 16));
+#define HEXMI_SKINNY(MT) \
+  hipLaunchKernelGGL((gemm_nt_skinny_kernel<T, OutT, MT>), grid, dim3(256), 0, s, A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, \
+                     bias, resid, ldr)
+    if (M <= 16) HEXMI_SKINNY(1); else if (M <= 32) HEXMI_SKINNY(2); else HEXMI_SKINNY(4);
+#undef HEXMI_SKINNY
     return launch_status();
   }
   const bool fast = K % BK == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && N % 8 == 0 && N >= 8 &&

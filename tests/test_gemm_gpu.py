@@ -72,11 +72,12 @@ def test_gemm_parity(hexmi, oracle, shape, dtype, trans_b):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 9, 12, 13, 16])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 9, 12, 13, 16, 17, 32, 33, 48, 64])
 @pytest.mark.parametrize("N,K", [(64, 8), (100, 64), (4096, 2048), (1000, 2056), (257, 4096), (130, 11008)])
 def test_gemm_few_rows_against_transposed_weights(hexmi, oracle, dtype, M, N, K):
-    # up to sixteen rows with B as [N,K]: the weight-streaming kernel (a wave per output channel, eight rows a pass),
-    # with and without the epilogue operands, 16-bit and fp32 results
+    # up to 64 rows with B as [N,K]: the weight-streaming kernels (a wave per output channel up to eight rows, a
+    # workgroup per 16 channels on the matrix cores beyond), with and without the epilogue operands, 16-bit and fp32
+    # results
     a, b = _inputs(M, N, K, dtype, True, seed=M + N)
     got32 = hexmi.matmul(a.cuda(), b.cuda(), out_dtype=torch.float32, trans_b=True).cpu()
     want32 = _oracle_mm(oracle, a, b, torch.float32, True)
