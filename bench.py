@@ -229,15 +229,15 @@ class Gemm(Workload):
 
 
 class GemmNT(Workload):
-    """A[M,K] x W[N,K]^T fp16 off the square benchmark shapes: a decode step (one row: a stream of the weights, priced
-    against HBM) and a vocabulary projection with an odd N (priced against the matrix cores)."""
+    """A[M,K] x W[N,K]^T fp16 off the square benchmark shapes: a decode step (one row or sixteen: a stream of the
+    weights, priced against HBM) and a vocabulary projection with an odd N (priced against the matrix cores)."""
     dtype = "f16"
 
     def __init__(self, M, N, K):
         self.M, self.N, self.K = M, N, K
         self.name = "gemm_f16_nt_%dx%dx%d" % (M, N, K)
-        self.bound = "hbm" if M <= 8 else "mfma"
-        self.kernel = "gemv_nt_kernel" if M <= 8 else "gemm_kernel_k64"
+        self.bound = "hbm" if M <= 64 else "mfma"
+        self.kernel = "gemv_nt_kernel" if M <= 8 else ("gemm_nt_skinny_kernel" if M <= 64 else "gemm_kernel_k64")
         self.desc = "C = A[%d,%d] . W[%d,%d]^T fp16 U(-1,1), fp32 accumulate, fp16 out" % (M, K, N, K)
 
     def setup(self, torch, hexmi):
@@ -609,7 +609,7 @@ def make_workloads():
         # off the kernels' own shapes: head sizes on padded tiles / two halves, ragged rows, [N,K] weights with one
         # row and with an odd N
         Attention(2, 16, 2048, 80), Attention(2, 16, 2048, 256), Softmax(8192, 50257, "f16"),
-        GemmNT(1, 4096, 4096), GemmNT(4096, 50257, 768),
+        GemmNT(1, 4096, 4096), GemmNT(16, 4096, 4096), GemmNT(4096, 50257, 768),
         MaskedAttention(32, 2048, 128), Elementwise("gelu"), Elementwise("silu"), Elementwise("rope"),
         Elementwise("sum"), LinearFused(), AddMatmulSoftmax(32, 32, 32, "f32"), AddMatmulSoftmax(512, 512, 64, "f16"),
         CopyCalibration())}

@@ -58,7 +58,15 @@ def _compile(src, force, hdr_mtime):
             and os.path.getmtime(obj) > max(os.path.getmtime(path), hdr_mtime)):
         return obj, False
     cmd = [HIPCC] + flags_for(src) + ["-c", path, "-o", obj]
-    r = subprocess.run(cmd, capture_output=True, text=True)
+    # hipcc reads the source once for the device pass and again for the host pass: a file saved in between gives an
+    # object whose launch stubs name kernels its code object does not hold (the first such launch aborts the process)
+    for _ in range(3):
+        before = os.path.getmtime(path)
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if os.path.getmtime(path) == before:
+            break
+    else:
+        raise RuntimeError("%s kept changing while it was compiled" % src)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
     return obj, True

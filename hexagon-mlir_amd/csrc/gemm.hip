@@ -26,6 +26,7 @@
 // as [N,K], odd ldc, unaligned C) -> the same kernels with the tile leaving through LDS one element per lane;
 // anything else (unaligned operand rows, K % 8 != 0) -> gemm_kernel_any, which stages the slabs through registers.
 // Up to eight rows against B as [N,K] -> gemv_nt_kernel, a stream of the weights with one wave per output channel.
+// Nine to 64 rows against B as [N,K], where a fitted cost says so -> gemm_nt_skinny_kernel, a workgroup per 16 channels.
 #include <algorithm>
 #include <type_traits>
 
