@@ -126,13 +126,19 @@ __device__ __forceinline__ float rsqrt_newton(float x) {
 // issue of the next ones.
 // Without PIPE a workgroup handles exactly one row group (gridDim.x == number of groups) and accesses are masked.
 // RAGGED (never with PIPE): rows at any alignment and of any length; the masks are per element.
-template <typename T, int OP, int CHUNKS, int THREADS, int ROWS_PER_BLOCK, bool PIPE, bool RAGGED = false>
+// SPAN (softmax, RAGGED, x and y rows equally far off a 16-byte boundary): the row is walked as the aligned 16-byte
+// chunks that cover it, the first of them starting up to N - 1 elements before the row. Whole chunks are read and
+// written aligned (the bytes of the first and last chunk outside the row are read, sit inside the same 16 aligned
+// bytes as the row's own, and are masked); only the row's two end chunks are stored element by element. An access
+// at the alignment of the element type costs about 1.6 times an aligned one.
+template <typename T, int OP, int CHUNKS, int THREADS, int ROWS_PER_BLOCK, bool PIPE, bool RAGGED = false, bool SPAN = false>
 __global__ __launch_bounds__(THREADS * ROWS_PER_BLOCK)
 void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict__ w,
                 const T* __restrict__ b, float* __restrict__ mean_out, float* __restrict__ rstd_out,
                 int64_t rows, int cols, int64_t ld_x, int64_t ld_y, float eps) {
   constexpr bool FULL = PIPE;
   static_assert(!(PIPE && RAGGED), "the pipelined walk is for exact tiles");
+  static_assert(!SPAN || (RAGGED && OP == kSoftmax), "aligned spans: softmax over ragged rows");
   // MIX (fp16 norms, pipelined walk): the row is kept as loaded and every first use converts it inside the
   // arithmetic (v_fma_mix_f32 reads an fp16 half of a register as one operand of an fp32 fma, at the issue cost of
   // a plain fma), instead of sixteen conversions per thread and row up front. The norms issue vector instructions
@@ -177,17 +183,23 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
   };
   // Chunks past the end of the row load column 0 instead (and are ignored): the loads stay free of branches,
   // which lets them be issued back to back and waited for only where their values are used.
+  // SPAN: elements between the 16-byte boundary at or below the row's first element and that element; positions
+  // count from the boundary, the row is positions lead .. lead + cols - 1
+  int lead = 0;
+  if constexpr (SPAN)
+    lead = (int)((reinterpret_cast<uintptr_t>(x + row_of(blockIdx.x) * ld_x) / sizeof(T)) % N);
+  const int span = cols + lead;
   int load_col[CHUNKS];
 #pragma unroll
-  for (int c = 0; c < CHUNKS; ++c) load_col[c] = (c * THREADS + t) * N < cols ? (c * THREADS + t) * N : 0;
+  for (int c = 0; c < CHUNKS; ++c) load_col[c] = (c * THREADS + t) * N < span ? (c * THREADS + t) * N : 0;
   // RAGGED: elements of chunk c inside the row (a chunk past the end stands in for column 0's, as above)
   auto left = [&](int c) { return cols - load_col[c]; };
   Vec16<T> raw_a[CHUNKS];
   {
-    const T* xr = x + row_of(blockIdx.x) * ld_x;
+    const T* xr = x + row_of(blockIdx.x) * ld_x - lead;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
-      if constexpr (RAGGED) raw_a[c] = load16_any(xr + load_col[c], left(c));
+      if constexpr (RAGGED && !SPAN) raw_a[c] = load16_any(xr + load_col[c], left(c));
       else raw_a[c] = load16_stream(xr + load_col[c]);
     }
   }
@@ -221,11 +233,12 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
     if constexpr (!MIX) {
 #pragma unroll
       for (int c = 0; c < CHUNKS; ++c) {
-        const bool in = FULL || (c * THREADS + t) * N < cols;
+        const bool in = FULL || (c * THREADS + t) * N < span;
 #pragma unroll
         for (int i = 0; i < N; ++i)
-          v[c][i] = in && (!RAGGED || (c * THREADS + t) * N + i < cols) ? to_f32<T>(raw[c].v[i])
-                                                                         : (OP == kSoftmax ? -INFINITY : 0.0f);
+          v[c][i] = in && (!RAGGED || (c * THREADS + t) * N + i < span) && (!SPAN || (c * THREADS + t) * N + i >= lead)
+                        ? to_f32<T>(raw[c].v[i])
+                        : (OP == kSoftmax ? -INFINITY : 0.0f);
       }
     }
     flush_stats();
@@ -252,12 +265,24 @@ void row_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict_
 #pragma unroll
       for (int c = 0; c < CHUNKS; ++c) {
         const int col = (c * THREADS + t) * N;
-        if (FULL || (col < cols && row_valid)) {
+        if (FULL || (col < span && row_valid)) {
           Vec16<T> o;
 #pragma unroll
           for (int i = 0; i < N; ++i) o.v[i] = from_f32<T>(v[c][i] * inv);
-          if constexpr (RAGGED) store16_any(yr + col, o, cols - col);
-          else store16_stream(yr + col, o);
+          if constexpr (SPAN) {
+            T* ya = yr - lead + col;                      // 16-byte aligned: y's rows are as far off as x's
+            if (col >= lead && col + N <= span) {
+              store16_stream(ya, o);
+            } else {
+#pragma unroll
+              for (int i = 0; i < N; ++i)
+                if (col + i >= lead && col + i < span) ya[i] = o.v[i];
+            }
+          } else if constexpr (RAGGED) {
+            store16_any(yr + col, o, cols - col);
+          } else {
+            store16_stream(yr + col, o);
+          }
         }
       }
     } else {
@@ -706,6 +731,28 @@ int dispatch_rows(const void* xv, void* yv, const void* wv, const void* bv, floa
 #define HEXMI_RAGGED(C, TH, RPB) \
   { hipLaunchKernelGGL((row_kernel<T, OP, C, TH, RPB, false, true>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(TH * RPB), 0, s, \
                        x, y, w, b, mean, rstd, rows, (int)cols, ld_x, ld_y, eps); return launch_status(); }
+  // softmax with x and y rows equally far off a 16-byte boundary (contiguous tensors with an odd number of columns,
+  // equal column slices of aligned ones): aligned chunks over the span that covers the row, one chunk more at most
+  if constexpr (OP == kSoftmax) {
+    const bool same_offset = aligned_to(x, sizeof(T)) && aligned_to(y, sizeof(T)) &&
+                             (reinterpret_cast<uintptr_t>(x) - reinterpret_cast<uintptr_t>(y)) % 16 == 0 &&
+                             ((ld_x - ld_y) * (int64_t)sizeof(T)) % 16 == 0;
+    const int64_t span_chunks = (cols + 2 * N - 2) / N;
+    if (!vec_ok && same_offset && rows <= 0x7fffffff && cols < 0x7ffffff0) {
+#define HEXMI_SPAN(C, TH, RPB) \
+  { hipLaunchKernelGGL((row_kernel<T, OP, C, TH, RPB, false, true, true>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(TH * RPB), 0, \
+                       s, x, y, w, b, mean, rstd, rows, (int)cols, ld_x, ld_y, eps); return launch_status(); }
+      if (span_chunks <= 64 * 1) HEXMI_SPAN(1, 64, 4);
+      if (span_chunks <= 64 * 2) HEXMI_SPAN(2, 64, 4);
+      if (span_chunks <= 64 * 4) HEXMI_SPAN(4, 64, 4);
+      if (span_chunks <= 256 * 2) HEXMI_SPAN(2, 256, 1);
+      if (span_chunks <= 256 * 4) HEXMI_SPAN(4, 256, 1);
+      if (span_chunks <= 512 * 4) HEXMI_SPAN(4, 512, 1);
+      if (span_chunks <= 1024 * 4) HEXMI_SPAN(4, 1024, 1);
+      if (span_chunks <= 1024 * 8) HEXMI_SPAN(8, 1024, 1);
+#undef HEXMI_SPAN
+    }
+  }
   if (!vec_ok && rows <= 0x7fffffff) {
     if (chunks <= 64 * 1) HEXMI_RAGGED(1, 64, 4);
     if (chunks <= 64 * 2) HEXMI_RAGGED(2, 64, 4);

@@ -369,14 +369,18 @@ def test_rows_that_are_not_whole_chunks(hexmi, oracle, dtype, cols):
     a, tag = to_np(x)
     wn, bn = to_np(w)[0], to_np(b)[0]
 
-    def window():
+    def window(lead=32):
         buf = torch.full((rows * cols + 64,), 5.0, dtype=dtype, device="cuda")
-        return buf, buf[32:32 + rows * cols].view(rows, cols)
+        return buf, buf[lead:lead + rows * cols].view(rows, cols)
 
-    buf, out = window()
-    hexmi.softmax(x.cuda(), out=out)
-    _check(out, from_np(oracle.softmax(a, dtype=tag), dtype), dtype, atol16=1e-7)
-    assert (buf[:32] == 5.0).all() and (buf[32 + rows * cols:] == 5.0).all()
+    # softmax: output rows as far off the 16-byte boundaries as the input's (whole aligned chunks over the span that
+    # covers a row), then three elements further (accesses at the alignment of the element type)
+    want_sm = from_np(oracle.softmax(a, dtype=tag), dtype)
+    for lead in (32, 35):
+        buf, out = window(lead)
+        hexmi.softmax(x.cuda(), out=out)
+        _check(out, want_sm, dtype, atol16=1e-7)
+        assert (buf[:lead] == 5.0).all() and (buf[lead + rows * cols:] == 5.0).all()
     buf, out = window()
     hexmi.rms_norm(x.cuda(), w.cuda(), 1e-5, out=out)
     _check(out, from_np(oracle.rms_norm(a, wn, 1e-5, dtype=tag), dtype), dtype)
