@@ -1010,8 +1010,8 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, typen
       // contiguous bytes per row) instead of 8-byte pieces of 16 rows. Each wave stages its tile in one of the four
       // operand stages (same size or larger); chunks are XOR-swizzled so both the 8-byte writes and the 16-byte
       // reads spread over the banks.
-      // out_elems: the output side allows no 16-byte pieces (an odd N or leading dimension, an unaligned base): the
-      // staged tile leaves one element per lane, 64 neighbours of a row per instruction.
+      // out_elems: the rows of the output start off the 16-byte boundaries (an odd N or leading dimension, an
+      // unaligned base): the staged tile leaves in the aligned pieces each row holds, its ends by elements.
       __syncthreads();                                // every wave has finished reading fragments
       OutT* cs = wave == 0 ? reinterpret_cast<OutT*>(a_p0) : wave == 1 ? reinterpret_cast<OutT*>(a_p1)
                  : wave == 2 ? reinterpret_cast<OutT*>(b_p0) : reinterpret_cast<OutT*>(b_p1);
@@ -1030,15 +1030,44 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, typen
         }
       }
       if (by_elements) {
-#pragma unroll 4
-        for (int row = 0; row < TM * 16; ++row) {
+        // A row of C starts anywhere, but most of it is whole 16-byte pieces: a lane gathers the eight elements of
+        // one aligned piece from the staged tile (they straddle two of its chunks) and stores them at once, 64 / CP
+        // rows per instruction; what a row has before its first boundary and after its last whole piece (up to
+        // seven elements each) goes element by element, a lane per row.
+        constexpr int W = TN * 16;                    // columns of the wave's tile
+        const int gbase = n0 + wn * W;
+        const int ncols = N - gbase < W ? (int)(N - gbase) : W;
+        const int64_t c_elem = (int64_t)(reinterpret_cast<uintptr_t>(C) / sizeof(OutT));
+        auto staged = [&](int row, int col) {
+          return cs[row * PITCH + (((col / kChunk) ^ swz(row)) * kChunk) + col % kChunk];
+        };
+        // columns up to the row's first 16-byte boundary
+        auto lead_of = [&](int64_t e0) { return (int)((kChunk - ((c_elem + e0) & (kChunk - 1))) & (kChunk - 1)); };
+        constexpr int RPS = 64 / CP;
+#pragma unroll 2
+        for (int r0 = 0; r0 < TM * 16; r0 += RPS) {
+          const int row = r0 + lane / CP, q = lane % CP;
           const int grow = m0 + wm * TM * 16 + row;
-          if (grow >= M) break;
+          const int64_t e0 = (int64_t)grow * ldc + gbase;
+          const int c0 = lead_of(e0) + kChunk * q;
+          if (grow < M && c0 + kChunk <= ncols) {
+            __attribute__((aligned(16))) OutT o[kChunk];
 #pragma unroll
-          for (int h = 0; h < TN * 16 / 64; ++h) {
-            const int col = h * 64 + lane, gcol = n0 + wn * TN * 16 + col;
-            if (gcol < N)
-              C[(int64_t)grow * ldc + gcol] = cs[row * PITCH + (((col / kChunk) ^ swz(row)) * kChunk) + col % kChunk];
+            for (int i = 0; i < kChunk; ++i) o[i] = staged(row, c0 + i);
+            __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(o), reinterpret_cast<u32x4*>(C + e0 + c0));
+          }
+        }
+#pragma unroll 1
+        for (int r0 = 0; r0 < TM * 16; r0 += 64) {
+          const int row = r0 + lane;
+          const int grow = m0 + wm * TM * 16 + row;
+          if (row < TM * 16 && grow < M && ncols > 0) {
+            const int64_t e0 = (int64_t)grow * ldc + gbase;
+            const int lead = lead_of(e0);
+            const int head = lead < ncols ? lead : ncols;
+            const int tail = ncols > lead ? lead + ((ncols - lead) & ~(kChunk - 1)) : ncols;
+            for (int c = 0; c < head; ++c) C[e0 + c] = staged(row, c);
+            for (int c = tail; c < ncols; ++c) C[e0 + c] = staged(row, c);
           }
         }
         return;

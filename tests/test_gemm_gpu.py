@@ -164,6 +164,30 @@ def test_gemm_odd_width_on_large_tiles(hexmi, dtype):
     assert (got.cpu()[rows].double() - ref).abs().max() <= 2e-2 * math.sqrt(K)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gemm_output_rows_off_the_boundaries(hexmi, dtype):
+    # [N,K] weights, whole 64-wide slabs, output rows that start anywhere (odd widths, leading dimensions wider than
+    # the rows, a base 2 or 6 bytes into its buffer; C ABI): the staged tile leaves in the aligned 16-byte pieces of
+    # each row and its ends by elements. Bit for bit the dense call's values, nothing outside the window written.
+    from hexmi import _lib
+    L = _lib.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    dt = _lib.F16 if dtype == torch.float16 else _lib.BF16
+    for M, N, K, pad, lead in ((300, 1001, 256, 0, 0), (300, 1001, 256, 3, 1), (129, 70, 64, 1, 3), (520, 777, 128, 6, 0),
+                               (4096, 2049, 128, 0, 1), (64, 5, 64, 2, 1), (257, 263, 192, 4, 3)):
+        a, b = _inputs(M, N, K, dtype, True, seed=M + N + pad)
+        ldc = N + pad
+        c_buf = torch.full((M * ldc + lead + 9,), 7.0, dtype=dtype, device="cuda")
+        ad, bd = a.cuda(), b.cuda()
+        rc = L.hexmi_gemm(M, N, K, ad.data_ptr(), K, bd.data_ptr(), K, c_buf.data_ptr() + 2 * lead, ldc, dt, dt, 1, st)
+        assert rc == 0
+        b_pad = torch.cat([b, torch.zeros((-N) % 8, K, dtype=dtype)])
+        want = hexmi.matmul(ad, b_pad.cuda(), trans_b=True)[:, :N]
+        c = c_buf[lead:lead + M * ldc].view(M, ldc)
+        assert torch.equal(c[:, :N], want), (M, N, K, pad, lead)
+        assert (c_buf[:lead] == 7.0).all() and (c[:, N:] == 7.0).all() and (c_buf[lead + M * ldc:] == 7.0).all()
+
+
 def test_gemm_unaligned_views(hexmi):
     # operands and result that start 2 bytes into their buffers, odd leading dimensions (C ABI only): the any-shape
     # kernel; nothing outside the result's window is written
