@@ -248,12 +248,12 @@ __device__ __forceinline__ void add_epilogue4(f32x4& a, const OutT* __restrict__
   }
 }
 
-// The output tile of a workgroup (waves 2 x NWN, each WM x WN MFMA tiles of 32x32) leaves through LDS in rows, one
-// element per lane, for output sides that allow no runs of four columns (an odd N or leading dimension, an unaligned
-// base). Storing a lane's accumulators one by one would be 64 pieces of 64 different rows per instruction (measured:
-// 876 us against 324 for the aligned neighbour of [4096, 768] x [50257, 768]^T), so the tile is staged kRows rows at
-// a time -- a pass takes its rows of one MFMA tile row from the waves that hold it -- and every store instruction
-// then covers 64 neighbours of one row. Bias and residual are added on the way in, element by element (a residual
+// The output tile of a workgroup (waves 2 x NWN, each WM x WN MFMA tiles of 32x32) leaves through LDS in rows, for
+// output sides that allow no runs of four columns (an odd N or leading dimension, an unaligned base). Storing a
+// lane's accumulators one by one would be 64 pieces of 64 different rows per instruction (measured: 876 us against
+// 324 for the aligned neighbour of [4096, 768] x [50257, 768]^T), so the tile is staged kRows rows at a time -- a
+// pass takes its rows of one MFMA tile row from the waves that hold it -- and leaves in the aligned 16-byte pieces
+// of each row. Bias and residual are added on the way in, element by element (a residual
 // that is the output buffer is read before any element of the pass is stored).
 // c_s: kRows x (BN + 4) elements: 32 rows of 16-bit results or 16 of fp32 (8.25 KiB at BN = 128); the pitch keeps the
 // rows of a wave's 8- or 16-byte writes on different banks.
@@ -297,16 +297,40 @@ __device__ __forceinline__ void store_tile_by_rows(const f32x16 (&acc)[WM][WN], 
         }
     }
     __syncthreads();
+    // the staged rows leave in the aligned 16-byte pieces each holds (a lane gathers a piece's elements), the up to
+    // E - 1 elements before a row's first boundary and after its last whole piece by elements, a lane per row
+    constexpr int E = 16 / (int)sizeof(OutT), CPR = BN / E;
+    const int ncols = N - n0 < BN ? N - n0 : BN;
+    const int64_t c_elem = (int64_t)(reinterpret_cast<uintptr_t>(C) / sizeof(OutT));
+    auto lead_of = [&](int64_t e0) { return (int)((E - ((c_elem + e0) & (E - 1))) & (E - 1)); };
+    const int tid = wave * 64 + lane;
 #pragma unroll
-    for (int rr = 0; rr < PR / NW; ++rr) {
-      const int lr = wave * (PR / NW) + rr, row = m0 + p * PR + lr;
-      if (row < M) {
+    for (int idx = tid; idx < PR * CPR; idx += NW * 64) {
+      const int lr = idx / CPR, q = idx % CPR, row = m0 + p * PR + lr;
+      const int64_t e0 = (int64_t)row * ldc + n0;
+      const int c0 = lead_of(e0) + E * q;
+      if (row < M && c0 + E <= ncols) {
+        __attribute__((aligned(16))) OutT o[E];
 #pragma unroll
-        for (int h = 0; h < BN / 64; ++h) {
-          const int col = h * 64 + lane;
-          if (n0 + col < N) C[(int64_t)row * ldc + n0 + col] = c_s[lr * PITCH + col];
-        }
+        for (int i = 0; i < E; ++i) o[i] = c_s[lr * PITCH + c0 + i];
+        *reinterpret_cast<u32x4*>(C + e0 + c0) = *reinterpret_cast<const u32x4*>(o);
       }
+    }
+    // (every read of the staged row ahead of the first store, the stores under masks: a loop with one read and one
+    // store per turn would put a pass's worth of LDS latencies end to end on one wave while the others wait)
+    if (tid < 2 * PR && m0 + p * PR + tid % PR < M && ncols > 0) {
+      const int lr = tid % PR;
+      const int64_t e0 = (int64_t)(m0 + p * PR + lr) * ldc + n0;
+      const int lead = lead_of(e0);
+      // lanes 0 .. PR - 1: the columns before the first boundary; PR .. 2 PR - 1: those after the last whole piece
+      const int from = tid < PR ? 0 : (ncols > lead ? lead + ((ncols - lead) & ~(E - 1)) : ncols);
+      const int to = tid < PR ? (lead < ncols ? lead : ncols) : ncols;
+      OutT ends[E - 1];
+#pragma unroll
+      for (int k = 0; k < E - 1; ++k) ends[k] = c_s[lr * PITCH + (from + k < BN ? from + k : BN - 1)];
+#pragma unroll
+      for (int k = 0; k < E - 1; ++k)
+        if (from + k < to) C[e0 + from + k] = ends[k];
     }
     __syncthreads();
   }
@@ -1066,8 +1090,19 @@ void gemm_kernel_k64(const T* __restrict__ A, const void* __restrict__ Bv, typen
             const int lead = lead_of(e0);
             const int head = lead < ncols ? lead : ncols;
             const int tail = ncols > lead ? lead + ((ncols - lead) & ~(kChunk - 1)) : ncols;
-            for (int c = 0; c < head; ++c) C[e0 + c] = staged(row, c);
-            for (int c = tail; c < ncols; ++c) C[e0 + c] = staged(row, c);
+            // every read ahead of the first store, the stores under masks (one read and one store per turn of a loop
+            // would put their latencies end to end)
+            OutT hv[kChunk - 1], tv[kChunk - 1];
+#pragma unroll
+            for (int k = 0; k < kChunk - 1; ++k) {
+              hv[k] = staged(row, k);
+              tv[k] = staged(row, tail + k < W ? tail + k : W - 1);
+            }
+#pragma unroll
+            for (int k = 0; k < kChunk - 1; ++k) {
+              if (k < head) C[e0 + k] = hv[k];
+              if (tail + k < ncols) C[e0 + tail + k] = tv[k];
+            }
           }
         }
         return;
