@@ -66,7 +66,11 @@ int hexmi_num_cus(void);
  * NUM_COLS, BLOCK_SIZE)` of test/python/triton/test_softmax.py:44-72 and
  * nn.Softmax(dim=1) of test/python/torch-mlir/test_softmax_torch.py:24-31.
  * ld_x / ld_y: elements between consecutive rows (>= cols).
- * dtype: HEXMI_F32, HEXMI_F16 or HEXMI_BF16 (input and output alike). */
+ * dtype: HEXMI_F32, HEXMI_F16 or HEXMI_BF16 (input and output alike).
+ * Rows off the 16-byte boundaries (an odd cols, a view) run within a tenth
+ * of the aligned rate when the rows of x and y are equally far off them
+ * (x - y and (ld_x - ld_y) * element size multiples of 16 bytes: contiguous
+ * tensors, equal column slices), at about two thirds of it otherwise. */
 int hexmi_softmax(const void *x, void *y, int64_t rows, int64_t cols,
                   int64_t ld_x, int64_t ld_y, int dtype, hexmi_stream_t stream);
 
@@ -150,9 +154,10 @@ int hexmi_matmul_f16f16_f32(int64_t n_row, int64_t n_col, int64_t n_inner,
  * (the fp16 x fp16 -> fp32 form of docs/tutorials/triton/matmul_hexkl.md:61-97).
  * Any shape, leading dimension and alignment of the element type is taken.
  * Fastest: K % 64 == 0, operand rows on 16-byte boundaries (lda, ldb
- * multiples of 8, aligned bases), B as [K,N] with N % 8 == 0; K % 8 == 0 or an
- * odd N with B as [N,K] costs up to half the rate, unaligned operand rows about
- * two thirds.
+ * multiples of 8, aligned bases), B as [K,N] with N % 8 == 0; an odd N with B
+ * as [N,K] costs about a fifth of the rate, K % 8 == 0 up to half, unaligned
+ * operand rows about two thirds. Up to 64 rows against B as [N,K] are a
+ * stream of the weights (no tiles).
  * in_dtype == out_dtype == HEXMI_F32: fp32 operands multiplied in fp32 (no
  * rounding of the operands): the fp32 matmuls of the reference's torch-mlir
  * graphs (test/python/torch-mlir/test_add_matmul_softmax.py:25-29). K % 32 == 0
